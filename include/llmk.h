@@ -1,0 +1,170 @@
+/* llmk.h -- C ABI of libllmk_gfx950.so: MI355X (gfx950) kernels for the quantized-GEMM
+ * path of Jzz24/LLM_Kernels.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated; the library never allocates,
+ *     frees or synchronises; work is enqueued on `stream` (a hipStream_t, NULL = default).
+ *   - return value: 0 on success, negative LLMK_ERR_* otherwise; llmk_last_error()
+ *     gives a thread-local message.
+ *   - matrices are row-major and contiguous.  dtype codes: LLMK_F32/F16/BF16.
+ *   - "ref:" comments cite the file:line of the reference interface each entry replaces.
+ */
+#ifndef LLMK_H
+#define LLMK_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLMK_OK          0
+#define LLMK_ERR_SHAPE  (-1)   /* shape / alignment precondition violated                */
+#define LLMK_ERR_DTYPE  (-2)   /* unsupported dtype / mode code                          */
+#define LLMK_ERR_LAUNCH (-3)   /* hipGetLastError() reported a launch failure            */
+#define LLMK_ERR_ARG    (-4)   /* null pointer or inconsistent argument                  */
+
+#define LLMK_F32  0
+#define LLMK_F16  1
+#define LLMK_BF16 2
+
+/* rounding rules of the three reference quantizers */
+#define LLMK_ROUND_HALF_AWAY 0 /* libdevice.round   ref: quantization/int8_kernel.py:27,84          */
+#define LLMK_ROUND_HALF_UP   1 /* floor(v + 0.5)    ref: quantization/w4a8_kernel.py:164,222        */
+
+/* element kinds of the grouped GEMM */
+#define LLMK_KIND_I8   0       /* int8 x int8, 128x128 / 1x128 block scales (fp16 or fp32 scales)    */
+#define LLMK_KIND_FP8  1       /* e4m3 x e4m3, block scales fp32                                      */
+#define LLMK_KIND_F16  2       /* fp16 x fp16, no scales                                              */
+#define LLMK_KIND_BF16 3       /* bf16 x bf16, no scales                                              */
+
+int         llmk_version(void);
+const char* llmk_last_error(void);
+/* Number of bytes of split-K scratch llmk_gemm_* may use for (M,N); 0 means none needed. */
+int64_t     llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* ------------------------------------------------------------------ bit packing
+ * ref: quantization/bitpack.py:228-293 (pack rows), :84-149 (pack cols),
+ *      :308-373 (unpack rows), :163-226 (unpack cols); aliases :376-379.
+ * in_bytes: element size of the unpacked matrix (1, 2, 4 or 8; little endian integers).
+ * pack_bits in {8,16,32,64}, nbits in {1,2,4,8}; e = pack_bits / nbits.
+ * pack rows:  out[r, c] = OR_i (in[r*e+i, c] << i*nbits), in [rows_out*e, cols]
+ * pack cols:  out[r, c] = OR_i (in[r, c*e+i] << i*nbits), in [rows, cols_out*e]
+ * unpack:     (packed >> i*nbits) & mask, written as out_bytes-wide integers.      */
+int llmk_pack_rows(const void* in, int in_bytes, void* out, int64_t rows_out, int64_t cols,
+                   int nbits, int pack_bits, void* stream);
+int llmk_pack_cols(const void* in, int in_bytes, void* out, int64_t rows, int64_t cols_out,
+                   int nbits, int pack_bits, void* stream);
+int llmk_unpack_rows(const void* packed, int pack_bits, void* out, int out_bytes,
+                     int64_t rows_packed, int64_t cols, int nbits, int e, void* stream);
+int llmk_unpack_cols(const void* packed, int pack_bits, void* out, int out_bytes,
+                     int64_t rows, int64_t cols_packed, int nbits, int e, void* stream);
+
+/* ------------------------------------------------------------------ quantizers
+ * 1 x block activation groups (block = 128 in every reference call).
+ * ref: quantization/fp8_kernel.py:9-52   -> llmk_act_quant_fp8  (s fp32 [n_groups])
+ *      quantization/int8_kernel.py:9-56  -> llmk_act_quant_i8, LLMK_ROUND_HALF_AWAY (s fp16)
+ *      quantization/w4a8_kernel.py:145-193 -> llmk_act_quant_i8, LLMK_ROUND_HALF_UP          */
+int llmk_act_quant_fp8(const void* x, int x_dtype, void* y_e4m3, float* s, int64_t n_groups,
+                       int block, void* stream);
+int llmk_act_quant_i8(const void* x, int x_dtype, int8_t* y, void* s_f16, int64_t n_groups,
+                      int block, int round_mode, void* stream);
+
+/* block x block weight quantizers over W [M, N].
+ * ref: quantization/int8_kernel.py:59-113 (qmax 127, half-away, no clamp)
+ *      quantization/w4a8_kernel.py:196-225 (qmax 119, half-up, clamp +-119)
+ * fp8: s = blockmax/448 fp32; the reference has no fp8 weight quantizer (analogue of the above). */
+int llmk_weight_quant_i8_block(const void* x, int x_dtype, int8_t* y, void* s_f16, int64_t M,
+                               int64_t N, int block, float qmax, int round_mode, int clamp,
+                               void* stream);
+int llmk_weight_quant_fp8_block(const void* x, int x_dtype, void* y_e4m3, float* s, int64_t M,
+                                int64_t N, int block, void* stream);
+/* second level of the w4a8 weight quantizer, in place on the int8 matrix y [M,N]:
+ * per (row, group): s4 = floor((max-min)/15+.5), z4 = floor(-min/s4+.5),
+ * y <- clamp(floor(y/s4+.5)+z4, 0, 15).   ref: quantization/w4a8_kernel.py:228-262 */
+int llmk_weight_quant_w4a8_level2(int8_t* y, int8_t* s4, int8_t* z4, int64_t M, int64_t N,
+                                  int group, void* stream);
+
+/* dequantizers: y = fp32(x) * s[block]  ref: fp8_kernel.py:55-105, int8_kernel.py:116-166 */
+int llmk_weight_dequant_fp8_block(const void* x_e4m3, const float* s, void* y, int y_dtype,
+                                  int64_t M, int64_t N, int block, void* stream);
+int llmk_weight_dequant_i8_block(const int8_t* x, const void* s, int s_dtype, void* y, int y_dtype,
+                                 int64_t M, int64_t N, int block, void* stream);
+/* packed [N/8, K] int32 (8 rows per word) -> fp16 [N, K]: ((q - z4) * s4 in int8) * s
+ * ref: quantization/w4a8_kernel.py:16-142 */
+int llmk_weight_dequant_w4a8(const int32_t* packed, const void* s_f16, const int8_t* s4,
+                             const int8_t* z4, void* y_f16, int64_t N, int64_t K, int block,
+                             int group, void* stream);
+
+/* ------------------------------------------------------------------ dense quantized GEMMs
+ * C[M,N] = sum_kb dot_kb(A, B) * a_s[m, kb] * b_s[n / 128, kb], K % 128 == 0, any M, N >= 1.
+ * A [M,K], B [N,K] both K-contiguous.  c_dtype selects the epilogue (torch default dtype).
+ * workspace/workspace_bytes: optional split-K scratch (may be NULL/0 -> no split-K).
+ * ref: quantization/fp8_kernel.py:113-191 (a_s, b_s fp32)                                   */
+int llmk_gemm_fp8_block(const void* a_e4m3, const float* a_s, const void* b_e4m3, const float* b_s,
+                        void* c, int c_dtype, int64_t M, int64_t N, int64_t K,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+/* ref: quantization/int8_kernel.py:174-257 (scales fp16 in the reference; s_dtype F16/BF16/F32) */
+int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const void* b_s,
+                       int s_dtype, void* c, int c_dtype, int64_t M, int64_t N, int64_t K,
+                       void* workspace, int64_t workspace_bytes, void* stream);
+/* per-token x per-channel W8A8 with one full-K int32 accumulation (the BASELINE config-2 scheme;
+ * no counterpart function in the reference).  c may be NULL; c_i32 (raw accumulators) may be NULL. */
+int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, const float* b_s,
+                        void* c, int c_dtype, int32_t* c_i32, int64_t M, int64_t N, int64_t K,
+                        void* stream);
+/* b packed [N/8, K] int32, nibble (n % 8) of word [n/8, k]; b8 = int8((q - z4[n,kg]) * s4[n,kg]).
+ * ref: quantization/w4a8_kernel.py:317-448 */
+int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, const void* b_s,
+                   int s_dtype, const int8_t* b_s4, const int8_t* b_z4, void* c, int c_dtype,
+                   int64_t M, int64_t N, int64_t K, int group_int4,
+                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ W4A16
+ * C[M,N] (fp16) = A[M,K] (fp16) x ((nibble - 8) * s[k / groupsize, n]); B and s in the
+ * simple-Marlin packed layout produced by QuantUtils.pack (B int32 [K/16, 2N], s fp16 [K/g, N]
+ * permuted per 64 columns).  M, N, K % 16 == 0 (rc -1 otherwise, as the reference launcher),
+ * additionally N % 64 == 0 and groupsize % 16 == 0.
+ * ref: fast_dequant/simple_marlin/marlin_w4a16_gemm.cu:283-326 (simple_marlin_cuda),
+ *      marlin_w4a16_gemm.cpp:23-111 (mul).                                                    */
+int llmk_gemm_w4a16_marlin(const void* a_f16, const int32_t* b, void* c_f16, const void* s_f16,
+                           int64_t M, int64_t N, int64_t K, int groupsize,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+/* Same product for W stored [N, K/8] int32 by pack_weights_over_cols (nibble i of a word = k*8+i)
+ * with s fp16 [N, K/g]; a/c fp16 or bf16 (dtype code).  BASELINE config-1 layout. */
+int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s_f16,
+                       int ac_dtype, int64_t M, int64_t N, int64_t K, int groupsize,
+                       void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ MoE (one GPU's experts)
+ * ref: moe/group_gemm_kernel.py:19-45 (segment pointers, src2dst), :81-117 (pre_reorder),
+ *      :120-235 (silu/gelu and mul), :238-288 (post_reorder), :291-513 (grouped GEMM).       */
+int llmk_moe_seg_indptr(const int64_t* sorted_ids, int64_t* seg_indptr, int64_t num_toks,
+                        int num_experts, void* stream);
+int llmk_moe_src2dst(const int64_t* reorder_ids, int32_t* src2dst, int64_t num_toks, void* stream);
+/* ids_bytes: 4 or 8 (topk_ids int32 / int64).  a1_scales may be NULL (fp32 per expert). */
+int llmk_moe_pre_reorder(const void* x, int x_dtype, void* out, int out_dtype, const int32_t* src2dst,
+                         const void* topk_ids, int ids_bytes, const float* a1_scales,
+                         int start_expert, int end_expert, int topk, int64_t T, int64_t hidden,
+                         void* stream);
+/* act: 0 silu, 1 tanh-gelu.  gateup [M, 2I] -> out [M, I]; scales may be NULL. */
+int llmk_moe_act_and_mul(const void* gateup, int in_dtype, void* out, int out_dtype,
+                         const void* reorder_topk_ids, int ids_bytes, const float* scales,
+                         int start_expert, int end_expert, int64_t M, int64_t two_i, int act,
+                         void* stream);
+/* w_dtype: dtype code of topk_weights. */
+int llmk_moe_post_reorder(const void* down_out, void* out, int dtype, const int32_t* src2dst,
+                          const void* topk_ids, int ids_bytes, const void* topk_weights, int w_dtype,
+                          int start_expert, int end_expert, int topk, int64_t T, int64_t hidden,
+                          void* stream);
+/* C[seg[e]:seg[e+1], :] = A[seg[e]:seg[e+1], :] x B[weight_indices[e]]^T  for e < E.
+ * a [M,K], b [E,N,K], c [M,N]; scale_a [M,K/128], scale_b [E,ceil(N/128),K/128] for the
+ * block-scaled kinds (s_dtype = dtype code of both), NULL otherwise. */
+int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind, int c_dtype, int E,
+                      int64_t M, int64_t N, int64_t K, const int64_t* seg_indptr,
+                      const int64_t* weight_indices, const void* scale_a, const void* scale_b,
+                      int s_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMK_H */

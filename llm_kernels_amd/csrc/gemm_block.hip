@@ -1,0 +1,65 @@
+// Dense block-scaled fp8 / int8 GEMM entry points.
+#include "gemm_direct.hpp"
+
+using namespace llmk;
+
+namespace {
+
+int check_common(const char* name, const void* a, const void* b, int64_t M, int64_t N, int64_t K, int c_dtype) {
+    if (M < 0 || N < 0 || K < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: negative dimension", name);
+    if (K % 128 != 0) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: K=%lld must be a multiple of 128", name, (long long)K);
+    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: dimension exceeds int32", name);
+    if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "%s: c_dtype %d", name, c_dtype);
+    if (M && N && K && (!a || !b)) LLMK_FAIL(LLMK_ERR_ARG, "%s: null operand", name);
+    if ((((uintptr_t)a) | ((uintptr_t)b)) & 15) LLMK_FAIL(LLMK_ERR_ARG, "%s: operands must be 16-byte aligned", name);
+    return LLMK_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    (void)M; (void)N; (void)K;
+    return 0;
+}
+
+extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                                   int c_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                   int64_t workspace_bytes, void* stream) {
+    (void)workspace; (void)workspace_bytes;
+    int rc = check_common("gemm_fp8_block", a, b, M, N, K, c_dtype);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!c || (K && (!a_s || !b_s))) LLMK_FAIL(LLMK_ERR_ARG, "gemm_fp8_block: null pointer");
+    DirectArgs p{};
+    p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
+    p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+    return launch_direct<K_FP8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_fp8_block");
+}
+
+extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const void* b_s, int s_dtype,
+                                  void* c, int c_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+    (void)workspace; (void)workspace_bytes;
+    int rc = check_common("gemm_i8_block", a, b, M, N, K, c_dtype);
+    if (rc) return rc;
+    if (s_dtype != LLMK_F32 && s_dtype != LLMK_F16 && s_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_i8_block: s_dtype %d", s_dtype);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!c || (K && (!a_s || !b_s))) LLMK_FAIL(LLMK_ERR_ARG, "gemm_i8_block: null pointer");
+    DirectArgs p{};
+    p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
+    p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+    return launch_direct<K_I8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_block");
+}
+
+extern "C" int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, const float* b_s, void* c,
+                                   int c_dtype, int32_t* c_i32, int64_t M, int64_t N, int64_t K, void* stream) {
+    int rc = check_common("gemm_i8_rowcol", a, b, M, N, K, c_dtype);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!c && !c_i32) LLMK_FAIL(LLMK_ERR_ARG, "gemm_i8_rowcol: no output buffer");
+    if (c && (!a_s || !b_s)) LLMK_FAIL(LLMK_ERR_ARG, "gemm_i8_rowcol: scales required for the scaled output");
+    DirectArgs p{};
+    p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.c_i32 = c_i32; p.a_s = a_s; p.b_s = b_s;
+    p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+    return launch_direct<K_I8_ROWCOL, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_rowcol");
+}

@@ -1,0 +1,297 @@
+// W4A16 GEMM kernels: fp16 activations x 4-bit weights dequantised in registers.
+//
+// nibble -> fp16 without integer->float converts: (q | 0x6400) is the fp16 number 1024 + q,
+// ((q << 4) | 0x6400) is 1024 + 16 q; one packed subtract / fma gives q - 8 exactly.
+#include "common.hpp"
+
+namespace {
+
+__device__ __forceinline__ v2h as_h2(unsigned u) { v2h r; __builtin_memcpy(&r, &u, 4); return r; }
+__device__ __forceinline__ unsigned as_u32(v2h h) { unsigned r; __builtin_memcpy(&r, &h, 4); return r; }
+
+// nibbles at bits [3:0] and [19:16] of w -> (q_lo - 8, q_hi - 8)
+__device__ __forceinline__ v2h deq_lo(unsigned w) {
+    const v2h k1032 = {(_Float16)1032.f, (_Float16)1032.f};
+    return as_h2((w & 0x000f000fu) | 0x64006400u) - k1032;
+}
+// nibbles at bits [7:4] and [23:20]
+__device__ __forceinline__ v2h deq_hi(unsigned w) {
+    const v2h k16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const v2h k72 = {(_Float16)72.f, (_Float16)72.f};
+    return as_h2((w & 0x00f000f0u) | 0x64006400u) * k16 - k72;
+}
+
+__device__ __forceinline__ v8h make8(v2h a, v2h b, v2h c, v2h d) {
+    v8h r;
+    r[0] = a[0]; r[1] = a[1]; r[2] = b[0]; r[3] = b[1];
+    r[4] = c[0]; r[5] = c[1]; r[6] = d[0]; r[7] = d[1];
+    return r;
+}
+
+// Tree reduction of per-wave accumulators through LDS; the total ends in wave 0.
+template <int NW, int NACC>
+__device__ __forceinline__ void reduce_waves(float (&acc)[NACC], float* buf, int wave, int lane) {
+#pragma unroll
+    for (int half = NW / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) {
+            float* dst = buf + (size_t)(wave - half) * NACC * 64;
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) dst[i * 64 + lane] = acc[i];
+        }
+        __syncthreads();
+        if (wave < half) {
+            const float* src = buf + (size_t)wave * NACC * 64;
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) acc[i] += src[i * 64 + lane];
+        }
+        __syncthreads();
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// simple-Marlin layout.  B viewed as 16-byte units: unit ((strip * N/64) + chunk) * 32 + 4c + q
+// holds, for mma lane (c = column within 8, q = k pair), word j = 16-column sub-tile j:
+//   bits  3:0 (k0, c)   7:4 (k0+8, c)   11:8 (k0, c+8)   15:12 (k0+8, c+8)      k0 = 2q
+//   bits 19:16 (k0+1,c) 23:20 (k0+9,c)  27:24 (k0+1,c+8) 31:28 (k0+9,c+8)
+// Scales are stored per 64-column chunk as [c][2j + b] (column 16j + 8b + c).
+//
+// gfx950 mapping: a wave owns two chunks (128 columns).  Lane l: r = l & 15 -> c = r & 7,
+// chunk half h = r >> 3; g = l >> 4 plays the role of the mma k-pair q.  One MFMA 16x16x32
+// step consumes two 16-K strips; MFMA (j, b) produces columns {64(2cp+h) + 16j + 8b + c}.
+// A fragment order per lane: k in {2g, 2g+1, 2g+8, 2g+9} of strip 0, then of strip 1.
+template <int MT, int NW, bool TO_WS>
+__global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
+    const _Float16* __restrict__ A, const v4i* __restrict__ B, const _Float16* __restrict__ S,
+    _Float16* __restrict__ C, float* __restrict__ ws, int M, int N, int K, int groupsize, int steps_per_z) {
+    extern __shared__ float red[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4, c = r & 7, h = r >> 3;
+    const int nchunks = N >> 6;
+    const int strips = K >> 4;
+    const int total_steps = (strips + 1) >> 1;
+    const int chunk_raw = 2 * blockIdx.x + h;
+    const bool chunk_ok = chunk_raw < nchunks;
+    const int chunk = chunk_ok ? chunk_raw : nchunks - 1;
+    const int m0 = blockIdx.y * 16 * MT;
+    const int ks_begin = blockIdx.z * steps_per_z;
+    const int ks_end = min(total_steps, ks_begin + steps_per_z);
+
+    const _Float16* arow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (int64_t)min(m0 + 16 * mt + r, M - 1) * K + 2 * g;
+
+    float acc[MT * 32];
+#pragma unroll
+    for (int i = 0; i < MT * 32; ++i) acc[i] = 0.f;
+
+    int cur_grp0 = -1, cur_grp1 = -1;
+    v8h s0 = {}, s1 = {};
+    for (int ks = ks_begin + wave; ks < ks_end; ks += NW) {
+        const int st0 = 2 * ks, st1 = 2 * ks + 1;
+        const bool have1 = st1 < strips;
+        const int st1c = have1 ? st1 : st0;
+        const v4i w0 = B[((int64_t)st0 * nchunks + chunk) * 32 + 4 * c + g];
+        const v4i w1 = B[((int64_t)st1c * nchunks + chunk) * 32 + 4 * c + g];
+        const int grp0 = (16 * st0) / groupsize, grp1 = (16 * st1c) / groupsize;
+        if (grp0 != cur_grp0) { s0 = *(const v8h*)(S + (int64_t)grp0 * N + 64 * chunk + 8 * c); cur_grp0 = grp0; }
+        if (grp1 != cur_grp1) { s1 = *(const v8h*)(S + (int64_t)grp1 * N + 64 * chunk + 8 * c); cur_grp1 = grp1; }
+
+        v8h a[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const unsigned* ap = (const unsigned*)(arow[mt] + 32 * ks);
+            unsigned x0 = ap[0], x1 = ap[4], x2 = have1 ? ap[8] : 0u, x3 = have1 ? ap[12] : 0u;
+            a[mt] = make8(as_h2(x0), as_h2(x1), as_h2(x2), as_h2(x3));
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int t = 2 * j + b;
+                const unsigned u0 = ((unsigned)w0[j]) >> (8 * b), u1 = ((unsigned)w1[j]) >> (8 * b);
+                const v2h sc0 = {s0[t], s0[t]}, sc1 = {s1[t], s1[t]};
+                const v8h bf = make8(deq_lo(u0) * sc0, deq_hi(u0) * sc0, deq_lo(u1) * sc1, deq_hi(u1) * sc1);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    v4f d = {acc[(mt * 8 + t) * 4 + 0], acc[(mt * 8 + t) * 4 + 1], acc[(mt * 8 + t) * 4 + 2], acc[(mt * 8 + t) * 4 + 3]};
+                    d = mfma_f16_16x16x32(a[mt], bf, d);
+                    acc[(mt * 8 + t) * 4 + 0] = d[0]; acc[(mt * 8 + t) * 4 + 1] = d[1];
+                    acc[(mt * 8 + t) * 4 + 2] = d[2]; acc[(mt * 8 + t) * 4 + 3] = d[3];
+                }
+            }
+        }
+    }
+
+    reduce_waves<NW, MT * 32>(acc, red, wave, lane);
+    if (wave != 0 || !chunk_ok) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = m0 + 16 * mt + 4 * g + i;
+                const int n = 64 * chunk + 16 * (t >> 1) + 8 * (t & 1) + c;
+                if (m < M) {
+                    const float v = acc[(mt * 8 + t) * 4 + i];
+                    if constexpr (TO_WS) ws[((int64_t)blockIdx.z * M + m) * N + n] = v;
+                    else C[(int64_t)m * N + n] = (_Float16)v;
+                }
+            }
+}
+
+__global__ void splitk_reduce_f16_kernel(const float* __restrict__ ws, _Float16* __restrict__ C, int64_t MN, int Z) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= MN) return;
+    float s = 0.f;
+    for (int z = 0; z < Z; ++z) s += ws[(int64_t)z * MN + i];
+    C[i] = (_Float16)s;
+}
+
+// ------------------------------------------------------------------------------------------
+// [N, K/8] layout (pack_weights_over_cols: nibble i of word w of row n is k = 8w + i) with
+// scales [N, K/g].  Lane (r = column, g) loads one 16-byte unit = 32 consecutive k of its row per
+// 128-K step; word j feeds MFMA j, whose fragment order is k offsets [0,4,1,5,2,6,3,7] -- the A
+// fragment is permuted to the same order with v_perm_b32.
+template <int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void w4a16_nk_kernel(
+    const _Float16* __restrict__ A, const int32_t* __restrict__ B, const _Float16* __restrict__ S,
+    _Float16* __restrict__ C, int M, int N, int K, int groupsize) {
+    extern __shared__ float red[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16 * MT;
+    const int nrow = min(n0 + r, N - 1);
+    const int steps = K >> 7;
+    const int ngroups = K / groupsize;
+    const int32_t* brow = B + (int64_t)nrow * (K >> 3) + 4 * g;
+    const _Float16* srow = S + (int64_t)nrow * ngroups;
+    const _Float16* arow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (int64_t)min(m0 + 16 * mt + r, M - 1) * K + 32 * g;
+
+    float acc[MT * 4];
+#pragma unroll
+    for (int i = 0; i < MT * 4; ++i) acc[i] = 0.f;
+
+#pragma unroll 2
+    for (int ks = wave; ks < steps; ks += NW) {
+        const v4i w = *(const v4i*)(brow + ks * 16);
+        const int kbase = ks * 128 + 32 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const _Float16 sv = srow[(kbase + 8 * j) / groupsize];
+            const v2h sc = {sv, sv};
+            const unsigned u = (unsigned)w[j], u8 = u >> 8;
+            const v8h bf = make8(deq_lo(u) * sc, deq_hi(u) * sc, deq_lo(u8) * sc, deq_hi(u8) * sc);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const v4i x = *(const v4i*)(arow[mt] + ks * 128 + 8 * j);
+                v4i y;
+                y[0] = (int)__builtin_amdgcn_perm((unsigned)x[2], (unsigned)x[0], 0x05040100u);  // k0,k4
+                y[1] = (int)__builtin_amdgcn_perm((unsigned)x[2], (unsigned)x[0], 0x07060302u);  // k1,k5
+                y[2] = (int)__builtin_amdgcn_perm((unsigned)x[3], (unsigned)x[1], 0x05040100u);  // k2,k6
+                y[3] = (int)__builtin_amdgcn_perm((unsigned)x[3], (unsigned)x[1], 0x07060302u);  // k3,k7
+                v8h a;
+                __builtin_memcpy(&a, &y, 16);
+                v4f d = {acc[mt * 4 + 0], acc[mt * 4 + 1], acc[mt * 4 + 2], acc[mt * 4 + 3]};
+                d = mfma_f16_16x16x32(a, bf, d);
+                acc[mt * 4 + 0] = d[0]; acc[mt * 4 + 1] = d[1]; acc[mt * 4 + 2] = d[2]; acc[mt * 4 + 3] = d[3];
+            }
+        }
+    }
+    reduce_waves<NW, MT * 4>(acc, red, wave, lane);
+    if (wave != 0) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m0 + 16 * mt + 4 * g + i, n = n0 + r;
+            if (m < M && n < N) C[(int64_t)m * N + n] = (_Float16)acc[mt * 4 + i];
+        }
+}
+
+}  // namespace
+
+extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, const void* s, int64_t M, int64_t N,
+                                      int64_t K, int groupsize, void* workspace, int64_t workspace_bytes,
+                                      void* stream) {
+    // the reference launcher returns -1 for any dimension not divisible by 16 (marlin_w4a16_gemm.cu:300-302)
+    if (M % 16 || N % 16 || K % 16 || M < 0 || N < 0 || K < 0)
+        LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: M, N, K must be multiples of 16 (M=%lld N=%lld K=%lld)", (long long)M, (long long)N, (long long)K);
+    if (N % 64) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: N=%lld must be a multiple of 64 (packed chunk width)", (long long)N);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (K == 0) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: K == 0");
+    if (groupsize == -1) groupsize = (int)K;
+    if (groupsize < 16 || groupsize % 16 || K % groupsize)
+        LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: groupsize=%d must be a multiple of 16 dividing K=%lld", groupsize, (long long)K);
+    if (!a || !b || !c || !s) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a16_marlin: null pointer");
+    if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)s) & 15) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a16_marlin: operands must be 16-byte aligned");
+    if (M > 0x7fffffff / 2 || N > 0x7fffffff / 2 || K > 0x7fffffff / 2) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: dimension too large");
+
+    const int total_steps = (int)((K / 16 + 1) / 2);
+    const int col_groups = (int)((N / 64 + 1) / 2);
+    hipStream_t st = (hipStream_t)stream;
+    const _Float16* A = (const _Float16*)a;
+    const v4i* B = (const v4i*)b;
+    const _Float16* S = (const _Float16*)s;
+    _Float16* C = (_Float16*)c;
+
+    if (M <= 16) {
+        constexpr int NW = 8;
+        // split K over workgroups until the grid covers the chip; each workgroup keeps >= NW steps
+        int z = 1;
+        while (col_groups * z < 256 && total_steps / (z * 2) >= NW) z *= 2;
+        const int64_t need = (int64_t)z * M * N * 4;
+        if (z > 1 && (!workspace || workspace_bytes < need)) z = 1;
+        const int spz = (total_steps + z - 1) / z;
+        dim3 grid(col_groups, 1, z), blk(NW * 64);
+        const size_t smem = (size_t)(NW / 2) * 32 * 64 * sizeof(float);
+        if (z == 1) {
+            w4a16_marlin_kernel<1, NW, false><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, spz);
+            LLMK_CHECK_LAUNCH("gemm_w4a16_marlin");
+        } else {
+            w4a16_marlin_kernel<1, NW, true><<<grid, blk, smem, st>>>(A, B, S, C, (float*)workspace, (int)M, (int)N, (int)K, groupsize, spz);
+            LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(split)");
+            splitk_reduce_f16_kernel<<<(unsigned)cdiv64(M * N, 256), 256, 0, st>>>((const float*)workspace, C, M * N, z);
+            LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(reduce)");
+        }
+    } else {
+        constexpr int MT = 4, NW = 2;
+        dim3 grid(col_groups, (unsigned)cdiv64(M, 16 * MT), 1), blk(NW * 64);
+        const size_t smem = (size_t)(NW / 2) * MT * 32 * 64 * sizeof(float);
+        w4a16_marlin_kernel<MT, NW, false><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, total_steps);
+        LLMK_CHECK_LAUNCH("gemm_w4a16_marlin");
+    }
+    return LLMK_OK;
+}
+
+extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s, int ac_dtype,
+                                  int64_t M, int64_t N, int64_t K, int groupsize, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+    (void)workspace; (void)workspace_bytes;
+    if (ac_dtype != LLMK_F16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a16_nk: only fp16 activations/outputs are supported (dtype code %d)", ac_dtype);
+    if (M < 0 || N < 0 || K < 0 || K % 128) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_nk: K=%lld must be a multiple of 128", (long long)K);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (K == 0) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_nk: K == 0");
+    if (groupsize == -1) groupsize = (int)K;
+    if (groupsize < 8 || groupsize % 8 || K % groupsize)
+        LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_nk: groupsize=%d must be a multiple of 8 dividing K", groupsize);
+    if (!a || !b_packed || !c || !s) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a16_nk: null pointer");
+    if (((uintptr_t)a | (uintptr_t)b_packed) & 15) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a16_nk: operands must be 16-byte aligned");
+    if (M > 0x7fffffff / 2 || N > 0x7fffffff / 2 || K > 0x7fffffff / 2) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_nk: dimension too large");
+    hipStream_t st = (hipStream_t)stream;
+    const _Float16* A = (const _Float16*)a;
+    const _Float16* S = (const _Float16*)s;
+    _Float16* C = (_Float16*)c;
+    const unsigned gx = (unsigned)cdiv64(N, 16);
+    if (M <= 16) {
+        constexpr int NW = 8;
+        w4a16_nk_kernel<1, NW><<<dim3(gx, 1), NW * 64, (NW / 2) * 4 * 64 * sizeof(float), st>>>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize);
+    } else {
+        constexpr int MT = 4, NW = 4;
+        w4a16_nk_kernel<MT, NW><<<dim3(gx, (unsigned)cdiv64(M, 16 * MT)), NW * 64, (NW / 2) * MT * 4 * 64 * sizeof(float), st>>>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize);
+    }
+    LLMK_CHECK_LAUNCH("gemm_w4a16_nk");
+    return LLMK_OK;
+}

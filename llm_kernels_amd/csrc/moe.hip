@@ -1,0 +1,189 @@
+// Single-GPU expert-parallel MoE path: segment bookkeeping, token permute / un-permute,
+// gated activation, and the grouped GEMM over one GPU's experts.
+#include "gemm_direct.hpp"
+
+using namespace llmk;
+
+namespace {
+
+// seg_indptr[e + 1] = number of sorted ids <= e (binary search for the right boundary)
+__global__ void seg_indptr_kernel(const int64_t* __restrict__ sorted_ids, int64_t* __restrict__ seg_indptr,
+                                  int64_t num_toks, int num_experts) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= num_experts) return;
+    int64_t lo = 0, hi = num_toks;       // first index with id > e
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (sorted_ids[mid] > e) hi = mid; else lo = mid + 1;
+    }
+    seg_indptr[e + 1] = lo;
+    if (e == 0) seg_indptr[0] = 0;
+}
+
+__global__ void src2dst_kernel(const int64_t* __restrict__ reorder_ids, int32_t* __restrict__ src2dst, int64_t n) {
+    const int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (d < n) src2dst[reorder_ids[d]] = (int32_t)d;
+}
+
+__device__ __forceinline__ int64_t ld_id(const void* p, int64_t i, int bytes) {
+    return bytes == 8 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
+}
+
+// one workgroup per token: copy (x * 1/a1_scale[e]) into each destination row of its local experts
+template <int IDT, int ODT>
+__global__ void pre_reorder_kernel(const void* __restrict__ x, void* __restrict__ out, const int32_t* __restrict__ src2dst,
+                                   const void* __restrict__ topk_ids, int ids_bytes, const float* __restrict__ a1_scales,
+                                   int start_e, int end_e, int topk, int64_t hidden) {
+    const int64_t t = blockIdx.x;
+    for (int j = 0; j < topk; ++j) {
+        const int64_t e = ld_id(topk_ids, t * topk + j, ids_bytes);
+        if (e < start_e || e > end_e) continue;
+        const float scale = a1_scales ? 1.0f / a1_scales[e - start_e] : 1.0f;
+        const int64_t dst = src2dst[t * topk + j];
+        for (int64_t c = threadIdx.x; c < hidden; c += blockDim.x)
+            FloatIO<ODT>::st(out, dst * hidden + c, FloatIO<IDT>::ld(x, t * hidden + c) * scale);
+    }
+}
+
+// round-trip through the storage type: the reference multiplies in the tensor dtype
+template <int DT> __device__ __forceinline__ float rnd(float v) {
+    if constexpr (DT == LLMK_F16) return f16_to_f32(f32_to_f16(v));
+    else if constexpr (DT == LLMK_BF16) return bf16_to_f32(f32_to_bf16(v));
+    else return v;
+}
+
+template <int IDT, int ODT>
+__global__ void act_and_mul_kernel(const void* __restrict__ gateup, void* __restrict__ out,
+                                   const void* __restrict__ reorder_topk_ids, int ids_bytes,
+                                   const float* __restrict__ scales, int start_e, int end_e, int64_t two_i, int act) {
+    const int64_t row = blockIdx.x;
+    const int64_t e = ld_id(reorder_topk_ids, row, ids_bytes);
+    if (e < start_e || e > end_e) return;
+    const int64_t I = two_i / 2;
+    const bool has_scale = scales != nullptr;
+    const float scale = has_scale ? rnd<IDT>(1.0f / scales[e - start_e]) : 1.0f;
+    for (int64_t c = threadIdx.x; c < I; c += blockDim.x) {
+        float gv = FloatIO<IDT>::ld(gateup, row * two_i + c);
+        const float up = FloatIO<IDT>::ld(gateup, row * two_i + I + c);
+        if (act == 0) {
+            gv = gv * (1.0f / (1.0f + expf(-gv)));
+        } else {
+            const float kAlpha = 0.7978845608028654f;
+            const float u = kAlpha * (gv + 0.044715f * gv * gv * gv);
+            const float th = 2.0f * (1.0f / (1.0f + expf(-2.0f * u))) - 1.0f;
+            gv = 0.5f * gv * (1.0f + th);
+        }
+        gv = rnd<IDT>(gv);
+        float r = rnd<IDT>(gv * up);
+        if (has_scale) r = rnd<IDT>(r * scale);
+        FloatIO<ODT>::st(out, row * I + c, r);
+    }
+}
+
+template <int DT, int WDT>
+__global__ void post_reorder_kernel(const void* __restrict__ down, void* __restrict__ out, const int32_t* __restrict__ src2dst,
+                                    const void* __restrict__ topk_ids, int ids_bytes, const void* __restrict__ topk_w,
+                                    int start_e, int end_e, int topk, int64_t hidden) {
+    const int64_t t = blockIdx.x;
+    for (int64_t c = threadIdx.x; c < hidden; c += blockDim.x) {
+        float sum = 0.f;
+        for (int j = 0; j < topk; ++j) {
+            const int64_t e = ld_id(topk_ids, t * topk + j, ids_bytes);
+            if (e < start_e || e > end_e) continue;
+            const int64_t dst = src2dst[t * topk + j];
+            const float w = rnd<DT>(FloatIO<WDT>::ld(topk_w, t * topk + j));
+            const float v = FloatIO<DT>::ld(down, dst * hidden + c);
+            sum = rnd<DT>(sum + rnd<DT>(v * w));     // product and running sum both live in the tensor dtype
+        }
+        FloatIO<DT>::st(out, t * hidden + c, sum);
+    }
+}
+
+}  // namespace
+
+extern "C" int llmk_moe_seg_indptr(const int64_t* sorted_ids, int64_t* seg_indptr, int64_t num_toks, int num_experts,
+                                   void* stream) {
+    if (num_experts < 0 || num_toks < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_seg_indptr: negative size");
+    if (!seg_indptr || (num_toks && !sorted_ids)) LLMK_FAIL(LLMK_ERR_ARG, "moe_seg_indptr: null pointer");
+    if (num_experts == 0) return LLMK_OK;
+    seg_indptr_kernel<<<(unsigned)cdiv64(num_experts, 64), 64, 0, (hipStream_t)stream>>>(sorted_ids, seg_indptr, num_toks, num_experts);
+    LLMK_CHECK_LAUNCH("moe_seg_indptr");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_moe_src2dst(const int64_t* reorder_ids, int32_t* src2dst, int64_t num_toks, void* stream) {
+    if (num_toks < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_src2dst: negative size");
+    if (num_toks == 0) return LLMK_OK;
+    if (!reorder_ids || !src2dst) LLMK_FAIL(LLMK_ERR_ARG, "moe_src2dst: null pointer");
+    src2dst_kernel<<<(unsigned)cdiv64(num_toks, 256), 256, 0, (hipStream_t)stream>>>(reorder_ids, src2dst, num_toks);
+    LLMK_CHECK_LAUNCH("moe_src2dst");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_moe_pre_reorder(const void* x, int x_dtype, void* out, int out_dtype, const int32_t* src2dst,
+                                    const void* topk_ids, int ids_bytes, const float* a1_scales, int start_expert,
+                                    int end_expert, int topk, int64_t T, int64_t hidden, void* stream) {
+    if (T < 0 || hidden < 0 || topk < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_pre_reorder: negative size");
+    if (ids_bytes != 4 && ids_bytes != 8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_pre_reorder: ids_bytes %d", ids_bytes);
+    if (T == 0 || hidden == 0 || topk == 0) return LLMK_OK;
+    if (!x || !out || !src2dst || !topk_ids) LLMK_FAIL(LLMK_ERR_ARG, "moe_pre_reorder: null pointer");
+    LLMK_DISPATCH_FLOAT(x_dtype, IDT, LLMK_DISPATCH_FLOAT(out_dtype, ODT,
+        (pre_reorder_kernel<IDT, ODT><<<(unsigned)T, 256, 0, (hipStream_t)stream>>>(x, out, src2dst, topk_ids, ids_bytes, a1_scales, start_expert, end_expert, topk, hidden))));
+    LLMK_CHECK_LAUNCH("moe_pre_reorder");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_moe_act_and_mul(const void* gateup, int in_dtype, void* out, int out_dtype,
+                                    const void* reorder_topk_ids, int ids_bytes, const float* scales, int start_expert,
+                                    int end_expert, int64_t M, int64_t two_i, int act, void* stream) {
+    if (M < 0 || two_i < 0 || two_i % 2) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_act_and_mul: bad shape");
+    if (ids_bytes != 4 && ids_bytes != 8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul: ids_bytes %d", ids_bytes);
+    if (act != 0 && act != 1) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul: act %d", act);
+    if (M == 0 || two_i == 0) return LLMK_OK;
+    if (!gateup || !out || !reorder_topk_ids) LLMK_FAIL(LLMK_ERR_ARG, "moe_act_and_mul: null pointer");
+    LLMK_DISPATCH_FLOAT(in_dtype, IDT, LLMK_DISPATCH_FLOAT(out_dtype, ODT,
+        (act_and_mul_kernel<IDT, ODT><<<(unsigned)M, 256, 0, (hipStream_t)stream>>>(gateup, out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, two_i, act))));
+    LLMK_CHECK_LAUNCH("moe_act_and_mul");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_moe_post_reorder(const void* down_out, void* out, int dtype, const int32_t* src2dst,
+                                     const void* topk_ids, int ids_bytes, const void* topk_weights, int w_dtype,
+                                     int start_expert, int end_expert, int topk, int64_t T, int64_t hidden,
+                                     void* stream) {
+    if (T < 0 || hidden < 0 || topk < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_post_reorder: negative size");
+    if (ids_bytes != 4 && ids_bytes != 8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_post_reorder: ids_bytes %d", ids_bytes);
+    if (T == 0 || hidden == 0) return LLMK_OK;
+    if (!down_out || !out || !src2dst || !topk_ids || !topk_weights) LLMK_FAIL(LLMK_ERR_ARG, "moe_post_reorder: null pointer");
+    LLMK_DISPATCH_FLOAT(dtype, DT, LLMK_DISPATCH_FLOAT(w_dtype, WDT,
+        (post_reorder_kernel<DT, WDT><<<(unsigned)T, 256, 0, (hipStream_t)stream>>>(down_out, out, src2dst, topk_ids, ids_bytes, topk_weights, start_expert, end_expert, topk, hidden))));
+    LLMK_CHECK_LAUNCH("moe_post_reorder");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind, int c_dtype, int E, int64_t M,
+                                 int64_t N, int64_t K, const int64_t* seg_indptr, const int64_t* weight_indices,
+                                 const void* scale_a, const void* scale_b, int s_dtype, void* stream) {
+    if (M < 0 || N < 0 || K < 0 || E < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "grouped_gemm: negative dimension");
+    if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm: c_dtype %d", c_dtype);
+    const bool scaled = (kind == LLMK_KIND_I8 || kind == LLMK_KIND_FP8);
+    const int kstep = scaled ? 128 : 64;
+    if (K % kstep) LLMK_FAIL(LLMK_ERR_SHAPE, "grouped_gemm: K=%lld must be a multiple of %d for this element kind", (long long)K, kstep);
+    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) LLMK_FAIL(LLMK_ERR_SHAPE, "grouped_gemm: dimension exceeds int32");
+    if (M == 0 || N == 0 || E == 0) return LLMK_OK;
+    if (!a || !b || !c || !seg_indptr) LLMK_FAIL(LLMK_ERR_ARG, "grouped_gemm: null pointer");
+    if (scaled && (!scale_a || !scale_b)) LLMK_FAIL(LLMK_ERR_ARG, "grouped_gemm: block scales required for int8 / fp8 operands");
+    if ((((uintptr_t)a) | ((uintptr_t)b)) & 15) LLMK_FAIL(LLMK_ERR_ARG, "grouped_gemm: operands must be 16-byte aligned");
+    DirectArgs p{};
+    p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = scale_a; p.b_s = scale_b;
+    p.seg_indptr = seg_indptr; p.weight_indices = weight_indices;
+    p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = E;
+    hipStream_t st = (hipStream_t)stream;
+    switch (kind) {
+        case LLMK_KIND_I8:   return launch_direct<K_I8_BLOCK, true>(p, (int)M, st, "grouped_gemm(i8)");
+        case LLMK_KIND_FP8:  return launch_direct<K_FP8_BLOCK, true>(p, (int)M, st, "grouped_gemm(fp8)");
+        case LLMK_KIND_F16:  return launch_direct<K_F16, true>(p, (int)M, st, "grouped_gemm(f16)");
+        case LLMK_KIND_BF16: return launch_direct<K_BF16, true>(p, (int)M, st, "grouped_gemm(bf16)");
+        default: LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm: kind %d", kind);
+    }
+}

@@ -1,0 +1,337 @@
+// Activation / weight quantizers and dequantizers (streaming kernels, HBM bound).
+//
+// Arithmetic follows the reference kernels exactly: fp32 math, IEEE division by the
+// un-rounded fp32 scale, then the scale is stored in its (possibly narrower) type.
+#include "common.hpp"
+
+namespace {
+
+constexpr int EPL = 8;   // elements per lane in the 1 x block kernels
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* p, int64_t i, float (&v)[EPL]) {
+    if constexpr (DT == LLMK_F32) {
+        const float4* q = (const float4*)((const float*)p + i);
+        float4 a = q[0], b = q[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        uint4 u = *(const uint4*)((const unsigned short*)p + i);
+        unsigned w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            unsigned short lo = (unsigned short)(w[j] & 0xffff), hi = (unsigned short)(w[j] >> 16);
+            v[2 * j]     = (DT == LLMK_F16) ? f16_to_f32(lo) : bf16_to_f32(lo);
+            v[2 * j + 1] = (DT == LLMK_F16) ? f16_to_f32(hi) : bf16_to_f32(hi);
+        }
+    }
+}
+
+__device__ __forceinline__ float round_mode(float v, int mode) {
+    // half-away: roundf is exact; half-up: floor(v + 0.5f) with the fp32 add as the reference states it
+    return mode == LLMK_ROUND_HALF_AWAY ? roundf(v) : floorf(v + 0.5f);
+}
+
+__device__ __forceinline__ unsigned pack_fp8x4(float a, float b, float c, float d) {
+    // saturate finite values to +-448 (comparisons leave NaN untouched), then RNE hardware convert
+    auto sat = [](float x) { return x > 448.f ? 448.f : (x < -448.f ? -448.f : x); };
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(a), sat(b), 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(c), sat(d), w, true);
+    return (unsigned)w;
+}
+
+// group max over the LPG lanes that share a group (LPG power of two <= 64)
+template <int LPG>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+    for (int o = LPG / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+template <int LPG>
+__device__ __forceinline__ float group_min(float v) {
+#pragma unroll
+    for (int o = LPG / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// ---------------------------------------------------------------- 1 x block activation quant
+// LPG lanes cooperate on one group of LPG*8 contiguous elements.
+template <int DT, int LPG, bool FP8>
+__global__ void act_quant_kernel(const void* __restrict__ x, void* __restrict__ y, void* __restrict__ s,
+                                 int64_t n_groups, int mode) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t grp = tid / LPG;
+    const bool live = grp < n_groups;
+    const int64_t gsafe = live ? grp : 0;
+    const int64_t off = gsafe * (LPG * EPL) + (tid % LPG) * EPL;
+    float v[EPL];
+    load8<DT>(x, off, v);
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) m = fmaxf(m, fabsf(v[j]));
+    m = group_max<LPG>(m);
+    if (!live) return;
+    if constexpr (FP8) {
+        const float sc = m / 448.f;
+        float q[EPL];
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) q[j] = v[j] / sc;
+        uint2 o;
+        o.x = pack_fp8x4(q[0], q[1], q[2], q[3]);
+        o.y = pack_fp8x4(q[4], q[5], q[6], q[7]);
+        *(uint2*)((uint8_t*)y + off) = o;
+        if (tid % LPG == 0) ((float*)s)[grp] = sc;
+    } else {
+        const float sc = m / 127.f;
+        unsigned w[2] = {0, 0};
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) {
+            int qi = (int)round_mode(v[j] / sc, mode);
+            w[j >> 2] |= ((unsigned)(qi & 0xff)) << (8 * (j & 3));
+        }
+        *(uint2*)((int8_t*)y + off) = make_uint2(w[0], w[1]);
+        if (tid % LPG == 0) ((unsigned short*)s)[grp] = f32_to_f16(sc);
+    }
+}
+
+// ---------------------------------------------------------------- block x block weight quant
+// one 256-thread workgroup per (BLOCK x BLOCK) tile, BLOCK <= 128, BLOCK % 8 == 0.
+// thread t: column chunk (t % 16) * 8, rows t / 16 + 16 * j.
+template <int DT, bool FP8>
+__global__ void weight_quant_block_kernel(const void* __restrict__ x, void* __restrict__ y, void* __restrict__ s,
+                                          int64_t M, int64_t N, int block, float qmax, int mode, int clamp) {
+    __shared__ float red[4];
+    const int nb = (int)((N + block - 1) / block);
+    const int64_t r0 = (int64_t)blockIdx.y * block, c0 = (int64_t)blockIdx.x * block;
+    const int t = threadIdx.x;
+    const int cc = (t & 15) * EPL;
+    float v[8][EPL];
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int rr = (t >> 4) + 16 * j;
+        const int64_t r = r0 + rr;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const int64_t c = c0 + cc + e;
+            float val = 0.f;
+            if (rr < block && cc + e < block && r < M && c < N) {
+                val = FloatIO<DT>::ld(x, r * N + c);
+            }
+            v[j][e] = val;
+            m = fmaxf(m, fabsf(val));
+        }
+    }
+    m = wave_max(m);
+    if ((t & 63) == 0) red[t >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float sc = m / qmax;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int rr = (t >> 4) + 16 * j;
+        const int64_t r = r0 + rr;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const int64_t c = c0 + cc + e;
+            if (rr < block && cc + e < block && r < M && c < N) {
+                float q = v[j][e] / sc;
+                if constexpr (FP8) {
+                    unsigned w = pack_fp8x4(q, 0.f, 0.f, 0.f);
+                    ((uint8_t*)y)[r * N + c] = (uint8_t)(w & 0xff);
+                } else {
+                    q = round_mode(q, mode);
+                    if (clamp) q = fminf(fmaxf(q, -qmax), qmax);
+                    ((int8_t*)y)[r * N + c] = (int8_t)(int)q;
+                }
+            }
+        }
+    }
+    if (t == 0) {
+        if constexpr (FP8) ((float*)s)[(int64_t)blockIdx.y * nb + blockIdx.x] = sc;
+        else ((unsigned short*)s)[(int64_t)blockIdx.y * nb + blockIdx.x] = f32_to_f16(sc);
+    }
+}
+
+// ---------------------------------------------------------------- w4a8 second level (in place)
+template <int LPG>
+__global__ void w4a8_level2_kernel(int8_t* __restrict__ y, int8_t* __restrict__ s4, int8_t* __restrict__ z4,
+                                   int64_t n_groups) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t grp = tid / LPG;
+    const bool live = grp < n_groups;
+    const int64_t off = (live ? grp : 0) * (LPG * EPL) + (tid % LPG) * EPL;
+    uint2 u = *(const uint2*)(y + off);
+    float v[EPL];
+    unsigned w[2] = {u.x, u.y};
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) v[j] = (float)(int8_t)((w[j >> 2] >> (8 * (j & 3))) & 0xff);
+    float mx = v[0], mn = v[0];
+#pragma unroll
+    for (int j = 1; j < EPL; ++j) { mx = fmaxf(mx, v[j]); mn = fminf(mn, v[j]); }
+    mx = group_max<LPG>(mx);
+    mn = group_min<LPG>(mn);
+    if (!live) return;
+    const float fs4 = floorf((mx - mn) / 15.0f + 0.5f);
+    const float fz4 = floorf(-mn / fs4 + 0.5f);
+    unsigned o[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+        float q = floorf(v[j] / fs4 + 0.5f) + fz4;
+        q = fminf(fmaxf(q, 0.f), 15.f);
+        o[j >> 2] |= ((unsigned)((int)q & 0xff)) << (8 * (j & 3));
+    }
+    *(uint2*)(y + off) = make_uint2(o[0], o[1]);
+    if (tid % LPG == 0) { s4[grp] = (int8_t)(int)fs4; z4[grp] = (int8_t)(int)fz4; }
+}
+
+// ---------------------------------------------------------------- dequantizers
+template <int ODT, int SDT, bool FP8>
+__global__ void weight_dequant_block_kernel(const uint8_t* __restrict__ x, const void* __restrict__ s,
+                                            void* __restrict__ y, int64_t M, int64_t N, int block) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= M * N) return;
+    const int64_t r = idx / N, c = idx - r * N;
+    const int64_t nb = (N + block - 1) / block;
+    const float sc = FloatIO<SDT>::ld(s, (r / block) * nb + c / block);
+    float xv;
+    if constexpr (FP8) {
+        xv = __builtin_amdgcn_cvt_f32_fp8((int)x[idx], 0);
+    } else {
+        xv = (float)(int8_t)x[idx];
+    }
+    FloatIO<ODT>::st(y, idx, xv * sc);
+}
+
+__global__ void w4a8_dequant_kernel(const int32_t* __restrict__ packed, const unsigned short* __restrict__ s,
+                                    const int8_t* __restrict__ s4, const int8_t* __restrict__ z4,
+                                    unsigned short* __restrict__ y, int64_t N, int64_t K, int block, int group) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t np = N / 8;
+    if (idx >= np * K) return;
+    const int64_t pr = idx / K, k = idx - pr * K;
+    const unsigned w = (unsigned)packed[idx];
+    const int64_t kg = (K + group - 1) / group, kb = (K + block - 1) / block;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int64_t n = pr * 8 + i;
+        const int8_t q = (int8_t)((w >> (4 * i)) & 0xf);
+        const int8_t d = (int8_t)(q - z4[n * kg + k / group]);
+        const int8_t d8 = (int8_t)(d * s4[n * kg + k / group]);   // int8 wrap-around, as the reference evaluates it
+        const float sc = f16_to_f32(s[(n / block) * kb + k / block]);
+        y[n * K + k] = f32_to_f16((float)d8 * sc);
+    }
+}
+
+bool lpg_ok(int block) {
+    return block == 8 || block == 16 || block == 32 || block == 64 || block == 128 || block == 256 || block == 512;
+}
+
+}  // namespace
+
+#define LPG_SWITCH(block, CALL)                                                       \
+    switch ((block) / EPL) {                                                          \
+        case 1: CALL(1); break;  case 2: CALL(2); break;  case 4: CALL(4); break;     \
+        case 8: CALL(8); break;  case 16: CALL(16); break; case 32: CALL(32); break;  \
+        default: CALL(64); break;                                                     \
+    }
+
+extern "C" int llmk_act_quant_fp8(const void* x, int x_dtype, void* y, float* s, int64_t n_groups,
+                                  int block, void* stream) {
+    if (!lpg_ok(block)) LLMK_FAIL(LLMK_ERR_SHAPE, "act_quant_fp8: block %d unsupported (power of two in 8..512)", block);
+    if (n_groups == 0) return LLMK_OK;
+    if (!x || !y || !s || n_groups < 0) LLMK_FAIL(LLMK_ERR_ARG, "act_quant_fp8: bad argument");
+    const int64_t threads = n_groups * (block / EPL);
+    dim3 grid((unsigned)cdiv64(threads, 256)), blk(256);
+#define CALL(L) LLMK_DISPATCH_FLOAT(x_dtype, DT, (act_quant_kernel<DT, L, true><<<grid, blk, 0, (hipStream_t)stream>>>(x, y, s, n_groups, 0)))
+    LPG_SWITCH(block, CALL)
+#undef CALL
+    LLMK_CHECK_LAUNCH("act_quant_fp8");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_act_quant_i8(const void* x, int x_dtype, int8_t* y, void* s, int64_t n_groups,
+                                 int block, int round_mode, void* stream) {
+    if (!lpg_ok(block)) LLMK_FAIL(LLMK_ERR_SHAPE, "act_quant_i8: block %d unsupported (power of two in 8..512)", block);
+    if (round_mode != LLMK_ROUND_HALF_AWAY && round_mode != LLMK_ROUND_HALF_UP)
+        LLMK_FAIL(LLMK_ERR_DTYPE, "act_quant_i8: round_mode %d", round_mode);
+    if (n_groups == 0) return LLMK_OK;
+    if (!x || !y || !s || n_groups < 0) LLMK_FAIL(LLMK_ERR_ARG, "act_quant_i8: bad argument");
+    const int64_t threads = n_groups * (block / EPL);
+    dim3 grid((unsigned)cdiv64(threads, 256)), blk(256);
+#define CALL(L) LLMK_DISPATCH_FLOAT(x_dtype, DT, (act_quant_kernel<DT, L, false><<<grid, blk, 0, (hipStream_t)stream>>>(x, y, s, n_groups, round_mode)))
+    LPG_SWITCH(block, CALL)
+#undef CALL
+    LLMK_CHECK_LAUNCH("act_quant_i8");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_weight_quant_i8_block(const void* x, int x_dtype, int8_t* y, void* s, int64_t M, int64_t N,
+                                          int block, float qmax, int round_mode, int clamp, void* stream) {
+    if (block < 8 || block > 128 || block % 8) LLMK_FAIL(LLMK_ERR_SHAPE, "weight_quant_i8_block: block %d (need 8..128, %%8)", block);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!x || !y || !s || M < 0 || N < 0) LLMK_FAIL(LLMK_ERR_ARG, "weight_quant_i8_block: bad argument");
+    dim3 grid((unsigned)cdiv64(N, block), (unsigned)cdiv64(M, block)), blk(256);
+    LLMK_DISPATCH_FLOAT(x_dtype, DT, (weight_quant_block_kernel<DT, false><<<grid, blk, 0, (hipStream_t)stream>>>(x, y, s, M, N, block, qmax, round_mode, clamp)));
+    LLMK_CHECK_LAUNCH("weight_quant_i8_block");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_weight_quant_fp8_block(const void* x, int x_dtype, void* y, float* s, int64_t M, int64_t N,
+                                           int block, void* stream) {
+    if (block < 8 || block > 128 || block % 8) LLMK_FAIL(LLMK_ERR_SHAPE, "weight_quant_fp8_block: block %d (need 8..128, %%8)", block);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!x || !y || !s || M < 0 || N < 0) LLMK_FAIL(LLMK_ERR_ARG, "weight_quant_fp8_block: bad argument");
+    dim3 grid((unsigned)cdiv64(N, block), (unsigned)cdiv64(M, block)), blk(256);
+    LLMK_DISPATCH_FLOAT(x_dtype, DT, (weight_quant_block_kernel<DT, true><<<grid, blk, 0, (hipStream_t)stream>>>(x, y, s, M, N, block, 448.f, 0, 0)));
+    LLMK_CHECK_LAUNCH("weight_quant_fp8_block");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_weight_quant_w4a8_level2(int8_t* y, int8_t* s4, int8_t* z4, int64_t M, int64_t N, int group,
+                                             void* stream) {
+    if (!lpg_ok(group) || N % group) LLMK_FAIL(LLMK_ERR_SHAPE, "w4a8_level2: group %d / N %lld", group, (long long)N);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!y || !s4 || !z4) LLMK_FAIL(LLMK_ERR_ARG, "w4a8_level2: null pointer");
+    const int64_t n_groups = M * (N / group);
+    const int64_t threads = n_groups * (group / EPL);
+    dim3 grid((unsigned)cdiv64(threads, 256)), blk(256);
+#define CALL(L) w4a8_level2_kernel<L><<<grid, blk, 0, (hipStream_t)stream>>>(y, s4, z4, n_groups)
+    LPG_SWITCH(group, CALL)
+#undef CALL
+    LLMK_CHECK_LAUNCH("w4a8_level2");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_weight_dequant_fp8_block(const void* x, const float* s, void* y, int y_dtype, int64_t M, int64_t N,
+                                             int block, void* stream) {
+    if (block < 1) LLMK_FAIL(LLMK_ERR_SHAPE, "weight_dequant_fp8_block: block %d", block);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!x || !s || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_fp8_block: null pointer");
+    dim3 grid((unsigned)cdiv64(M * N, 256)), blk(256);
+    LLMK_DISPATCH_FLOAT(y_dtype, ODT, (weight_dequant_block_kernel<ODT, LLMK_F32, true><<<grid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block)));
+    LLMK_CHECK_LAUNCH("weight_dequant_fp8_block");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_weight_dequant_i8_block(const int8_t* x, const void* s, int s_dtype, void* y, int y_dtype,
+                                            int64_t M, int64_t N, int block, void* stream) {
+    if (block < 1) LLMK_FAIL(LLMK_ERR_SHAPE, "weight_dequant_i8_block: block %d", block);
+    if (M == 0 || N == 0) return LLMK_OK;
+    if (!x || !s || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_i8_block: null pointer");
+    dim3 grid((unsigned)cdiv64(M * N, 256)), blk(256);
+    LLMK_DISPATCH_FLOAT(y_dtype, ODT, LLMK_DISPATCH_FLOAT(s_dtype, SDT, (weight_dequant_block_kernel<ODT, SDT, false><<<grid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block))));
+    LLMK_CHECK_LAUNCH("weight_dequant_i8_block");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_weight_dequant_w4a8(const int32_t* packed, const void* s, const int8_t* s4, const int8_t* z4,
+                                        void* y, int64_t N, int64_t K, int block, int group, void* stream) {
+    if (N % 8 || block < 1 || group < 1) LLMK_FAIL(LLMK_ERR_SHAPE, "weight_dequant_w4a8: N %% 8 != 0 or bad block/group");
+    if (N == 0 || K == 0) return LLMK_OK;
+    if (!packed || !s || !s4 || !z4 || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_w4a8: null pointer");
+    dim3 grid((unsigned)cdiv64((N / 8) * K, 256)), blk(256);
+    w4a8_dequant_kernel<<<grid, blk, 0, (hipStream_t)stream>>>(packed, (const unsigned short*)s, s4, z4,
+                                                               (unsigned short*)y, N, K, block, group);
+    LLMK_CHECK_LAUNCH("weight_dequant_w4a8");
+    return LLMK_OK;
+}

@@ -1,0 +1,36 @@
+"""W4A16 GEMM for weights kept in the plain [N, K] bit-packed layout.
+
+W [N, K] is quantised symmetrically along K in groups (s = absmax / 7, q = clamp(rne(w / s), -8, 7) + 8)
+and stored with quantization.bitpack.pack_weights_over_cols as int32 [N, K/8] (nibble i of a word is
+k = 8*word + i).  The simple-Marlin layout has its own entry point (simple_marlin.marlin.mul).
+"""
+import torch
+
+from .. import _lib
+from ..quantization.bitpack import pack_weights_over_cols
+
+
+def quantize_nk(w: torch.Tensor, group_size: int = 128):
+    """W [N, K] float -> (packed int32 [N, K/8], scales fp16 [N, K/group_size], q uint8 [N, K])."""
+    assert w.dim() == 2 and w.shape[1] % group_size == 0
+    N, K = w.shape
+    g = w.float().reshape(N, K // group_size, group_size)
+    s = (g.abs().amax(dim=2) / 7.0).to(torch.float16)
+    q = (torch.clamp(torch.round(g / s.float().unsqueeze(-1)), -8, 7) + 8).reshape(N, K).to(torch.uint8)
+    packed, _ = pack_weights_over_cols(q, 4, 32, transpose=False)
+    return packed, s, q
+
+
+def w4a16_gemm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, group_size: int = 128):
+    """y[..., n] = sum_k x[..., k] * (nibble(n, k) - 8) * scales[n, k // group_size]; fp16 in / out."""
+    assert x.is_contiguous() and w_packed.is_contiguous() and scales.is_contiguous(), 'Input tensors must be contiguous'
+    assert w_packed.dtype == torch.int32 and scales.dtype == torch.float16
+    _lib.require_gpu(x, w_packed, scales)
+    K = x.size(-1)
+    M = x.numel() // K
+    N = w_packed.size(0)
+    assert w_packed.size(1) * 8 == K, 'packed weight must be [N, K/8]'
+    y = x.new_empty(*x.size()[:-1], N)
+    _lib.call("llmk_gemm_w4a16_nk", _lib.ptr(x), _lib.ptr(w_packed), _lib.ptr(y), _lib.ptr(scales),
+              _lib.dt(x.dtype), M, N, K, group_size, None, 0, _lib.stream(x), exc=AssertionError)
+    return y

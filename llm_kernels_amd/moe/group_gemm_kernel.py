@@ -1,0 +1,178 @@
+"""EP-MoE device ops on MI355X (reference moe/group_gemm_kernel.py).
+
+run_moe_ep_preproess (:48), grouped_gemm_triton (:442) keep their names and signatures.  The four
+Triton kernels of the reference (pre_reorder :81, silu_and_mul :120, gelu_and_mul :176,
+post_reorder :238) are exposed twice: as plain functions, and as `*_triton_kernel` objects that
+accept the reference's `kernel[grid](args..., BLOCK_SIZE=...)` call form, so that a caller written
+against the reference runs unchanged.
+"""
+from typing import List, Optional
+
+import torch
+
+from .. import _lib
+
+
+def _cdiv(a, b):
+    return (a + b - 1) // b
+
+
+def run_moe_ep_preproess(topk_ids: torch.Tensor, num_experts: int):
+    """Stable sort of the flattened expert ids -> (sorted ids, src2dst int32 [T*topk], seg_indptr int64 [E+1])."""
+    _lib.require_gpu(topk_ids)
+    reorder_topk_ids, reorder_ids = torch.sort(topk_ids.view(-1), stable=True)
+    n = topk_ids.numel()
+    seg_indptr = torch.zeros(num_experts + 1, device=topk_ids.device, dtype=torch.int64)
+    src2dst = torch.empty(n, device=topk_ids.device, dtype=torch.int32)
+    st = _lib.stream(topk_ids)
+    sorted64 = reorder_topk_ids if reorder_topk_ids.dtype == torch.int64 else reorder_topk_ids.to(torch.int64)
+    _lib.call("llmk_moe_seg_indptr", _lib.ptr(sorted64), _lib.ptr(seg_indptr), n, num_experts, st)
+    _lib.call("llmk_moe_src2dst", _lib.ptr(reorder_ids), _lib.ptr(src2dst), n, st)
+    return reorder_topk_ids, src2dst, seg_indptr
+
+
+def _ids_bytes(t):
+    if t.dtype == torch.int64:
+        return 8
+    if t.dtype == torch.int32:
+        return 4
+    raise TypeError("expert id tensors must be int32 or int64, got %s" % t.dtype)
+
+
+def _f32_or_none(t):
+    return None if t is None else t.float().contiguous()
+
+
+def pre_reorder(input, gateup_input, src2dst, topk_ids, a1_scales, start_expert_id, end_expert_id, topk,
+                hidden_size):
+    """gateup_input[src2dst[t, j]] = input[t] * (1 / a1_scales[e] or 1) for every local expert e of token t."""
+    _lib.require_gpu(input, gateup_input, src2dst, topk_ids)
+    assert input.is_contiguous() and gateup_input.is_contiguous() and src2dst.is_contiguous() and topk_ids.is_contiguous()
+    sc = _f32_or_none(a1_scales)
+    T = input.numel() // hidden_size
+    _lib.call("llmk_moe_pre_reorder", _lib.ptr(input), _lib.dt(input.dtype), _lib.ptr(gateup_input),
+              _lib.dt(gateup_input.dtype), _lib.ptr(src2dst), _lib.ptr(topk_ids), _ids_bytes(topk_ids), _lib.ptr(sc),
+              int(start_expert_id), int(end_expert_id), int(topk), T, int(hidden_size), _lib.stream(input))
+    return gateup_input
+
+
+def _act_and_mul(act, gateup_output, down_input, hidden_size, reorder_topk_ids, scales, start_expert_id,
+                 end_expert_id):
+    _lib.require_gpu(gateup_output, down_input, reorder_topk_ids)
+    assert gateup_output.is_contiguous() and down_input.is_contiguous() and reorder_topk_ids.is_contiguous()
+    sc = _f32_or_none(scales)
+    M = gateup_output.numel() // hidden_size
+    _lib.call("llmk_moe_act_and_mul", _lib.ptr(gateup_output), _lib.dt(gateup_output.dtype), _lib.ptr(down_input),
+              _lib.dt(down_input.dtype), _lib.ptr(reorder_topk_ids), _ids_bytes(reorder_topk_ids), _lib.ptr(sc),
+              int(start_expert_id), int(end_expert_id), M, int(hidden_size), act, _lib.stream(gateup_output))
+    return down_input
+
+
+def silu_and_mul(gateup_output, down_input, hidden_size, reorder_topk_ids, scales, start_expert_id, end_expert_id):
+    """down_input[r] = dtype(silu_fp32(gate)) * up * (1/scale[e]); gate = cols [0, I), up = [I, 2I)."""
+    return _act_and_mul(0, gateup_output, down_input, hidden_size, reorder_topk_ids, scales, start_expert_id,
+                        end_expert_id)
+
+
+def gelu_and_mul(gateup_output, down_input, hidden_size, reorder_topk_ids, scales, start_expert_id, end_expert_id):
+    return _act_and_mul(1, gateup_output, down_input, hidden_size, reorder_topk_ids, scales, start_expert_id,
+                        end_expert_id)
+
+
+def post_reorder(down_output, output, src2dst, topk_ids, topk_weights, start_expert_id, end_expert_id, topk,
+                 hidden_size):
+    """output[t] = sum_j down_output[src2dst[t, j]] * dtype(topk_weights[t, j]), summed in the tensor dtype."""
+    _lib.require_gpu(down_output, output, src2dst, topk_ids, topk_weights)
+    assert down_output.is_contiguous() and output.is_contiguous() and topk_weights.is_contiguous()
+    assert down_output.dtype == output.dtype
+    T = output.numel() // hidden_size
+    _lib.call("llmk_moe_post_reorder", _lib.ptr(down_output), _lib.ptr(output), _lib.dt(output.dtype),
+              _lib.ptr(src2dst), _lib.ptr(topk_ids), _ids_bytes(topk_ids), _lib.ptr(topk_weights),
+              _lib.dt(topk_weights.dtype), int(start_expert_id), int(end_expert_id), int(topk), T,
+              int(hidden_size), _lib.stream(output))
+    return output
+
+
+class _GridCall:
+    """Accepts `obj[grid](*args, BLOCK_SIZE=...)`; the grid and the tile size are chosen by the HIP launcher."""
+
+    def __init__(self, fn):
+        self._fn = fn
+        self.__doc__ = fn.__doc__
+
+    def __getitem__(self, grid):
+        def launch(*args, BLOCK_SIZE=None, **kw):
+            return self._fn(*args, **kw)
+        return launch
+
+    def __call__(self, *args, BLOCK_SIZE=None, **kw):
+        return self._fn(*args, **kw)
+
+
+pre_reorder_triton_kernel = _GridCall(pre_reorder)
+silu_and_mul_triton_kernel = _GridCall(silu_and_mul)
+gelu_and_mul_triton_kernel = _GridCall(gelu_and_mul)
+post_reorder_triton_kernel = _GridCall(post_reorder)
+
+
+def grouped_gemm_triton(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    c: torch.Tensor,
+    batch_size: int,
+    weight_column_major: bool,
+    seg_indptr: Optional[torch.Tensor] = None,
+    weight_indices: Optional[torch.Tensor] = None,
+    use_fp8_w8a8: bool = False,
+    scale_a: torch.Tensor = None,
+    scale_b: torch.Tensor = None,
+    block_shape: Optional[List[int]] = None,
+):
+    """c[seg[e]:seg[e+1]] = a[seg[e]:seg[e+1]] @ b[weight_indices[e]]^T for e < batch_size; c is written in place.
+
+    With `block_shape` and quantised weights the activations are quantised here per 1 x block_k group:
+    int8 weights -> int8 activations (the reference behaviour), float8_e4m3fn weights -> e4m3 activations.
+    """
+    assert weight_column_major == True  # noqa: E712  (same precondition as the reference)
+    if use_fp8_w8a8 and block_shape is None:
+        assert scale_a is not None and scale_b is not None
+    _lib.require_gpu(a, b, c)
+    assert seg_indptr is not None, 'seg_indptr is required'
+    quantised_w = b.dtype in (torch.int8, torch.float8_e4m3fn)
+    if block_shape is not None and quantised_w:
+        assert len(block_shape) == 2
+        block_n, block_k = block_shape[0], block_shape[1]
+        assert block_n == 128 and block_k == 128, 'block-scaled grouped GEMM uses 128 x 128 weight blocks'
+        if b.dtype == torch.int8:
+            from ..quantization.int8_kernel import act_quant as per_token_group_quant
+        else:
+            from ..quantization.fp8_kernel import act_quant as per_token_group_quant
+        a, scale_a = per_token_group_quant(a.contiguous(), block_k)
+        assert _cdiv(a.shape[-1], block_k) == scale_a.shape[-1]
+        assert _cdiv(b.shape[-2], block_n) == scale_b.shape[-2]
+        assert _cdiv(b.shape[-1], block_k) == scale_b.shape[-1]
+    elif quantised_w:
+        raise AssertionError('quantised weights need block_shape=[128, 128] and scale_b')
+    assert a.is_contiguous() and b.is_contiguous() and c.is_contiguous(), 'Input tensors must be contiguous'
+    assert b.dim() == 3 and a.shape[-1] == b.shape[-1] and c.shape[-1] == b.shape[1] and c.shape[0] == a.shape[0]
+    assert a.dtype == b.dtype, 'a and b must share a dtype after activation quantisation'
+    kind = {torch.int8: _lib.KIND_I8, torch.float8_e4m3fn: _lib.KIND_FP8,
+            torch.float16: _lib.KIND_F16, torch.bfloat16: _lib.KIND_BF16}.get(b.dtype)
+    assert kind is not None, 'unsupported operand dtype %s' % b.dtype
+    s_dt = 0
+    if kind in (_lib.KIND_I8, _lib.KIND_FP8):
+        scale_b = scale_b.contiguous()
+        if scale_b.dtype != scale_a.dtype:
+            scale_b = scale_b.to(scale_a.dtype)
+        s_dt = _lib.dt(scale_a.dtype)
+    else:
+        scale_a = scale_b = None
+    seg = seg_indptr if seg_indptr.dtype == torch.int64 else seg_indptr.to(torch.int64)
+    seg = seg.contiguous()
+    wi = None
+    if weight_indices is not None:
+        wi = (weight_indices if weight_indices.dtype == torch.int64 else weight_indices.to(torch.int64)).contiguous()
+    _lib.call("llmk_grouped_gemm", _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), kind, _lib.dt(c.dtype), int(batch_size),
+              a.shape[0], b.shape[1], b.shape[2], _lib.ptr(seg), _lib.ptr(wi), _lib.ptr(scale_a), _lib.ptr(scale_b),
+              s_dt, _lib.stream(a), exc=AssertionError)
+    return c
