@@ -107,7 +107,7 @@ int llmk_gemm_fp8_block(const void* a_e4m3, const float* a_s, const void* b_e4m3
 int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const void* b_s,
                        int s_dtype, void* c, int c_dtype, int64_t M, int64_t N, int64_t K,
                        void* workspace, int64_t workspace_bytes, void* stream);
-/* per-token x per-channel W8A8 with one full-K int32 accumulation (the BASELINE config-2 scheme;
+/* per-token x per-channel W8A8 with one full-K int32 accumulation (a scheme with
  * no counterpart function in the reference).  c may be NULL; c_i32 (raw accumulators) may be NULL. */
 int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, const float* b_s,
                         void* c, int c_dtype, int32_t* c_i32, int64_t M, int64_t N, int64_t K,
@@ -126,11 +126,14 @@ int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, co
  * additionally N % 64 == 0 and groupsize % 16 == 0.
  * ref: fast_dequant/simple_marlin/marlin_w4a16_gemm.cu:283-326 (simple_marlin_cuda),
  *      marlin_w4a16_gemm.cpp:23-111 (mul).                                                    */
+/* bytes of fp32 split-K scratch llmk_gemm_w4a16_marlin uses for this shape (0 = none). Without it
+ * (workspace NULL / too small) the kernel runs with fewer K slices. */
+int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int llmk_gemm_w4a16_marlin(const void* a_f16, const int32_t* b, void* c_f16, const void* s_f16,
                            int64_t M, int64_t N, int64_t K, int groupsize,
                            void* workspace, int64_t workspace_bytes, void* stream);
 /* Same product for W stored [N, K/8] int32 by pack_weights_over_cols (nibble i of a word = k*8+i)
- * with s fp16 [N, K/g]; a/c fp16 or bf16 (dtype code).  BASELINE config-1 layout. */
+ * with s fp16 [N, K/g]; a/c fp16 or bf16 (dtype code).  fp16 only at present. */
 int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s_f16,
                        int ac_dtype, int64_t M, int64_t N, int64_t K, int groupsize,
                        void* workspace, int64_t workspace_bytes, void* stream);

@@ -41,6 +41,7 @@ SIGNATURES = {
     "llmk_gemm_i8_block": [_p, _p, _p, _p, _i, _p, _i, _l, _l, _l, _p, _l, _p],
     "llmk_gemm_i8_rowcol": [_p, _p, _p, _p, _p, _i, _p, _l, _l, _l, _p],
     "llmk_gemm_w4a8": [_p, _p, _p, _p, _i, _p, _p, _p, _i, _l, _l, _l, _i, _p, _l, _p],
+    "llmk_gemm_w4a16_marlin_workspace_bytes": [_l, _l, _l],
     "llmk_gemm_w4a16_marlin": [_p, _p, _p, _p, _l, _l, _l, _i, _p, _l, _p],
     "llmk_gemm_w4a16_nk": [_p, _p, _p, _p, _i, _l, _l, _l, _i, _p, _l, _p],
     "llmk_moe_seg_indptr": [_p, _p, _l, _i, _p],
@@ -50,7 +51,8 @@ SIGNATURES = {
     "llmk_moe_post_reorder": [_p, _p, _i, _p, _p, _i, _p, _i, _i, _i, _i, _l, _l, _p],
     "llmk_grouped_gemm": [_p, _p, _p, _i, _i, _i, _l, _l, _l, _p, _p, _p, _p, _i, _p],
 }
-_RESTYPE = {"llmk_last_error": _c.c_char_p, "llmk_gemm_workspace_bytes": _l}
+_RESTYPE = {"llmk_last_error": _c.c_char_p, "llmk_gemm_workspace_bytes": _l,
+            "llmk_gemm_w4a16_marlin_workspace_bytes": _l}
 
 _lib = None
 

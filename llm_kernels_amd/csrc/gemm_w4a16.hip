@@ -211,7 +211,20 @@ __global__ __launch_bounds__(NW * 64) void w4a16_nk_kernel(
         }
 }
 
+// number of K slices (workgroups along z) used for decode-sized M
+int marlin_split_k(int col_groups, int total_steps) {
+    int z = 1;
+    while (col_groups * z < 256 && total_steps / (z * 2) >= 8) z *= 2;
+    return z;
+}
+
 }  // namespace
+
+extern "C" int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || M > 16) return 0;
+    const int z = marlin_split_k((int)((N / 64 + 1) / 2), (int)((K / 16 + 1) / 2));
+    return z > 1 ? (int64_t)z * M * N * 4 : 0;
+}
 
 extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, const void* s, int64_t M, int64_t N,
                                       int64_t K, int groupsize, void* workspace, int64_t workspace_bytes,
@@ -240,10 +253,8 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
     if (M <= 16) {
         constexpr int NW = 8;
         // split K over workgroups until the grid covers the chip; each workgroup keeps >= NW steps
-        int z = 1;
-        while (col_groups * z < 256 && total_steps / (z * 2) >= NW) z *= 2;
-        const int64_t need = (int64_t)z * M * N * 4;
-        if (z > 1 && (!workspace || workspace_bytes < need)) z = 1;
+        int z = marlin_split_k(col_groups, total_steps);
+        while (z > 1 && (!workspace || workspace_bytes < (int64_t)z * M * N * 4)) z >>= 1;
         const int spz = (total_steps + z - 1) / z;
         dim3 grid(col_groups, 1, z), blk(NW * 64);
         const size_t smem = (size_t)(NW / 2) * 32 * 64 * sizeof(float);

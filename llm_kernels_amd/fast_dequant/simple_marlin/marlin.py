@@ -38,7 +38,7 @@ def mul(A, B, C, s, workspace, thread_k=-1, thread_n=-1, sms=-1, max_par=16):
             raise RuntimeError(f"K dimension not divisible by groupsize: K={prob_k}, groupsize={groupsize}")
     if B_c.numel() * 8 != prob_k * prob_n:
         raise RuntimeError("B does not hold K*N packed 4-bit values")
-    ws_bytes = 8 * prob_m * prob_n * 4 if prob_m <= 16 else 0
+    ws_bytes = _lib.load().llmk_gemm_w4a16_marlin_workspace_bytes(prob_m, prob_n, prob_k)
     ws = _lib.workspace(A.device, ws_bytes) if ws_bytes else None
     _lib.call("llmk_gemm_w4a16_marlin", _lib.ptr(A_c), _lib.ptr(B_c), _lib.ptr(C), _lib.ptr(s_c),
               prob_m, prob_n, prob_k, groupsize, _lib.ptr(ws), ws.numel() if ws is not None else 0,

@@ -144,7 +144,7 @@ def w4a8_weight_dequant(q, s, s4, z4, block_size=128, group_size_int4=128):
 def w4a16_quant_nk(w, group_size=128):
     """Symmetric int4 along K for W [N,K]: s = absmax/7 (fp16), q = clamp(rne(w/s), -8, 7) + 8.
 
-    This is the BASELINE config-1 wording (not the Marlin 2*absmax/15 rule).
+    This is the absmax/7 rule (not the Marlin 2*absmax/15 rule).
     """
     N, K = w.shape
     g = w.float().reshape(N, K // group_size, group_size)

@@ -1,0 +1,155 @@
+"""HIP block-scaled GEMMs vs the float64 oracle.
+
+Tolerance: |c - ref| <= 1e-2 * rms(ref) + 1e-2 * |ref| (rtol 1e-2 / atol 1e-2 relative to the output
+scale).  Integer accumulators are checked bit-exactly.
+"""
+import pytest
+import torch
+
+from oracle import gemm_ref as g, quant_ref as q, bitpack_ref as bp
+from llm_kernels_amd.quantization import fp8_kernel, int8_kernel, w4a8_kernel
+from helpers import announce, assert_close_scaled, default_dtype
+
+pytestmark = pytest.mark.gpu
+
+SMALL = [(1, 128, 128), (16, 256, 512), (5, 130, 256), (33, 200, 384), (70, 64, 1024), (128, 512, 256)]
+
+
+def _quant_inputs_fp8(M, N, K, seed):
+    torch.manual_seed(seed)
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    a, a_s = q.act_quant_fp8(x)
+    b, b_s = q.weight_quant_fp8(w)
+    return a, a_s, b, b_s
+
+
+@pytest.mark.parametrize("M,N,K", SMALL)
+@pytest.mark.parametrize("out", [torch.bfloat16, torch.float16, torch.float32])
+def test_fp8_gemm_small(dev, M, N, K, out):
+    announce("fp8_gemm", M, N, K, out)
+    a, a_s, b, b_s = _quant_inputs_fp8(M, N, K, M + N)
+    with default_dtype(out):
+        c = fp8_kernel.fp8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert c.dtype == out and c.shape == (M, N)
+    assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="fp8_gemm")
+
+
+def test_fp8_gemm_batched_leading_dims_and_asserts(dev):
+    announce("fp8_gemm leading dims")
+    a, a_s, b, b_s = _quant_inputs_fp8(6, 256, 256, 3)
+    with default_dtype(torch.bfloat16):
+        c = fp8_kernel.fp8_gemm(a.view(2, 3, 256).to(dev), a_s.view(2, 3, 2).to(dev), b.to(dev), b_s.to(dev))
+    assert c.shape == (2, 3, 256)
+    assert_close_scaled(c.view(6, 256), g.gemm_blockwise(a, a_s, b, b_s))
+    with pytest.raises(AssertionError):
+        fp8_kernel.fp8_gemm(a.to(dev).t(), a_s.to(dev), b.to(dev), b_s.to(dev))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (16, 4096, 4096), (16, 6144, 4096), (256, 4096, 4096)])
+def test_fp8_gemm_llama_shapes(dev, M, N, K):
+    announce("fp8_gemm llama", M, N, K)
+    a, a_s, b, b_s = _quant_inputs_fp8(M, N, K, 11)
+    with default_dtype(torch.bfloat16):
+        c = fp8_kernel.fp8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="fp8 llama")
+
+
+def test_fp8_gemm_quantize_on_device_end_to_end(dev):
+    """act_quant + weight_quant + fp8_gemm on the GPU against the unquantised product (reference-style check)."""
+    announce("fp8 end to end 64x4096x14336")
+    torch.manual_seed(5)
+    x = torch.randn(64, 14336, device=dev).bfloat16()
+    w = (torch.randn(4096, 14336, device=dev) * 0.02)
+    a, a_s = fp8_kernel.act_quant(x)
+    b, b_s = fp8_kernel.weight_quant(w)
+    with default_dtype(torch.bfloat16):
+        c = fp8_kernel.fp8_gemm(a, a_s, b, b_s)
+    ref = x.float() @ w.t()
+    cos = torch.nn.functional.cosine_similarity(c.float().flatten(), ref.flatten(), dim=0)
+    assert cos > 0.999
+    assert_close_scaled(c, g.gemm_blockwise(a.cpu(), a_s.cpu(), b.cpu(), b_s.cpu()), what="fp8 e2e")
+
+
+# ------------------------------------------------------------------------------------------- int8
+@pytest.mark.parametrize("M,N,K", SMALL + [(16, 4096, 4096), (128, 14336, 4096)])
+def test_int8_gemm(dev, M, N, K):
+    announce("int8_gemm", M, N, K)
+    torch.manual_seed(M * 7 + N)
+    a, a_s = q.act_quant_int8(torch.randn(M, K))
+    b, b_s = q.weight_quant_int8(torch.randn(N, K) * 0.02)
+    with default_dtype(torch.bfloat16):
+        c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert c.dtype == torch.bfloat16
+    assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="int8_gemm")
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 128, 128), (16, 256, 4096), (37, 130, 512), (128, 512, 14336)])
+def test_int8_block_accumulators_bit_exact(dev, M, N, K):
+    """Unit scales and fp32 output: the result is the exact integer product (every 128-K int32 partial
+    and their sum stay below 2^24 for |values| <= 15)."""
+    announce("int8 exact", M, N, K)
+    torch.manual_seed(K)
+    a = torch.randint(-15, 16, (M, K), dtype=torch.int8)
+    b = torch.randint(-15, 16, (N, K), dtype=torch.int8)
+    a_s = torch.ones(M, K // 128, dtype=torch.float16)
+    b_s = torch.ones((N + 127) // 128, K // 128, dtype=torch.float16)
+    with default_dtype(torch.float32):
+        c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert torch.equal(c.cpu().long(), a.long() @ b.long().T)
+    # full-range values, one K block: a single int32 partial (|sum| <= 128*127*127 < 2^24) is exact in fp32
+    a1 = torch.randint(-127, 128, (M, 128), dtype=torch.int8)
+    b1 = torch.randint(-127, 128, (N, 128), dtype=torch.int8)
+    with default_dtype(torch.float32):
+        c1 = int8_kernel.int8_gemm(a1.to(dev), a_s[:, :1].contiguous().to(dev), b1.to(dev), b_s[:, :1].contiguous().to(dev))
+    assert torch.equal(c1.cpu().long(), a1.long() @ b1.long().T)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (16, 4096, 4096), (130, 200, 1024), (128, 4096, 14336)])
+def test_int8_per_token_int32_bit_exact(dev, M, N, K):
+    announce("int8 rowcol", M, N, K)
+    torch.manual_seed(M + K)
+    a, a_s = q.int8_quant_rowwise(torch.randn(M, K))
+    b, b_s = q.int8_quant_rowwise(torch.randn(N, K) * 0.02)
+    with default_dtype(torch.bfloat16):
+        c, acc = int8_kernel.int8_gemm_per_token(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev), return_int32=True)
+    assert acc.dtype == torch.int32 and torch.equal(acc.cpu(), g.int8_gemm_int32(a, b))
+    assert_close_scaled(c, g.int8_gemm_rowcol(a, a_s, b, b_s), what="int8 rowcol")
+    ag, asg = int8_kernel.act_quant_per_token(torch.randn(M, K, device=dev))
+    assert ag.dtype == torch.int8 and asg.shape == (M,)
+
+
+# ------------------------------------------------------------------------------------------- w4a8
+@pytest.mark.parametrize("M,N,K", [(1, 128, 128), (16, 256, 512), (37, 136, 256), (16, 4096, 4096), (128, 1024, 7168)])
+def test_w4a8_gemm(dev, M, N, K):
+    announce("w4a8_gemm", M, N, K)
+    torch.manual_seed(N + K)
+    wq, s, s4, z4 = q.w4a8_weight_quant_levels(torch.randn(N, K) * 0.02)
+    a, a_s = q.act_quant_int8(torch.randn(M, K).bfloat16(), rounding="up")
+    packed, _ = bp.pack_rows(wq.numpy(), 4, 32)
+    with default_dtype(torch.bfloat16):
+        c = w4a8_kernel.w4a8_gemm(a.to(dev), a_s.to(dev), torch.from_numpy(packed).to(dev), s.to(dev),
+                                  s4.to(dev), z4.to(dev), 128, 8, "row")
+    assert c.shape == (M, N) and c.dtype == torch.bfloat16
+    assert_close_scaled(c, g.w4a8_gemm(a, a_s, wq, s, s4, z4), what="w4a8_gemm")
+
+
+def test_w4a8_exact_and_wrap(dev):
+    """Unit block scales + fp32 out: exact integers, including out-of-contract s4/z4 that wrap in int8."""
+    announce("w4a8 exact/wrap")
+    torch.manual_seed(9)
+    M, N, K = 8, 64, 256
+    wq = torch.randint(0, 16, (N, K), dtype=torch.uint8)
+    s4 = torch.randint(1, 4, (N, K // 128), dtype=torch.int8)
+    z4 = torch.randint(0, 16, (N, K // 128), dtype=torch.int8)
+    s4[0, 0], z4[0, 0] = 20, 2            # (15 - 2) * 20 = 260 wraps
+    s4[1, 1], z4[1, 1] = -9, 15           # negative scale
+    a = torch.randint(-7, 8, (M, K), dtype=torch.int8)
+    ones_a = torch.ones(M, K // 128, dtype=torch.float16)
+    ones_b = torch.ones(1, K // 128, dtype=torch.float16)
+    packed, _ = bp.pack_rows(wq.numpy(), 4, 32)
+    with default_dtype(torch.float32):
+        c = w4a8_kernel.w4a8_gemm(a.to(dev), ones_a.to(dev), torch.from_numpy(packed).to(dev), ones_b.to(dev),
+                                  s4.to(dev), z4.to(dev))
+    b8 = q.w4a8_dequant_int8(wq, s4, z4)
+    assert torch.equal(c.cpu().long(), a.long() @ b8.long().T)

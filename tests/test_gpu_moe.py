@@ -1,0 +1,167 @@
+"""Single-GPU EP-MoE path vs the torch-CPU oracle."""
+import pytest
+import torch
+
+from oracle import moe_ref as m, quant_ref as q, gemm_ref as g
+from llm_kernels_amd.moe import group_gemm_kernel as gk
+from llm_kernels_amd.moe.ep_moe import ep_moe_forward, softmax_topk_router
+from llm_kernels_amd.quantization import int8_kernel, fp8_kernel
+from helpers import announce, assert_close_scaled
+
+pytestmark = pytest.mark.gpu
+
+
+def test_preprocess_worked_example(dev):
+    announce("moe preprocess example")
+    topk_ids = torch.tensor([[0, 2], [1, 3], [0, 1], [2, 3], [1, 2], [0, 3]], device=dev)
+    rids, src2dst, seg = gk.run_moe_ep_preproess(topk_ids, 4)
+    assert src2dst.tolist() == [0, 6, 3, 9, 1, 4, 7, 10, 5, 8, 2, 11]
+    assert rids.tolist() == [0, 0, 0, 1, 1, 1, 2, 2, 2, 3, 3, 3]
+    assert seg.tolist() == [0, 3, 6, 9, 12] and seg.dtype == torch.int64 and src2dst.dtype == torch.int32
+
+
+@pytest.mark.parametrize("T,E,topk", [(4096, 8, 2), (37, 16, 4), (1, 4, 2), (64, 8, 1)])
+def test_preprocess_random_incl_empty_experts(dev, T, E, topk):
+    announce("moe preprocess", T, E, topk)
+    torch.manual_seed(T)
+    logits = torch.randn(T, E)
+    logits[:, E - 1] = -1e9                                     # last expert never chosen -> empty segment
+    ids = torch.topk(logits, topk, dim=-1)[1]
+    rids, s2d, seg = gk.run_moe_ep_preproess(ids.to(dev), E)
+    orids, os2d, oseg = m.run_moe_ep_preprocess(ids, E)
+    assert torch.equal(rids.cpu(), orids) and torch.equal(s2d.cpu(), os2d) and torch.equal(seg.cpu(), oseg)
+    assert seg[-1].item() == T * topk and seg[E].item() == seg[E - 1].item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_reorder_and_activation_kernels(dev, dtype):
+    announce("moe aux", dtype)
+    torch.manual_seed(1)
+    T, H, I, E, topk = 50, 384, 256, 8, 2
+    x = torch.randn(T, H).to(dtype)
+    ids, w = m.softmax_top2_router(torch.randn(T, E), topk)
+    rids, s2d, seg = m.run_moe_ep_preprocess(ids, E)
+    # local experts 2..5 only: other destination rows stay untouched
+    gin = torch.full((T * topk, H), -3.0, dtype=dtype, device=dev)
+    gk.pre_reorder_triton_kernel[(T,)](x.to(dev), gin, s2d.to(dev), ids.to(dev), None, 2, 5, topk, H, BLOCK_SIZE=512)
+    ogin = m.pre_reorder(x, s2d, ids, None, 2, 5, topk, out=torch.full((T * topk, H), -3.0, dtype=dtype))
+    assert torch.equal(gin.cpu(), ogin)
+    a1 = torch.rand(4) + 0.5
+    gin2 = torch.zeros((T * topk, H), dtype=dtype, device=dev)
+    gk.pre_reorder(x.to(dev), gin2, s2d.to(dev), ids.to(dev), a1.to(dev), 2, 5, topk, H)
+    assert_close_scaled(gin2, m.pre_reorder(x, s2d, ids, a1, 2, 5, topk), rtol=4e-3, atol=1e-6)
+
+    gu = torch.randn(T * topk, 2 * I).to(dtype)
+    for act, fn in (("silu", gk.silu_and_mul_triton_kernel), ("gelu", gk.gelu_and_mul_triton_kernel)):
+        di = torch.zeros(T * topk, I, dtype=dtype, device=dev)
+        fn[(T * topk,)](gu.to(dev), di, 2 * I, rids.to(dev), None, 0, E - 1, BLOCK_SIZE=512)
+        odi, _ = m.silu_and_mul(gu, rids, None, 0, E - 1, act=act)
+        # sigmoid differs by an ulp between libraries; after rounding to the tensor dtype at most one step
+        assert_close_scaled(di, odi, rtol=2 ** -7 if dtype == torch.bfloat16 else 2e-3, atol=1e-5, what=act)
+        exact = (di.cpu() == odi).float().mean().item()
+        assert exact > 0.97, exact
+
+    do = torch.randn(T * topk, H).to(dtype)
+    out = torch.empty(T, H, dtype=dtype, device=dev)
+    gk.post_reorder_triton_kernel[(T,)](do.to(dev), out, s2d.to(dev), ids.to(dev), w.to(dev), 0, E - 1, topk, H,
+                                        BLOCK_SIZE=512)
+    assert torch.equal(out.cpu(), m.post_reorder(do, s2d, ids, w, 0, E - 1, topk))
+    out2 = torch.full((T, H), 9.0, dtype=dtype, device=dev)
+    gk.post_reorder(do.to(dev), out2, s2d.to(dev), ids.to(dev), w.to(dev), 2, 5, topk, H)
+    assert torch.equal(out2.cpu(), m.post_reorder(do, s2d, ids, w, 2, 5, topk))
+
+
+def _segments(T, E, topk, seed, empty_last=True):
+    torch.manual_seed(seed)
+    logits = torch.randn(T, E)
+    if empty_last:
+        logits[:, E - 1] = -1e9
+    ids, w = m.softmax_top2_router(logits, topk)
+    return ids, w, m.run_moe_ep_preprocess(ids, E)
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8", "fp16", "bf16"])
+@pytest.mark.parametrize("T,E,N,K", [(40, 4, 256, 256), (300, 8, 200, 512), (9, 8, 128, 128)])
+def test_grouped_gemm(dev, kind, T, E, N, K):
+    announce("grouped_gemm", kind, T, E, N, K)
+    topk = 2
+    ids, w, (rids, s2d, seg) = _segments(T, E, topk, T + N)
+    M = T * topk
+    torch.manual_seed(3)
+    a = torch.randn(M, K)
+    wts = torch.randn(E, N, K) * 0.05
+    widx = torch.arange(E)
+    out_dt = torch.bfloat16 if kind != "fp16" else torch.float16
+    c = torch.full((M, N), 5.0, dtype=out_dt, device=dev)
+    if kind in ("int8", "fp8"):
+        wq = q.weight_quant_int8 if kind == "int8" else q.weight_quant_fp8
+        aq = q.act_quant_int8 if kind == "int8" else q.act_quant_fp8
+        qs = [wq(wts[e]) for e in range(E)]
+        b = torch.stack([x[0].view(torch.uint8) if kind == "fp8" else x[0] for x in qs])
+        if kind == "fp8":
+            b = b.view(torch.float8_e4m3fn)
+        b_s = torch.stack([x[1] for x in qs])
+        a_in = a.to(out_dt)
+        ret = gk.grouped_gemm_triton(a_in.to(dev), b.to(dev), c, E, True, seg.to(dev), widx.to(dev), False, None,
+                                     b_s.to(dev), [128, 128])
+        a_q, a_s = aq(a_in)
+        ref = m.grouped_gemm(a_q, b, seg, widx, a_s, b_s)
+    else:
+        dt = torch.float16 if kind == "fp16" else torch.bfloat16
+        a_in, b = a.to(dt), wts.to(dt)
+        ret = gk.grouped_gemm_triton(a_in.to(dev), b.to(dev), c, E, True, seg.to(dev), widx.to(dev))
+        ref = m.grouped_gemm(a_in, b, seg, widx)
+    assert ret is c
+    assert_close_scaled(c, ref, what="grouped " + kind)
+
+
+def test_grouped_gemm_single_expert_equals_dense_and_weight_indices(dev):
+    announce("grouped single expert")
+    torch.manual_seed(4)
+    M, N, K = 70, 256, 256
+    a = torch.randn(M, K).bfloat16()
+    w = (torch.randn(3, N, K) * 0.05).bfloat16()
+    seg = torch.tensor([0, M])
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    gk.grouped_gemm_triton(a.to(dev), w.to(dev), c, 1, True, seg.to(dev), torch.tensor([2]).to(dev))
+    assert_close_scaled(c, a.double() @ w[2].double().T, what="single expert")
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8", "bf16"])
+def test_ep_moe_forward_small(dev, kind):
+    announce("ep_moe_forward", kind)
+    torch.manual_seed(5)
+    T, H, I, E, topk = 96, 256, 384, 8, 2
+    dt = torch.bfloat16
+    x = torch.randn(T, H).to(dt)
+    logits = torch.randn(T, E)
+    ids, w = m.softmax_top2_router(logits, topk)
+    w13 = torch.randn(E, 2 * I, H) * 0.05
+    w2 = torch.randn(E, H, I) * 0.05
+    if kind == "bf16":
+        out = ep_moe_forward(x.to(dev), ids.to(dev), w.to(dev), w13.to(dt).to(dev), w2.to(dt).to(dev))
+        dense = m.dense_moe_forward(x, ids, w, w13.to(dt), w2.to(dt))
+        assert_close_scaled(out, dense, rtol=3e-2, atol=3e-2, what="moe bf16 vs dense")
+        return
+    wq = q.weight_quant_int8 if kind == "int8" else q.weight_quant_fp8
+    aq = q.act_quant_int8 if kind == "int8" else q.act_quant_fp8
+    q13 = [wq(w13[e]) for e in range(E)]
+    q2 = [wq(w2[e]) for e in range(E)]
+    stack = (lambda xs: torch.stack([t.view(torch.uint8) for t in xs]).view(torch.float8_e4m3fn)) if kind == "fp8" else torch.stack
+    w13q, w13s = stack([t[0] for t in q13]), torch.stack([t[1] for t in q13])
+    w2q, w2s = stack([t[0] for t in q2]), torch.stack([t[1] for t in q2])
+    out = ep_moe_forward(x.to(dev), ids.to(dev), w.to(dev), w13q.to(dev), w2q.to(dev), w13s.to(dev), w2s.to(dev),
+                         block_shape=[128, 128])
+    ref = m.ep_moe_forward(x, ids, w, w13q, w13s, w2q, w2s, aq, dtype=dt)
+    assert out.shape == (T, H) and out.dtype == dt
+    assert_close_scaled(out, ref, rtol=3e-2, atol=3e-2, what="moe " + kind)
+    dense = m.dense_moe_forward(x, ids, w, w13, w2)
+    cos = torch.nn.functional.cosine_similarity(out.float().cpu().flatten(), dense.float().flatten(), dim=0)
+    assert cos > 0.99
+
+
+def test_router(dev):
+    logits = torch.randn(33, 8)
+    ids, w = softmax_topk_router(logits.to(dev), 2)
+    oids, ow = m.softmax_top2_router(logits, 2)
+    assert torch.equal(ids.cpu(), oids) and torch.allclose(w.cpu(), ow, atol=1e-6)

@@ -1,0 +1,97 @@
+"""HIP quantizers / dequantizers vs the torch-CPU oracle: bit-exact integers and scales."""
+import pytest
+import torch
+
+from oracle import quant_ref as q, bitpack_ref as bp
+from llm_kernels_amd.quantization import fp8_kernel, int8_kernel, w4a8_kernel
+from helpers import announce, default_dtype
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 128), (16, 4096), (3, 5, 256), (257, 14336)])
+def test_act_quant_int8_both_roundings(dev, dtype, shape):
+    announce("act_quant_i8", dtype, shape)
+    torch.manual_seed(0)
+    x = torch.randn(*shape).to(dtype)
+    x.view(-1)[:8] = torch.tensor([0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 127.0, -127.0]).to(dtype)  # ties in group 0
+    xg = x.to(dev)
+    for mod, mode in ((int8_kernel, "away"), (w4a8_kernel, "up")):
+        y, s = mod.act_quant(xg)
+        oy, os_ = q.act_quant_int8(x, 128, mode)
+        assert y.dtype == torch.int8 and s.dtype == torch.float16 and s.shape == os_.shape
+        assert torch.equal(s.cpu(), os_), mode
+        assert torch.equal(y.cpu(), oy), mode
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 128), (16, 4096), (2, 3, 384), (300, 4096)])
+def test_act_quant_fp8(dev, dtype, shape):
+    announce("act_quant_fp8", dtype, shape)
+    torch.manual_seed(1)
+    x = torch.randn(*shape).to(dtype)
+    y, s = fp8_kernel.act_quant(x.to(dev))
+    oy, os_ = q.act_quant_fp8(x)
+    assert y.dtype == torch.float8_e4m3fn and s.dtype == torch.float32
+    assert torch.equal(s.cpu(), os_)
+    assert torch.equal(y.cpu().view(torch.uint8), oy.view(torch.uint8))
+
+
+def test_act_quant_fp8_zero_group_nan_and_asserts(dev):
+    announce("act_quant_fp8 zero group")
+    x = torch.randn(2, 256)
+    x[1, 128:] = 0
+    y, s = fp8_kernel.act_quant(x.to(dev))
+    assert s[1, 1].item() == 0.0 and y[1, 128:].float().isnan().all() and not y[0].float().isnan().any()
+    with pytest.raises(AssertionError):
+        fp8_kernel.act_quant(torch.randn(4, 100, device=dev))
+    with pytest.raises(AssertionError):
+        int8_kernel.act_quant(torch.randn(4, 256, device=dev).t())
+
+
+@pytest.mark.parametrize("shape", [(128, 128), (512, 1024), (200, 300), (4096, 4096)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_weight_quant_int8_and_dequant(dev, shape, dtype):
+    announce("weight_quant_i8", shape, dtype)
+    torch.manual_seed(2)
+    w = (torch.randn(*shape) * 0.02).to(dtype)
+    y, s = int8_kernel.weight_quant(w.to(dev))
+    oy, os_ = q.weight_quant_int8(w)
+    assert torch.equal(s.cpu(), os_) and torch.equal(y.cpu(), oy)
+    for dd in (torch.float16, torch.bfloat16, torch.float32):
+        with default_dtype(dd):
+            d = int8_kernel.weight_dequant(y, s)
+        assert d.dtype == dd
+        assert torch.equal(d.cpu(), q.weight_dequant_block(oy, os_, 128, dd))
+
+
+@pytest.mark.parametrize("shape", [(128, 256), (300, 200), (4096, 4096)])
+def test_weight_quant_fp8_and_dequant(dev, shape):
+    announce("weight_quant_fp8", shape)
+    torch.manual_seed(3)
+    w = torch.randn(*shape) * 0.02
+    y, s = fp8_kernel.weight_quant(w.to(dev))
+    oy, os_ = q.weight_quant_fp8(w)
+    assert torch.equal(s.cpu(), os_)
+    assert torch.equal(y.cpu().view(torch.uint8), oy.view(torch.uint8))
+    with default_dtype(torch.bfloat16):
+        d = fp8_kernel.weight_dequant(y, s)
+    assert torch.equal(d.cpu(), q.weight_dequant_block(oy, os_, 128, torch.bfloat16))
+
+
+@pytest.mark.parametrize("shape", [(128, 128), (1024, 7168), (4096, 4096)])
+def test_w4a8_weight_quant_dequant(dev, shape):
+    announce("w4a8 weight_quant", shape)
+    torch.manual_seed(4)
+    w = (torch.randn(*shape) * 0.02).half()
+    yp, s, s4, z4 = w4a8_kernel.weight_quant(w.to(dev))
+    oq, os_, os4, oz4 = q.w4a8_weight_quant_levels(w)
+    assert yp.dtype == torch.int32 and yp.shape == (shape[0] // 8, shape[1])
+    assert torch.equal(s.cpu(), os_) and torch.equal(s4.cpu(), os4) and torch.equal(z4.cpu(), oz4)
+    opacked, _ = bp.pack_rows(oq.numpy(), 4, 32)
+    assert torch.equal(yp.cpu(), torch.from_numpy(opacked))
+    d = w4a8_kernel.weight_dequant(yp, s, s4, z4)
+    assert d.dtype == torch.float16 and torch.equal(d.cpu(), q.w4a8_weight_dequant(oq, os_, os4, oz4))
+    cos = torch.nn.functional.cosine_similarity(d.float().flatten().cpu(), w.float().flatten(), dim=0)
+    assert cos > 0.98

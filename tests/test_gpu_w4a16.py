@@ -1,0 +1,115 @@
+"""W4A16 GEMMs (simple-Marlin layout `mul`, and the [N, K/8] bit-packed layout) vs the oracle."""
+import pytest
+import torch
+
+from oracle import gemm_ref as g, marlin_ref as mr, quant_ref as q, bitpack_ref as bp
+from llm_kernels_amd.fast_dequant.simple_marlin.utils import QuantUtils
+from llm_kernels_amd.fast_dequant.simple_marlin.marlin import mul
+from llm_kernels_amd.fast_dequant import w4a16
+from helpers import announce, assert_close_scaled
+
+pytestmark = pytest.mark.gpu
+
+# the 14 shapes of the reference's own accuracy test (fast_dequant/simple_marlin/test.py:139-157)
+REFERENCE_CASES = [
+    (16, 64, 128, 128), (16, 128, 128, 128), (16, 64, 512, 128), (16, 64, 1024, 128),
+    (256, 512, 1024, 128), (512, 256, 1024, 128), (1024, 1024, 512, 128), (128, 2048, 1024, 128),
+    (1024, 2048, 2048, 128), (2048, 1024, 1024, 128), (512, 4096, 2048, 128),
+    (256, 512, 1024, 64), (256, 512, 1024, 256), (512, 512, 512, 512),
+]
+
+
+@pytest.mark.parametrize("M,N,K,groupsize", REFERENCE_CASES)
+def test_mul_reference_recipe(dev, M, N, K, groupsize):
+    """Recipe of the reference test: seed 42, inputs randn * 0.1, pass = every |diff| <= 0.05."""
+    announce("marlin mul", M, N, K, groupsize)
+    torch.manual_seed(42)
+    A = (torch.randn(M, K) * 0.1).half()
+    W = (torch.randn(K, N) * 0.1).half()
+    ref_deq, W_int4, scales = mr.fake_quantize(W, groupsize)
+    B, sp = mr.pack(W_int4, scales, groupsize)
+    C = torch.zeros(M, N, dtype=torch.half, device=dev)
+    workspace = torch.zeros(N // 128 * 16 + 16, dtype=torch.int32, device=dev)
+    ret = mul(A.to(dev), B.to(dev), C, sp.to(dev), workspace)
+    assert ret is None
+    ref = g.w4a16_gemm(A, W_int4, scales, groupsize)
+    assert (C.cpu().double() - ref).abs().max() <= 0.05            # the reference's acceptance threshold
+    assert_close_scaled(C, ref, what="marlin mul")
+    assert torch.allclose(ref, A.double() @ ref_deq.double())
+
+
+def test_mul_quantize_and_pack_on_device(dev):
+    announce("marlin device-side pack")
+    torch.manual_seed(1)
+    M, N, K, g_ = 16, 4096, 4096, 128
+    A = torch.randn(M, K, device=dev).half()
+    W = (torch.randn(K, N, device=dev) * 0.02).half()
+    ref_deq, W_int4, scales = QuantUtils.fake_quantize(W, g_)
+    B, sp = QuantUtils.pack(W_int4, scales, g_)
+    assert B.shape == (K // 16, 2 * N) and B.dtype == torch.int32 and B.device == W.device
+    oB, osp = mr.pack(W_int4.cpu(), scales.cpu(), g_)
+    assert torch.equal(B.cpu(), oB) and torch.equal(sp.cpu(), osp)
+    C = torch.zeros(M, N, dtype=torch.half, device=dev)
+    mul(A, B, C, sp, torch.zeros(512, dtype=torch.int32, device=dev))
+    assert_close_scaled(C, A.double().cpu() @ ref_deq.double().cpu(), what="marlin 16x4096x4096")
+
+
+@pytest.mark.parametrize("M,N,K,groupsize", [(16, 64, 16, 16), (16, 192, 48, 16), (32, 64, 256, 32), (48, 320, 128, -1)])
+def test_mul_edge_shapes(dev, M, N, K, groupsize):
+    announce("marlin edge", M, N, K, groupsize)
+    torch.manual_seed(M + N + K)
+    A = (torch.randn(M, K) * 0.5).half()
+    W = (torch.randn(K, N) * 0.1).half()
+    _, W_int4, scales = mr.fake_quantize(W, groupsize)
+    # the kernel reads scales in the grouped permutation; pack with an explicit group size of K for -1
+    B, sp = mr.pack(W_int4, scales, K if groupsize == -1 else groupsize)
+    C = torch.full((M, N), 7.0, dtype=torch.half, device=dev)
+    mul(A.to(dev), B.to(dev), C, sp.to(dev), torch.zeros(64, dtype=torch.int32, device=dev))
+    assert_close_scaled(C, g.w4a16_gemm(A, W_int4, scales, groupsize), what="marlin edge")
+
+
+def test_mul_error_behaviour(dev):
+    announce("marlin errors")
+    A = torch.zeros(16, 64, dtype=torch.half, device=dev)
+    B = torch.zeros(4, 128, dtype=torch.int32, device=dev)
+    C = torch.zeros(16, 64, dtype=torch.half, device=dev)
+    s = torch.ones(1, 64, dtype=torch.half, device=dev)
+    ws = torch.zeros(16, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError):
+        mul(A[:15], B, C[:15], s, ws)                       # M % 16
+    with pytest.raises(RuntimeError):
+        mul(A.float(), B, C, s, ws)                         # dtype
+    with pytest.raises(RuntimeError):
+        mul(A, B.long(), C, s, ws)
+    with pytest.raises(RuntimeError):
+        mul(A, B, C, s[:, :32].contiguous(), ws)            # scale N mismatch
+    with pytest.raises(RuntimeError):
+        mul(A, B, C.cpu(), s, ws)                           # device mismatch
+
+
+# ----------------------------------------------------------------------------- [N, K/8] layout (config 1)
+@pytest.mark.parametrize("M,N,K,gs", [(16, 4096, 4096, 128), (1, 64, 128, 128), (7, 100, 256, 64), (16, 256, 512, 32),
+                                      (40, 512, 1024, 128), (16, 128, 384, -1)])
+def test_w4a16_nk(dev, M, N, K, gs):
+    announce("w4a16 nk", M, N, K, gs)
+    torch.manual_seed(0)
+    x = torch.randn(M, K).half()
+    w = torch.randn(N, K) * 0.02
+    grp = K if gs == -1 else gs
+    qn, s = q.w4a16_quant_nk(w, grp)
+    packed, _ = bp.pack_cols(qn.numpy(), 4, 32)
+    y = w4a16.w4a16_gemm(x.to(dev), torch.from_numpy(packed).to(dev), s.to(dev), gs)
+    assert y.dtype == torch.half and y.shape == (M, N)
+    ref = g.w4a16_gemm(x, qn.t().int().contiguous(), s.t().contiguous(), grp)
+    assert_close_scaled(y, ref, what="w4a16 nk")
+
+
+def test_w4a16_nk_device_quantize_round_trip(dev):
+    announce("w4a16 nk quantize on device")
+    torch.manual_seed(3)
+    from llm_kernels_amd.quantization.bitpack import unpack_over_cols
+    w = torch.randn(4096, 4096, device=dev) * 0.02
+    packed, s, qd = w4a16.quantize_nk(w, 128)
+    oq, os_ = q.w4a16_quant_nk(w.cpu(), 128)
+    assert packed.shape == (4096, 512) and torch.equal(qd.cpu(), oq) and torch.equal(s.cpu(), os_)
+    assert torch.equal(unpack_over_cols(packed, 4, 4096), qd)       # pack/unpack round trip, bit exact
