@@ -15,7 +15,8 @@ def quantize_nk(w: torch.Tensor, group_size: int = 128):
     assert w.dim() == 2 and w.shape[1] % group_size == 0
     N, K = w.shape
     g = w.float().reshape(N, K // group_size, group_size)
-    s = (g.abs().amax(dim=2) / 7.0).to(torch.float16)
+    amax = g.abs().amax(dim=2)
+    s = (amax / torch.full_like(amax, 7.0)).to(torch.float16)     # tensor divisor: a true IEEE division on every device
     q = (torch.clamp(torch.round(g / s.float().unsqueeze(-1)), -8, 7) + 8).reshape(N, K).to(torch.uint8)
     packed, _ = pack_weights_over_cols(q, 4, 32, transpose=False)
     return packed, s, q

@@ -66,7 +66,8 @@ def int8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Te
 def _rowwise_quant(x: torch.Tensor):
     # one group per row: the 1 x block kernel needs a power-of-two block, so rows go through torch here
     xf = x.float()
-    s = xf.abs().amax(dim=-1) / 127.0
+    amax = xf.abs().amax(dim=-1)
+    s = amax / torch.full_like(amax, 127.0)                       # tensor divisor: a true IEEE division on every device
     v = xf / s.unsqueeze(-1)
     t = torch.trunc(v)
     y = (t + torch.sign(v) * ((v - t).abs() >= 0.5)).to(torch.int8)
