@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Throughput of the quantized-GEMM path on one MI355X, against its roofline, with a CPU baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all] [--no-cpu]
+
+A "step" is one GEMM call over one batch of synthetic input already resident in HBM.  Small-M
+(HBM-bound) workloads rotate through enough distinct weight copies to exceed the 256 MB on-die cache,
+so the figure is an HBM figure and not a cache figure.  Rank 0 prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# published MI355X peaks (dense)
+PEAK_HBM_GBS = 8000.0
+PEAK_TFLOPS = {"fp8": 5000.0, "int8": 5000.0, "fp16": 2500.0, "bf16": 2500.0}
+CACHE_DEFEAT_BYTES = 512 << 20
+
+
+def _bytes_fp8(M, N, K):
+    kb, nb = K // 128, (N + 127) // 128
+    return M * K + N * K + 4 * M * kb + 4 * nb * kb + 2 * M * N
+
+
+def _bytes_i8(M, N, K):
+    kb, nb = K // 128, (N + 127) // 128
+    return M * K + N * K + 2 * M * kb + 2 * nb * kb + 2 * M * N
+
+
+def _bytes_w4a16(M, N, K, g=128):
+    return 2 * M * K + N * K // 2 + 2 * N * K // g + 2 * M * N
+
+
+def _bytes_w4a8(M, N, K):
+    kb, nb = K // 128, (N + 127) // 128
+    return M * K + N * K // 2 + 2 * M * kb + 2 * nb * kb + 2 * N * kb + 2 * M * N
+
+
+class Case:
+    """One GEMM workload: device buffers (rotated), a launcher, algorithmic cost and a CPU restatement."""
+
+    def __init__(self, name, op, M, N, K):
+        self.name, self.op, self.M, self.N, self.K = name, op, M, N, K
+        self.flops = 2.0 * M * N * K
+        self.bytes = {"fp8": _bytes_fp8, "int8": _bytes_i8, "w4a8": _bytes_w4a8}.get(op, None)
+        self.bytes = self.bytes(M, N, K) if self.bytes else _bytes_w4a16(M, N, K)
+        self.mfma_dtype = {"fp8": "fp8", "int8": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
+        intensity = self.flops / self.bytes
+        ridge = PEAK_TFLOPS[self.mfma_dtype] * 1e12 / (PEAK_HBM_GBS * 1e9)
+        self.bound = "hbm" if intensity < ridge else "mfma"
+        self.dtype = {"fp8": "fp8_e4m3", "int8": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
+
+    # ---- device side
+    def setup(self, dev):
+        from llm_kernels_amd.quantization import fp8_kernel, int8_kernel, w4a8_kernel
+        from llm_kernels_amd.fast_dequant.simple_marlin.utils import QuantUtils
+        from llm_kernels_amd.fast_dequant.simple_marlin.marlin import mul
+        from llm_kernels_amd.fast_dequant import w4a16
+        M, N, K, op = self.M, self.N, self.K, self.op
+        torch.manual_seed(0)
+        wbytes = {"fp8": N * K, "int8": N * K}.get(op, N * K // 2)
+        nbuf = 1 if self.bound == "mfma" else max(2, min(64, -(-CACHE_DEFEAT_BYTES // wbytes)))
+        self.nbuf = nbuf
+        x = torch.randn(M, K, device=dev)
+        w = torch.randn(N, K, device=dev) * 0.02
+        self.host = (x.cpu(), w.cpu())
+        if op == "fp8":
+            a, a_s = fp8_kernel.act_quant(x.bfloat16())
+            b, b_s = fp8_kernel.weight_quant(w)
+            bs = [b.clone() for _ in range(nbuf)]
+            self.launch = lambda i: fp8_kernel.fp8_gemm(a, a_s, bs[i % nbuf], b_s)
+        elif op == "int8":
+            a, a_s = int8_kernel.act_quant(x.bfloat16())
+            b, b_s = int8_kernel.weight_quant(w)
+            bs = [b.clone() for _ in range(nbuf)]
+            self.launch = lambda i: int8_kernel.int8_gemm(a, a_s, bs[i % nbuf], b_s)
+        elif op == "w4a8":
+            a, a_s = w4a8_kernel.act_quant(x.bfloat16())
+            b, b_s, s4, z4 = w4a8_kernel.weight_quant(w.half())
+            bs = [b.clone() for _ in range(nbuf)]
+            self.launch = lambda i: w4a8_kernel.w4a8_gemm(a, a_s, bs[i % nbuf], b_s, s4, z4)
+        elif op == "w4a16":
+            A = x.half()
+            _, q, s = QuantUtils.fake_quantize(w.t().contiguous().half(), 128)
+            B, sp = QuantUtils.pack(q, s, 128)
+            Bs = [B.clone() for _ in range(nbuf)]
+            C = torch.empty(M, N, dtype=torch.half, device=dev)
+            ws = torch.zeros(max(16, N // 128 * 16), dtype=torch.int32, device=dev)
+            self.launch = lambda i: mul(A, Bs[i % nbuf], C, sp, ws)
+        elif op == "w4a16_nk":
+            A = x.half()
+            packed, s, _ = w4a16.quantize_nk(w, 128)
+            Ps = [packed.clone() for _ in range(nbuf)]
+            self.launch = lambda i: w4a16.w4a16_gemm(A, Ps[i % nbuf], s, 128)
+        else:
+            raise ValueError(op)
+
+    # ---- host side: the repo's torch reference semantics (dequantize, then matmul in fp32) on CPU cores
+    def cpu_seconds(self, max_rows):
+        from oracle import quant_ref, marlin_ref, gemm_ref
+        x, w = self.host
+        rows = min(self.M, max_rows)
+        x = x[:rows]
+        op = self.op
+        if op == "fp8":
+            a, a_s = quant_ref.act_quant_fp8(x.bfloat16())
+            b, b_s = quant_ref.weight_quant_fp8(w)
+
+            def run():
+                ad = a.float() * a_s.repeat_interleave(128, 1)
+                bd = quant_ref.weight_dequant_block(b, b_s)
+                return ad @ bd.T
+        elif op in ("int8", "w4a8"):
+            a, a_s = quant_ref.act_quant_int8(x.bfloat16(), rounding="away" if op == "int8" else "up")
+            if op == "int8":
+                b, b_s = quant_ref.weight_quant_int8(w)
+                deq = lambda: quant_ref.weight_dequant_block(b, b_s)
+            else:
+                qq, s, s4, z4 = quant_ref.w4a8_weight_quant_levels(w)
+                deq = lambda: quant_ref.w4a8_weight_dequant(qq, s, s4, z4).float()
+
+            def run():
+                ad = a.float() * a_s.float().repeat_interleave(128, 1)
+                return ad @ deq().T
+        else:
+            wk = w.t().contiguous().half()
+            _, q, s = marlin_ref.fake_quantize(wk, 128)
+
+            def run():
+                return x.half().float() @ gemm_ref.w4a16_dequant_kn(q, s, 128).float()
+        run()
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        return dt, rows
+
+
+WORKLOADS = {}
+for _op in ("fp8", "int8", "w4a8", "w4a16", "w4a16_nk"):
+    for _M in (1, 16, 128, 256, 1024, 4096):
+        for _N, _K in ((4096, 4096), (6144, 4096), (14336, 4096), (28672, 4096), (4096, 14336)):
+            WORKLOADS["%s_m%d_n%d_k%d" % (_op, _M, _N, _K)] = (_op, _M, _N, _K)
+
+DEFAULT_WORKLOAD = "fp8_m4096_n4096_k4096"
+HEADLINE_SET = ["w4a16_m16_n4096_k4096", "fp8_m16_n4096_k4096", "fp8_m16_n28672_k4096", "fp8_m16_n4096_k14336",
+                "w4a16_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "w4a8_m16_n4096_k4096"]
+
+
+def run_case(case, dev, steps, warmup, eager=False):
+    """Returns (wall seconds, HIP-event milliseconds) for exactly `steps` steps.
+
+    The steps are captured once into a HIP graph and replayed, so that the timed region is bound by the
+    GPU and not by the Python launch path (decode-sized kernels last a few microseconds).  Events are
+    recorded on the stream the replay runs on.
+    """
+    case.setup(dev)
+    for i in range(warmup):
+        case.launch(i)
+    torch.cuda.synchronize()
+    graph = None
+    if not eager:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(steps):
+                case.launch(warmup + i)
+        graph.replay()                   # untimed replay (first replay uploads the graph)
+        torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(steps):
+            case.launch(warmup + i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1)
+
+
+def record(case, wall, ev_ms, steps):
+    dur = ev_ms / 1e3 / steps                       # average launch-to-launch duration from HIP events
+    tflops = case.flops / dur / 1e12
+    gbs = case.bytes / dur / 1e9
+    if case.bound == "hbm":
+        roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    else:
+        pk = PEAK_TFLOPS[case.mfma_dtype]
+        roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": pk, "unit": "TFLOP/s",
+                "frac": round(tflops / pk, 4), "traffic": None}
+    return {"workload": case.name, "M": case.M, "N": case.N, "K": case.K, "us_per_launch": round(dur * 1e6, 2),
+            "tflops": round(tflops, 2), "gbs": round(gbs, 1), "alg_bytes": case.bytes, "flops": case.flops,
+            "weight_copies_rotated": case.nbuf, "wall_ms_per_step": round(wall * 1e3 / steps, 4), "roofline": roof}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
+    ap.add_argument("--all", action="store_true", help="also measure the other headline shapes (reported under 'cases')")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="launch every step from Python instead of replaying a HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    from llm_kernels_amd import _lib
+    _lib.load()                                      # fails loudly if the HIP library is not built
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.set_default_dtype(torch.bfloat16)
+
+    op, M, N, K = WORKLOADS[args.workload]
+    case = Case(args.workload, op, M, N, K)
+    wall, ev_ms = run_case(case, dev, args.steps, args.warmup, args.eager)
+    rec = record(case, wall, ev_ms, args.steps)
+
+    cases = []
+    if args.all:
+        for name in HEADLINE_SET:
+            if name == args.workload:
+                continue
+            c = Case(name, *WORKLOADS[name])
+            w2, e2 = run_case(c, dev, args.steps, args.warmup, args.eager)
+            cases.append(record(c, w2, e2, args.steps))
+            del c
+            torch.cuda.empty_cache()
+
+    cpu = None
+    if not args.no_cpu:
+        cores = os.cpu_count() or 1
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+        torch.set_num_threads(cores)
+        max_rows = 512                                # bounded sample of the same workload
+        dt, rows = case.cpu_seconds(max_rows)
+        cpu_tflops = 2.0 * rows * N * K / dt / 1e12
+        cpu = {"value": round(cpu_tflops, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
+                         "1 warm-up + 1 timed pass, weight dequantisation included (%.2f s)" % (rows, M, dt)}
+
+    out = {
+        "metric": "w4a16/fp8 GEMM TFLOPS & % roofline (HBM at M=16, MFMA at M=4096)",
+        "value": rec["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": rec["wall_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": case.dtype, "data": "synthetic",
+        "config": {"workload": args.workload, "M": M, "N": N, "K": K, "weight_copies_rotated": case.nbuf,
+                   "us_per_launch_hip_events": rec["us_per_launch"], "alg_bytes": rec["alg_bytes"],
+                   "flops": rec["flops"], "launch": "eager" if args.eager else "hip_graph"},
+        "roofline": rec["roofline"], "cpu_baseline": cpu,
+    }
+    if cases:
+        out["cases"] = cases
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,5 +1,5 @@
 // Dense block-scaled fp8 / int8 GEMM entry points.
-#include "gemm_direct.hpp"
+#include "gemm_tiled.hpp"
 
 using namespace llmk;
 
@@ -33,6 +33,7 @@ extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* 
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+    if (M > 64) return launch_tiled<K_FP8_BLOCK, false>(p, (hipStream_t)stream, "gemm_fp8_block(tiled)");
     return launch_direct<K_FP8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_fp8_block");
 }
 
@@ -48,6 +49,7 @@ extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+    if (M > 64) return launch_tiled<K_I8_BLOCK, false>(p, (hipStream_t)stream, "gemm_i8_block(tiled)");
     return launch_direct<K_I8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_block");
 }
 

@@ -1,6 +1,6 @@
 // Single-GPU expert-parallel MoE path: segment bookkeeping, token permute / un-permute,
 // gated activation, and the grouped GEMM over one GPU's experts.
-#include "gemm_direct.hpp"
+#include "gemm_tiled.hpp"
 
 using namespace llmk;
 
@@ -179,6 +179,9 @@ extern "C" int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind
     p.seg_indptr = seg_indptr; p.weight_indices = weight_indices;
     p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = E;
     hipStream_t st = (hipStream_t)stream;
+    const bool big = M > 64 * (int64_t)E;            // average segment long enough for 256-row tiles
+    if (big && kind == LLMK_KIND_I8) return launch_tiled<K_I8_BLOCK, true>(p, st, "grouped_gemm(i8, tiled)");
+    if (big && kind == LLMK_KIND_FP8) return launch_tiled<K_FP8_BLOCK, true>(p, st, "grouped_gemm(fp8, tiled)");
     switch (kind) {
         case LLMK_KIND_I8:   return launch_direct<K_I8_BLOCK, true>(p, (int)M, st, "grouped_gemm(i8)");
         case LLMK_KIND_FP8:  return launch_direct<K_FP8_BLOCK, true>(p, (int)M, st, "grouped_gemm(fp8)");
