@@ -1,26 +1,28 @@
 // LDS-tiled MFMA GEMM for the compute-bound (large M) block-scaled fp8 / int8 products.
 //
-// Workgroup: 256 threads = 4 waves (2 along M x 2 along N), output tile 256 x 128, K step 128
+// Workgroup: 512 threads = 8 waves (4 along M x 2 along N), output tile 256 x 128, K step 128
 // (= one scale block, one v_mfma_f32_16x16x128_f8f6f4 or two v_mfma_i32_16x16x64_i8 per 16x16 tile).
-// Wave tile 128 x 64: 8 x 4 accumulator tiles (128 accumulator registers per lane).
+// Wave tile 64 x 64: 4 x 4 accumulator tiles (64 accumulator registers per lane), so that two waves
+// share each SIMD and one wave's scale FMAs / LDS waits hide under the other's MFMAs.
 // Global -> registers -> LDS with two LDS stages: the loads of K step kt+1 are in flight while
 // step kt is multiplied, one barrier per step.  LDS rows are padded from 128 to 144 bytes so that
 // the 16 rows a b128 read touches fall into different banks.
 // Per K step the partial product of every tile is scaled by a_s[row] * b_s[column block] and
-// added to the fp32 accumulator, which is exactly the reference's accumulation order.
+// added to the fp32 accumulator (the reference's accumulation order; the two scales are multiplied
+// first, once per row, by the thread that stages them).
 #pragma once
 #include "gemm_direct.hpp"
 
 namespace llmk {
 
-constexpr int T_BM = 256, T_BN = 128, T_ROW = 144;
+constexpr int T_BM = 256, T_BN = 128, T_ROW = 144, T_THREADS = 512;
 constexpr int T_A_BYTES = T_BM * T_ROW;            // 36864
 constexpr int T_B_BYTES = T_BN * T_ROW;            // 18432
-constexpr int T_STAGE = T_A_BYTES + T_B_BYTES + T_BM * 4;   // + a_s column for this K step
+constexpr int T_STAGE = T_A_BYTES + T_B_BYTES + T_BM * 4;   // + the scale column of this K step
 constexpr int T_LDS = 2 * T_STAGE;                 // 112640 bytes
 
 template <int KIND, bool GROUPED>
-__global__ __launch_bounds__(256, 1) void gemm_tiled_kernel(DirectArgs p) {
+__global__ __launch_bounds__(T_THREADS) void gemm_tiled_kernel(DirectArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, g = lane >> 4;
@@ -52,38 +54,38 @@ __global__ __launch_bounds__(256, 1) void gemm_tiled_kernel(DirectArgs p) {
         m_end = min(p.M, m_start + T_BM);
     }
 
-    // ---- global -> register staging map: 8 threads cover one 128-byte row, 32 rows per pass
+    // ---- global -> register staging map: 8 threads cover one 128-byte row, 64 rows per pass
     const int lrow = tid >> 3, lchunk = (tid & 7) * 16;
-    const uint8_t* ag[8];
-    const uint8_t* bg[4];
+    const uint8_t* ag[4];
+    const uint8_t* bg[2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) ag[i] = p.a + (int64_t)min(m_start + i * 32 + lrow, m_end - 1) * K + lchunk;
+    for (int i = 0; i < 4; ++i) ag[i] = p.a + (int64_t)min(m_start + i * 64 + lrow, m_end - 1) * K + lchunk;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) bg[i] = bbase + (int64_t)min(n0 + i * 32 + lrow, N - 1) * K + lchunk;
-    const int64_t as_row = (int64_t)min(m_start + tid, m_end - 1) * KT;
+    for (int i = 0; i < 2; ++i) bg[i] = bbase + (int64_t)min(n0 + i * 64 + lrow, N - 1) * K + lchunk;
+    const int64_t as_row = (int64_t)min(m_start + (tid & 255), m_end - 1) * KT;
     const int64_t bs_row = bs_off + (int64_t)blockIdx.x * KT;     // T_BN == 128: one weight-scale block per tile
 
-    v4i ra[8], rb[4];
-    float rsa, rbs;
+    v4i ra[4], rb[2];
+    float rsa = 0.f;
     auto gload = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ra[i] = *(const v4i*)(ag[i] + (int64_t)kt * 128);
+        for (int i = 0; i < 4; ++i) ra[i] = *(const v4i*)(ag[i] + (int64_t)kt * 128);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) rb[i] = *(const v4i*)(bg[i] + (int64_t)kt * 128);
-        rsa = ld_scale(p.a_s, as_row + kt, p.s_dtype);
+        for (int i = 0; i < 2; ++i) rb[i] = *(const v4i*)(bg[i] + (int64_t)kt * 128);
+        if (tid < T_BM) rsa = ld_scale(p.a_s, as_row + kt, p.s_dtype) * ld_scale(p.b_s, bs_row + kt, p.s_dtype);
     };
     auto lstore = [&](int buf) {
         uint8_t* base = lds + buf * T_STAGE;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) *(v4i*)(base + (i * 32 + lrow) * T_ROW + lchunk) = ra[i];
+        for (int i = 0; i < 4; ++i) *(v4i*)(base + (i * 64 + lrow) * T_ROW + lchunk) = ra[i];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *(v4i*)(base + T_A_BYTES + (i * 32 + lrow) * T_ROW + lchunk) = rb[i];
-        ((float*)(base + T_A_BYTES + T_B_BYTES))[tid] = rsa;
+        for (int i = 0; i < 2; ++i) *(v4i*)(base + T_A_BYTES + (i * 64 + lrow) * T_ROW + lchunk) = rb[i];
+        if (tid < T_BM) ((float*)(base + T_A_BYTES + T_B_BYTES))[tid] = rsa;
     };
 
-    v4f acc[8][4];
+    v4f acc[4][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
@@ -97,19 +99,17 @@ __global__ __launch_bounds__(256, 1) void gemm_tiled_kernel(DirectArgs p) {
         const int buf = kt & 1;
         const bool more = kt + 1 < KT;
         if (more) gload(kt + 1);
-        rbs = ld_scale(p.b_s, bs_row + kt, p.s_dtype);
 
-        const uint8_t* As = lds + buf * T_STAGE + (wm * 128 + r) * T_ROW + 32 * g;
+        const uint8_t* As = lds + buf * T_STAGE + (wm * 64 + r) * T_ROW + 32 * g;
         const uint8_t* Bs = lds + buf * T_STAGE + T_A_BYTES + (wn * 64 + r) * T_ROW + 32 * g;
-        const float* Ss = (const float*)(lds + buf * T_STAGE + T_A_BYTES + T_B_BYTES) + wm * 128 + 4 * g;
+        const float* Ss = (const float*)(lds + buf * T_STAGE + T_A_BYTES + T_B_BYTES) + wm * 64 + 4 * g;
         v8i bf[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) bf[j] = ld32(Bs + j * 16 * T_ROW);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const v8i af = ld32(As + i * 16 * T_ROW);
-            v4f sa = *(const v4f*)(Ss + i * 16);
-            sa *= rbs;
+            const v4f sa = *(const v4f*)(Ss + i * 16);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const v4f t = step_dot<KIND>(af, bf[j]);
@@ -122,13 +122,13 @@ __global__ __launch_bounds__(256, 1) void gemm_tiled_kernel(DirectArgs p) {
 
     // ---- epilogue: lane holds rows 4g..4g+3 of column r in every 16x16 tile
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + wn * 64 + j * 16 + r;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int m = m_start + wm * 128 + i * 16 + 4 * g + q;
+                const int m = m_start + wm * 64 + i * 16 + 4 * g + q;
                 if (m < m_end && n < N) st_out(p.c, (int64_t)m * N + n, acc[i][j][q], p.c_dtype);
             }
         }
@@ -146,7 +146,7 @@ int launch_tiled(const DirectArgs& p, hipStream_t stream, const char* name) {
     const int tiles_m = (p.M + T_BM - 1) / T_BM + (GROUPED ? p.E : 0);
     dim3 grid((unsigned)((p.N + T_BN - 1) / T_BN), (unsigned)tiles_m);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
-    kern<<<grid, 256, T_LDS, stream>>>(p);
+    kern<<<grid, T_THREADS, T_LDS, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     return LLMK_OK;
 }
