@@ -39,7 +39,8 @@ extern "C" {
 
 int         llmk_version(void);
 const char* llmk_last_error(void);
-/* Number of bytes of split-K scratch llmk_gemm_* may use for (M,N); 0 means none needed. */
+/* Bytes of scratch llmk_gemm_fp8_block / _i8_block / _w4a8 / llmk_grouped_gemm can use for this shape
+ * (0 = none).  The scratch is optional: without it a slower kernel variant runs. */
 int64_t     llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* ------------------------------------------------------------------ bit packing
@@ -161,11 +162,12 @@ int llmk_moe_post_reorder(const void* down_out, void* out, int dtype, const int3
                           void* stream);
 /* C[seg[e]:seg[e+1], :] = A[seg[e]:seg[e+1], :] x B[weight_indices[e]]^T  for e < E.
  * a [M,K], b [E,N,K], c [M,N]; scale_a [M,K/128], scale_b [E,ceil(N/128),K/128] for the
- * block-scaled kinds (s_dtype = dtype code of both), NULL otherwise. */
+ * block-scaled kinds (s_dtype = dtype code of both), NULL otherwise.  workspace: optional scratch of
+ * llmk_gemm_workspace_bytes(M, N, K) bytes. */
 int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind, int c_dtype, int E,
                       int64_t M, int64_t N, int64_t K, const int64_t* seg_indptr,
                       const int64_t* weight_indices, const void* scale_a, const void* scale_b,
-                      int s_dtype, void* stream);
+                      int s_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -9,7 +9,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libllmk_gfx950.so")
+LIB_PATH = os.environ.get("LLMK_LIB", os.path.join(_HERE, "libllmk_gfx950.so"))
 
 F32, F16, BF16 = 0, 1, 2
 ROUND_HALF_AWAY, ROUND_HALF_UP = 0, 1
@@ -49,7 +49,7 @@ SIGNATURES = {
     "llmk_moe_pre_reorder": [_p, _i, _p, _i, _p, _p, _i, _p, _i, _i, _i, _l, _l, _p],
     "llmk_moe_act_and_mul": [_p, _i, _p, _i, _p, _i, _p, _i, _i, _l, _l, _i, _p],
     "llmk_moe_post_reorder": [_p, _p, _i, _p, _p, _i, _p, _i, _i, _i, _i, _l, _l, _p],
-    "llmk_grouped_gemm": [_p, _p, _p, _i, _i, _i, _l, _l, _l, _p, _p, _p, _p, _i, _p],
+    "llmk_grouped_gemm": [_p, _p, _p, _i, _i, _i, _l, _l, _l, _p, _p, _p, _p, _i, _p, _l, _p],
 }
 _RESTYPE = {"llmk_last_error": _c.c_char_p, "llmk_gemm_workspace_bytes": _l,
             "llmk_gemm_w4a16_marlin_workspace_bytes": _l}
@@ -109,6 +109,15 @@ def call(name, *args, exc=LlmkError):
         msg = lib.llmk_last_error()
         raise exc("%s failed (rc=%d): %s" % (name, rc, msg.decode() if msg else ""))
     return rc
+
+
+def gemm_workspace(device, M, N, K):
+    """(pointer, nbytes) of the optional GEMM scratch for this shape, (None, 0) when none is needed."""
+    n = load().llmk_gemm_workspace_bytes(M, N, K)
+    if n <= 0:
+        return None, 0
+    buf = workspace(device, n)
+    return ptr(buf), buf.numel()
 
 
 _ws = {}

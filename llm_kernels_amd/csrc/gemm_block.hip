@@ -1,5 +1,5 @@
 // Dense block-scaled fp8 / int8 GEMM entry points.
-#include "gemm_tiled.hpp"
+#include "gemm_dma.hpp"
 
 using namespace llmk;
 
@@ -18,14 +18,14 @@ int check_common(const char* name, const void* a, const void* b, int64_t M, int6
 }  // namespace
 
 extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    (void)M; (void)N; (void)K;
-    return 0;
+    (void)N;
+    // large-M kernels stream fp32 activation scales; 16-bit scales are widened into the workspace first
+    return (M > 64 && K > 0) ? M * (K / 128) * 4 : 0;
 }
 
 extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
                                    int c_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                    int64_t workspace_bytes, void* stream) {
-    (void)workspace; (void)workspace_bytes;
     int rc = check_common("gemm_fp8_block", a, b, M, N, K, c_dtype);
     if (rc) return rc;
     if (M == 0 || N == 0) return LLMK_OK;
@@ -33,14 +33,13 @@ extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* 
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
-    if (M > 64) return launch_tiled<K_FP8_BLOCK, false>(p, (hipStream_t)stream, "gemm_fp8_block(tiled)");
+    if (M > 64) return launch_big<K_FP8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_fp8_block(tiled)");
     return launch_direct<K_FP8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_fp8_block");
 }
 
 extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const void* b_s, int s_dtype,
                                   void* c, int c_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                   int64_t workspace_bytes, void* stream) {
-    (void)workspace; (void)workspace_bytes;
     int rc = check_common("gemm_i8_block", a, b, M, N, K, c_dtype);
     if (rc) return rc;
     if (s_dtype != LLMK_F32 && s_dtype != LLMK_F16 && s_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_i8_block: s_dtype %d", s_dtype);
@@ -49,7 +48,7 @@ extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
-    if (M > 64) return launch_tiled<K_I8_BLOCK, false>(p, (hipStream_t)stream, "gemm_i8_block(tiled)");
+    if (M > 64) return launch_big<K_I8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_i8_block(tiled)");
     return launch_direct<K_I8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_block");
 }
 

@@ -1,0 +1,349 @@
+// Large-M block-scaled fp8 / int8 GEMM with a three-stage global->LDS pipeline fed by the
+// direct-to-LDS loads of gfx950 (global_load_lds_dwordx4: no staging registers, no ds_write).
+//
+// Workgroup: 512 threads = 8 waves (4 along M x 2 along N), output tile 256 x 128, K step 128
+// (one scale block).  Wave tile 64 x 64 = 4 x 4 MFMA tiles, two waves per SIMD.
+//
+// LDS stage (50176 B): A 256 rows x 128 B, B 128 rows x 128 B, and the fp32 activation-scale column
+// of this K step.  A direct-to-LDS load writes lane l's 16 bytes at base + 16 l, so rows cannot be
+// padded; instead the 16-byte chunk index is XOR-swizzled with ((row >> 1) & 7) on the global side:
+// LDS slot s of row R holds global chunk s ^ ((R >> 1) & 7).  Two 128-byte rows span the 64 banks, so
+// the b128 fragment reads of 16 consecutive lanes (16 rows, same chunk) land in 16 different
+// 16-byte bank groups.
+//
+// Pipeline: stages kt+1 and kt+2 are in flight while stage kt is multiplied; the memory counter is
+// waited on by hand (the loads are issued from inline asm, so the compiler does not drain them
+// before every LDS read).  Each thread issues 7 loads per stage, hence vmcnt(7).
+// The loop contains no other vector-memory instruction: weight scales are copied to LDS up front.
+#pragma once
+#include "gemm_tiled.hpp"
+
+namespace llmk {
+
+constexpr int D_BM = 256, D_BN = 128, D_THREADS = 512, D_NSTAGE = 3;
+constexpr int D_A = D_BM * 128, D_B = D_BN * 128, D_S = D_BM * 4;
+constexpr int D_STAGE = D_A + D_B + D_S;                 // 50176
+constexpr int D_MAX_KT = 256;                            // weight-scale table entries (K <= 32768)
+constexpr int D_LDS = D_NSTAGE * D_STAGE + D_MAX_KT * 4; // 151552 bytes of the 160 KB
+
+__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+__device__ __forceinline__ void dma4(uint32_t lds_addr, uint32_t voff, const void* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+// s_waitcnt immediates for gfx9: vmcnt = imm[3:0] | imm[15:14] << 4, expcnt = imm[6:4] (7 = no wait),
+// lgkmcnt = imm[11:8] (15 = no wait)
+#define LLMK_WAIT_VMCNT_7 0x0F77
+#define LLMK_WAIT_VMCNT_0 0x0F70
+
+
+// 16 consecutive outputs of one row -> memory (vector stores when the row segment is 16-byte aligned)
+template <int ODT>
+__device__ __forceinline__ void store_row16(void* c, int64_t off, const v4f (&v)[4], int n_valid, bool vec_ok) {
+    if (vec_ok && n_valid >= 16) {
+        if constexpr (ODT == LLMK_F32) {
+            v4f* dst = (v4f*)((float*)c + off);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dst[j] = v[j];
+        } else {
+            v4i lo, hi;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                unsigned short h[8];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    h[q] = ODT == LLMK_F16 ? f32_to_f16(v[2 * j][q]) : f32_to_bf16(v[2 * j][q]);
+                    h[4 + q] = ODT == LLMK_F16 ? f32_to_f16(v[2 * j + 1][q]) : f32_to_bf16(v[2 * j + 1][q]);
+                }
+                v4i w = {(int)(h[0] | ((unsigned)h[1] << 16)), (int)(h[2] | ((unsigned)h[3] << 16)),
+                         (int)(h[4] | ((unsigned)h[5] << 16)), (int)(h[6] | ((unsigned)h[7] << 16))};
+                if (j == 0) lo = w; else hi = w;
+            }
+            v4i* dst = (v4i*)((unsigned short*)c + off);
+            dst[0] = lo;
+            dst[1] = hi;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (4 * j + q < n_valid) FloatIO<ODT>::st(c, off + 4 * j + q, v[j][q]);
+    }
+}
+
+template <int KIND, bool GROUPED>
+__global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int K = p.K, N = p.N;
+    const int KT = K >> 7;
+    const int n0 = blockIdx.x * D_BN;
+
+    int m_start, m_end;
+    const uint8_t* bbase = p.b;
+    int64_t bs_off = 0;
+    if constexpr (GROUPED) {
+        int tile = blockIdx.y, e = 0, cum = 0;
+        int64_t s0 = p.seg_indptr[0];
+        bool found = false;
+        for (; e < p.E; ++e) {
+            const int64_t s1 = p.seg_indptr[e + 1];
+            const int t = (int)((s1 - s0 + D_BM - 1) / D_BM);
+            if (tile < cum + t) { found = true; m_start = (int)s0 + (tile - cum) * D_BM; m_end = min((int)s1, m_start + D_BM); break; }
+            cum += t;
+            s0 = s1;
+        }
+        if (!found) return;
+        const int64_t widx = p.weight_indices ? p.weight_indices[e] : e;
+        bbase += widx * (int64_t)N * K;
+        bs_off = widx * (int64_t)((N + 127) / 128) * KT;
+    } else {
+        m_start = blockIdx.y * D_BM;
+        m_end = min(p.M, m_start + D_BM);
+    }
+
+    float* bsl = (float*)(lds + D_NSTAGE * D_STAGE);
+    const int64_t bs_row = bs_off + (int64_t)blockIdx.x * KT;
+
+    // ---- per-thread source offsets (bytes, 32 bit) of the 7 loads of a stage.
+    // Load i of a wave fills LDS rows 8q .. 8q+7 with q = wave*4+i (A) or wave*2+i (B), q & 1 == i & 1.
+    // A: LDS row R holds tile row R.  B: within each 64-row half, LDS row rho holds tile column
+    // 16*((rho & 15) >> 2) + 4*(rho >> 4) + (rho & 3): MFMA j then produces, in lane group g, the four
+    // columns 16g + 4j + (0..3), so that a lane ends up with 16 consecutive columns of one output row.
+    const int row8 = lane >> 3;
+    uint32_t aoff[4], boff[2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ (((i & 1) * 4 + (row8 >> 1)) & 7)) * 16u;
+        aoff[i] = (uint32_t)min(m_start + 8 * (wave * 4 + i) + row8, m_end - 1) * (uint32_t)K + chunk;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ (((i & 1) * 4 + (row8 >> 1)) & 7)) * 16u;
+        const int R = 8 * (wave * 2 + i) + row8, rho = R & 63;
+        const int col = (R & 64) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
+        boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
+    }
+    const uint32_t soff = (uint32_t)min(m_start + (wave & 3) * 64 + lane, m_end - 1) * (uint32_t)KT * 4u;
+
+    auto issue = [&](int kt) {
+        const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
+        const uint8_t* ga = p.a + (int64_t)kt * 128;
+        const uint8_t* gb = bbase + (int64_t)kt * 128;
+        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(st + (uint32_t)(wave * 4 + i) * 1024u, aoff[i], ga);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) dma16(st + D_A + (uint32_t)(wave * 2 + i) * 1024u, boff[i], gb);
+        dma4(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+    };
+
+    // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 64 x 64 tile
+    v4f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    if (KT > 0) issue(0);
+    if (KT > 1) issue(1);
+    // weight scales of this tile for every K step -> LDS.  These are the only compiler-tracked vector
+    // loads; they sit behind the first two stages in the memory queue, so waiting for them also waits
+    // for stage 0 and 1 (an acceptable one-off: the pipeline is being filled anyway).
+    for (int i = tid; i < KT; i += D_THREADS) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
+    __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
+    __syncthreads();
+
+    // fragment read offsets inside a 16-row slab: chunks 2g and 2g+1 of row r, swizzled
+    const int lo = r * 128 + (((2 * g) ^ ((r >> 1) & 7)) * 16);
+    const int hi = r * 128 + (((2 * g + 1) ^ ((r >> 1) & 7)) * 16);
+    auto ldfrag = [&](const uint8_t* base) {
+        const v4i x = *(const v4i*)(base + lo), y = *(const v4i*)(base + hi);
+        return (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+    };
+
+    // Software pipeline inside the wave: the 16 partial products of a K step live in two register sets,
+    // X (tile rows 0,1) and Y (tile rows 2,3).  While the MFMAs of one set run, the scale-and-accumulate
+    // FMAs of the other set (finished half a step earlier) issue on the VALU: one MFMA (32 cycles) covers
+    // the four FMAs (16 cycles) of one tile.
+    v4f tx[2][4], ty[2][4];
+    float sy[2] = {0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tx[i][j] = ty[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // fragments of the K step being multiplied (zero before the first load: multiplying them is a no-op)
+    v8i bf[4], af[4];
+    float sa[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bf[i] = af[i] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+        sa[i] = 0.f;
+    }
+    auto load_frags = [&](int kt) {
+        const uint8_t* st = lds + (kt % D_NSTAGE) * D_STAGE;
+        const uint8_t* As = st + (wm * 64) * 128;
+        const uint8_t* Bs = st + D_A + (wn * 64) * 128;
+        const float* Ss = (const float*)(st + D_A + D_B) + wm * 64 + r;
+        const float bs = bsl[kt];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bf[j] = ldfrag(Bs + j * 2048);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[i] = ldfrag(As + i * 2048);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sa[i] = Ss[i * 16] * bs;
+    };
+    // The weight fragment is the MFMA row operand and the activation fragment the column operand, i.e.
+    // the tile is produced transposed: a lane owns output row r and four consecutive columns per MFMA.
+    // Branch-free so that the whole body is a single scheduling region.
+    auto compute = [&]() {
+        // phase 1: X <- rows 0,1 of this step; retire Y of the previous step into acc rows 2,3
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[2 + i][j] += ty[i][j] * sy[i];
+                tx[i][j] = step_dot<KIND>(bf[j], af[i]);
+                __builtin_amdgcn_sched_group_barrier(0x008, KIND == K_FP8_BLOCK ? 1 : 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, KIND == K_FP8_BLOCK ? 4 : 8, 0);
+            }
+        // phase 2: Y <- rows 2,3 of this step; retire X into acc rows 0,1
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                ty[i][j] = step_dot<KIND>(bf[j], af[2 + i]);
+                acc[i][j] += tx[i][j] * sa[i];
+                __builtin_amdgcn_sched_group_barrier(0x008, KIND == K_FP8_BLOCK ? 1 : 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, KIND == K_FP8_BLOCK ? 4 : 8, 0);
+            }
+        sy[0] = sa[2];
+        sy[1] = sa[3];
+    };
+
+    // Ping-pong between the two wave groups that share every SIMD (waves 0-3 and 4-7): group 0 reads the
+    // fragments of step kt and multiplies them in the same iteration, group 1 multiplies the fragments it
+    // read one iteration earlier and then reads step kt.  While one wave of a SIMD waits for LDS, the other
+    // one keeps the matrix pipe busy.  Both groups hit the same barriers.
+    // Steady state: stage kt+2 is issued, stage kt consumed, stage kt+1 awaited.
+    int kt = 0;
+    if (wave < 4) {
+        for (; kt + 2 < KT; ++kt) {
+            issue(kt + 2);
+            load_frags(kt);
+            compute();
+            __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_7);
+            __syncthreads();
+        }
+        if (kt + 1 < KT) {
+            load_frags(kt);
+            compute();
+            __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
+            __syncthreads();
+            ++kt;
+        }
+        if (kt < KT) {
+            load_frags(kt);
+            compute();
+        }
+    } else {
+        for (; kt + 2 < KT; ++kt) {
+            issue(kt + 2);
+            compute();
+            __builtin_amdgcn_sched_barrier(0);
+            load_frags(kt);
+            __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_7);
+            __syncthreads();
+        }
+        if (kt + 1 < KT) {
+            compute();
+            __builtin_amdgcn_sched_barrier(0);
+            load_frags(kt);
+            __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
+            __syncthreads();
+            ++kt;
+        }
+        if (kt < KT) {
+            compute();
+            __builtin_amdgcn_sched_barrier(0);
+            load_frags(kt);
+        }
+        compute();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[2 + i][j] += ty[i][j] * sy[i];
+
+    // ---- epilogue: every lane writes 16 consecutive outputs of each of its four rows
+    const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
+    const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
+    const int nb = n0 + wn * 64 + 16 * g;
+    const int n_valid = N - nb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m_start + wm * 64 + 16 * i + r;
+        if (m >= m_end || n_valid <= 0) continue;
+        const int64_t off = (int64_t)m * N + nb;
+        if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
+        else if (p.c_dtype == LLMK_F16) store_row16<LLMK_F16>(p.c, off, acc[i], n_valid, vec_ok);
+        else store_row16<LLMK_F32>(p.c, off, acc[i], n_valid, vec_ok);
+    }
+}
+
+// fp16 / bf16 activation scales -> fp32 (the pipeline above streams 4-byte scale elements)
+template <int SDT>
+__global__ void scales_to_f32_kernel(const void* __restrict__ src, float* __restrict__ dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = FloatIO<SDT>::ld(src, i);
+}
+
+// true when the three-stage kernel can take this problem (32-bit source offsets, scale table size)
+inline bool dma_eligible(const DirectArgs& p) {
+    return (int64_t)p.M * p.K < (1ll << 32) && (int64_t)p.N * p.K < (1ll << 32) &&
+           (int64_t)p.M * (p.K >> 7) * 4 < (1ll << 32) && (p.K >> 7) <= D_MAX_KT && p.K > 0;
+}
+
+// a_s must be fp32 here (p.a_s); p.s_dtype describes b_s only.
+template <int KIND, bool GROUPED>
+int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
+    static bool configured = false;
+    auto kern = gemm_dma_kernel<KIND, GROUPED>;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, D_LDS);
+        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, D_LDS, hipGetErrorString(e));
+        configured = true;
+    }
+    const int tiles_m = (p.M + D_BM - 1) / D_BM + (GROUPED ? p.E : 0);
+    dim3 grid((unsigned)((p.N + D_BN - 1) / D_BN), (unsigned)tiles_m);
+    if (grid.x == 0 || grid.y == 0) return LLMK_OK;
+    kern<<<grid, D_THREADS, D_LDS, stream>>>(p);
+    LLMK_CHECK_LAUNCH(name);
+    return LLMK_OK;
+}
+
+// Dispatch for the compute-bound block-scaled GEMM: three-stage kernel when eligible (converting 16-bit
+// activation scales into `workspace` first), register-staged two-stage kernel otherwise.
+template <int KIND, bool GROUPED>
+int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream_t stream, const char* name) {
+    if (!dma_eligible(p)) return launch_tiled<KIND, GROUPED>(p, stream, name);
+    if (p.s_dtype != LLMK_F32) {
+        const int64_t n = (int64_t)p.M * (p.K >> 7);
+        if (!workspace || workspace_bytes < n * 4) return launch_tiled<KIND, GROUPED>(p, stream, name);
+        const unsigned blocks = (unsigned)cdiv64(n, 256);
+        if (p.s_dtype == LLMK_F16) scales_to_f32_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
+        else scales_to_f32_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
+        LLMK_CHECK_LAUNCH(name);
+        p.a_s = workspace;
+    }
+    return launch_dma<KIND, GROUPED>(p, stream, name);
+}
+
+}  // namespace llmk

@@ -21,8 +21,24 @@ constexpr int T_B_BYTES = T_BN * T_ROW;            // 18432
 constexpr int T_STAGE = T_A_BYTES + T_B_BYTES + T_BM * 4;   // + the scale column of this K step
 constexpr int T_LDS = 2 * T_STAGE;                 // 112640 bytes
 
-template <int KIND, bool GROUPED>
+// raw scale element (fp32 bits or 16-bit pattern) -> fp32; SDT is a dtype code known at compile time
+template <int SDT> struct ScaleIO;
+template <> struct ScaleIO<LLMK_F32> {
+    typedef float Raw;
+    static __device__ __forceinline__ float cvt(Raw v) { return v; }
+};
+template <> struct ScaleIO<LLMK_F16> {
+    typedef unsigned short Raw;
+    static __device__ __forceinline__ float cvt(Raw v) { return f16_to_f32(v); }
+};
+template <> struct ScaleIO<LLMK_BF16> {
+    typedef unsigned short Raw;
+    static __device__ __forceinline__ float cvt(Raw v) { return bf16_to_f32(v); }
+};
+
+template <int KIND, bool GROUPED, int SDT>
 __global__ __launch_bounds__(T_THREADS) void gemm_tiled_kernel(DirectArgs p) {
+    typedef typename ScaleIO<SDT>::Raw SRaw;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, g = lane >> 4;
@@ -66,13 +82,18 @@ __global__ __launch_bounds__(T_THREADS) void gemm_tiled_kernel(DirectArgs p) {
     const int64_t bs_row = bs_off + (int64_t)blockIdx.x * KT;     // T_BN == 128: one weight-scale block per tile
 
     v4i ra[4], rb[2];
-    float rsa = 0.f;
+    SRaw raw_as = 0, raw_bs = 0;
+    const SRaw* as_ptr = (const SRaw*)p.a_s + as_row;
+    const SRaw* bs_ptr = (const SRaw*)p.b_s + bs_row;
+    // the scale loads go first: the memory counter retires in order, and nothing may wait on them
+    // before the tile loads behind them have been issued
     auto gload = [&](int kt) {
+        raw_as = as_ptr[kt];
+        raw_bs = bs_ptr[kt];
 #pragma unroll
         for (int i = 0; i < 4; ++i) ra[i] = *(const v4i*)(ag[i] + (int64_t)kt * 128);
 #pragma unroll
         for (int i = 0; i < 2; ++i) rb[i] = *(const v4i*)(bg[i] + (int64_t)kt * 128);
-        if (tid < T_BM) rsa = ld_scale(p.a_s, as_row + kt, p.s_dtype) * ld_scale(p.b_s, bs_row + kt, p.s_dtype);
     };
     auto lstore = [&](int buf) {
         uint8_t* base = lds + buf * T_STAGE;
@@ -80,7 +101,7 @@ __global__ __launch_bounds__(T_THREADS) void gemm_tiled_kernel(DirectArgs p) {
         for (int i = 0; i < 4; ++i) *(v4i*)(base + (i * 64 + lrow) * T_ROW + lchunk) = ra[i];
 #pragma unroll
         for (int i = 0; i < 2; ++i) *(v4i*)(base + T_A_BYTES + (i * 64 + lrow) * T_ROW + lchunk) = rb[i];
-        if (tid < T_BM) ((float*)(base + T_A_BYTES + T_B_BYTES))[tid] = rsa;
+        if (tid < T_BM) ((float*)(base + T_A_BYTES + T_B_BYTES))[tid] = ScaleIO<SDT>::cvt(raw_as) * ScaleIO<SDT>::cvt(raw_bs);
     };
 
     v4f acc[4][4];
@@ -134,10 +155,10 @@ __global__ __launch_bounds__(T_THREADS) void gemm_tiled_kernel(DirectArgs p) {
         }
 }
 
-template <int KIND, bool GROUPED>
-int launch_tiled(const DirectArgs& p, hipStream_t stream, const char* name) {
+template <int KIND, bool GROUPED, int SDT>
+int launch_tiled_sdt(const DirectArgs& p, hipStream_t stream, const char* name) {
     static bool configured = false;
-    auto kern = gemm_tiled_kernel<KIND, GROUPED>;
+    auto kern = gemm_tiled_kernel<KIND, GROUPED, SDT>;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T_LDS);
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, T_LDS, hipGetErrorString(e));
@@ -149,6 +170,21 @@ int launch_tiled(const DirectArgs& p, hipStream_t stream, const char* name) {
     kern<<<grid, T_THREADS, T_LDS, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     return LLMK_OK;
+}
+
+template <int KIND, bool GROUPED>
+int launch_tiled(const DirectArgs& p, hipStream_t stream, const char* name) {
+    if constexpr (KIND == K_FP8_BLOCK) {
+        if (p.s_dtype != LLMK_F32) LLMK_FAIL(LLMK_ERR_DTYPE, "%s: fp8 block scales must be fp32", name);
+        return launch_tiled_sdt<KIND, GROUPED, LLMK_F32>(p, stream, name);
+    } else {
+        switch (p.s_dtype) {
+            case LLMK_F32:  return launch_tiled_sdt<KIND, GROUPED, LLMK_F32>(p, stream, name);
+            case LLMK_F16:  return launch_tiled_sdt<KIND, GROUPED, LLMK_F16>(p, stream, name);
+            case LLMK_BF16: return launch_tiled_sdt<KIND, GROUPED, LLMK_BF16>(p, stream, name);
+            default: LLMK_FAIL(LLMK_ERR_DTYPE, "%s: s_dtype %d", name, p.s_dtype);
+        }
+    }
 }
 
 }  // namespace llmk

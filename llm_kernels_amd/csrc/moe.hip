@@ -1,6 +1,6 @@
 // Single-GPU expert-parallel MoE path: segment bookkeeping, token permute / un-permute,
 // gated activation, and the grouped GEMM over one GPU's experts.
-#include "gemm_tiled.hpp"
+#include "gemm_dma.hpp"
 
 using namespace llmk;
 
@@ -163,7 +163,8 @@ extern "C" int llmk_moe_post_reorder(const void* down_out, void* out, int dtype,
 
 extern "C" int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind, int c_dtype, int E, int64_t M,
                                  int64_t N, int64_t K, const int64_t* seg_indptr, const int64_t* weight_indices,
-                                 const void* scale_a, const void* scale_b, int s_dtype, void* stream) {
+                                 const void* scale_a, const void* scale_b, int s_dtype, void* workspace,
+                                 int64_t workspace_bytes, void* stream) {
     if (M < 0 || N < 0 || K < 0 || E < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "grouped_gemm: negative dimension");
     if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm: c_dtype %d", c_dtype);
     const bool scaled = (kind == LLMK_KIND_I8 || kind == LLMK_KIND_FP8);
@@ -180,8 +181,8 @@ extern "C" int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind
     p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = E;
     hipStream_t st = (hipStream_t)stream;
     const bool big = M > 64 * (int64_t)E;            // average segment long enough for 256-row tiles
-    if (big && kind == LLMK_KIND_I8) return launch_tiled<K_I8_BLOCK, true>(p, st, "grouped_gemm(i8, tiled)");
-    if (big && kind == LLMK_KIND_FP8) return launch_tiled<K_FP8_BLOCK, true>(p, st, "grouped_gemm(fp8, tiled)");
+    if (big && kind == LLMK_KIND_I8) return launch_big<K_I8_BLOCK, true>(p, workspace, workspace_bytes, st, "grouped_gemm(i8, tiled)");
+    if (big && kind == LLMK_KIND_FP8) return launch_big<K_FP8_BLOCK, true>(p, workspace, workspace_bytes, st, "grouped_gemm(fp8, tiled)");
     switch (kind) {
         case LLMK_KIND_I8:   return launch_direct<K_I8_BLOCK, true>(p, (int)M, st, "grouped_gemm(i8)");
         case LLMK_KIND_FP8:  return launch_direct<K_FP8_BLOCK, true>(p, (int)M, st, "grouped_gemm(fp8)");

@@ -174,5 +174,6 @@ def grouped_gemm_triton(
         wi = (weight_indices if weight_indices.dtype == torch.int64 else weight_indices.to(torch.int64)).contiguous()
     _lib.call("llmk_grouped_gemm", _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), kind, _lib.dt(c.dtype), int(batch_size),
               a.shape[0], b.shape[1], b.shape[2], _lib.ptr(seg), _lib.ptr(wi), _lib.ptr(scale_a), _lib.ptr(scale_b),
-              s_dt, _lib.stream(a), exc=AssertionError)
+              s_dt, *_lib.gemm_workspace(a.device, a.shape[0], b.shape[1], b.shape[2]), _lib.stream(a),
+              exc=AssertionError)
     return c

@@ -58,7 +58,8 @@ def int8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Te
     assert a_s.dtype == b_s.dtype, 'activation and weight scales must share a dtype'
     c = a.new_empty(*a.size()[:-1], N, dtype=torch.get_default_dtype())
     _lib.call("llmk_gemm_i8_block", _lib.ptr(a), _lib.ptr(a_s), _lib.ptr(b), _lib.ptr(b_s), _lib.dt(a_s.dtype),
-              _lib.ptr(c), _lib.dt(c.dtype), M, N, K, None, 0, _lib.stream(a), exc=AssertionError)
+              _lib.ptr(c), _lib.dt(c.dtype), M, N, K, *_lib.gemm_workspace(a.device, M, N, K), _lib.stream(a),
+              exc=AssertionError)
     return c
 
 
