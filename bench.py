@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Throughput of the quantized-GEMM path on one MI355X, against its roofline, with a CPU baseline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--headline-only] [--no-cpu] [--eager]
 
 A "step" is one GEMM call over one batch of synthetic input already resident in HBM.  Small-M
 (HBM-bound) workloads rotate through enough distinct weight copies to exceed the 256 MB on-die cache,
@@ -42,6 +42,30 @@ def _bytes_w4a16(M, N, K, g=128):
 def _bytes_w4a8(M, N, K):
     kb, nb = K // 128, (N + 127) // 128
     return M * K + N * K // 2 + 2 * M * kb + 2 * nb * kb + 2 * N * kb + 2 * M * N
+
+
+class CopyCase:
+    """Plain device-to-device copy of a known size: the calibration point for the HBM traffic counters."""
+
+    def __init__(self, name, nbytes):
+        self.name, self.op, self.M, self.N, self.K = name, "copy", 0, 0, 0
+        self.nbytes = nbytes
+        self.flops = 0.0
+        self.bytes = 2 * nbytes
+        self.bound, self.mfma_dtype, self.dtype, self.nbuf = "hbm", "fp8", "u8", 1
+
+    def setup(self, dev):
+        src = torch.empty(self.nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        self.launch = lambda i: dst.copy_(src)
+
+    def cpu_seconds(self, max_rows):
+        a = torch.empty(self.nbytes, dtype=torch.uint8).random_(0, 255)
+        b = torch.empty_like(a)
+        b.copy_(a)
+        t0 = time.perf_counter()
+        b.copy_(a)
+        return time.perf_counter() - t0, 0
 
 
 class Case:
@@ -188,17 +212,26 @@ def run_case(case, dev, steps, warmup, eager=False):
     return wall, e0.elapsed_time(e1)
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE runs (profiles/traffic.json)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(workload, {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
 def record(case, wall, ev_ms, steps):
     dur = ev_ms / 1e3 / steps                       # average launch-to-launch duration from HIP events
     tflops = case.flops / dur / 1e12
     gbs = case.bytes / dur / 1e9
     if case.bound == "hbm":
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": measured_traffic(case.name)}
     else:
         pk = PEAK_TFLOPS[case.mfma_dtype]
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": pk, "unit": "TFLOP/s",
-                "frac": round(tflops / pk, 4), "traffic": None}
+                "frac": round(tflops / pk, 4), "traffic": measured_traffic(case.name)}
     return {"workload": case.name, "M": case.M, "N": case.N, "K": case.K, "us_per_launch": round(dur * 1e6, 2),
             "tflops": round(tflops, 2), "gbs": round(gbs, 1), "alg_bytes": case.bytes, "flops": case.flops,
             "weight_copies_rotated": case.nbuf, "wall_ms_per_step": round(wall * 1e3 / steps, 4), "roofline": roof}
@@ -210,7 +243,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
-    ap.add_argument("--all", action="store_true", help="also measure the other headline shapes (reported under 'cases')")
+    ap.add_argument("--headline-only", action="store_true", help="skip the other headline shapes (reported under 'cases')")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--eager", action="store_true", help="launch every step from Python instead of replaying a HIP graph")
     args = ap.parse_args()
@@ -223,13 +256,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.set_default_dtype(torch.bfloat16)
 
-    op, M, N, K = WORKLOADS[args.workload]
-    case = Case(args.workload, op, M, N, K)
+    if args.workload == "copy_256m":
+        op, M, N, K = "copy", 0, 0, 0
+        case = CopyCase(args.workload, 256 << 20)
+    else:
+        op, M, N, K = WORKLOADS[args.workload]
+        case = Case(args.workload, op, M, N, K)
     wall, ev_ms = run_case(case, dev, args.steps, args.warmup, args.eager)
     rec = record(case, wall, ev_ms, args.steps)
 
     cases = []
-    if args.all:
+    if not args.headline_only and args.workload in WORKLOADS:
         for name in HEADLINE_SET:
             if name == args.workload:
                 continue
@@ -246,10 +283,14 @@ def main():
         torch.set_num_threads(cores)
         max_rows = 512                                # bounded sample of the same workload
         dt, rows = case.cpu_seconds(max_rows)
-        cpu_tflops = 2.0 * rows * N * K / dt / 1e12
-        cpu = {"value": round(cpu_tflops, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-               "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
-                         "1 warm-up + 1 timed pass, weight dequantisation included (%.2f s)" % (rows, M, dt)}
+        if op == "copy":
+            cpu = {"value": round(case.bytes / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                   "sample": "host memcpy of the same size"}
+        else:
+            cpu = {"value": round(2.0 * rows * N * K / dt / 1e12, 4), "unit": "TFLOP/s",
+                   "cores": torch.get_num_threads(), "kind": "port",
+                   "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
+                             "1 warm-up + 1 timed pass, weight dequantisation included (%.2f s)" % (rows, M, dt)}
 
     out = {
         "metric": "w4a16/fp8 GEMM TFLOPS & % roofline (HBM at M=16, MFMA at M=4096)",
