@@ -68,7 +68,7 @@ struct DirectArgs {
     int M, N, K, E;
 };
 
-template <int KIND, int MT, int NW, bool GROUPED>
+template <int KIND, int MT, int NW, bool GROUPED, bool RESIDENT>
 __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     constexpr bool HALF = (KIND == K_F16 || KIND == K_BF16);
     constexpr int ESZ = HALF ? 2 : 1;
@@ -78,7 +78,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16;
     const int K = p.K, N = p.N;
     const int steps = K / KSTEP;
 
@@ -106,105 +105,218 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         m_end = min(p.M, m_start + 16 * MT);
     }
 
-    const int nrow = min(n0 + r, N - 1);
-    const uint8_t* bp = bbase + ((int64_t)nrow * K) * ESZ + 32 * g;
     const uint8_t* ap[MT];
-    int srow[MT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int arow = min(m_start + 16 * mt + r, m_end - 1);
         ap[mt] = p.a + ((int64_t)arow * K) * ESZ + 32 * g;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) srow[mt][i] = min(m_start + 16 * mt + 4 * g + i, m_end - 1);
     }
 
-    v4f acc[MT];
-    v4i acci[MT];
+    // A batch is U K-steps of this wave; all its loads are issued before any of them is consumed.  Steps
+    // past the end are clamped to the last step and nullified.  When the whole K range of a wave fits in
+    // one batch (RESIDENT), the activation fragments are loaded once and reused for every column tile the
+    // workgroup processes, and the weight batch of the next tile is requested before the current tile is
+    // reduced; otherwise batches are double-buffered along K.
+    constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+    struct BBatch {
+        v8i b[U];
+        float bs[U];
+    };
+    struct ABatch {
+        v8i a[U][MT];
+    };
+    const int ntiles = (N + 15) / 16;
+    auto ks_of = [&](int ks0, int u, bool& valid) {
+        const int ks = ks0 + u * NW;
+        valid = ks < steps;
+        return valid ? ks : steps - 1;
+    };
+    auto load_b = [&](BBatch& t, int tile, int ks0) {
+        const int nrow = min(tile * 16 + r, N - 1);
+        const uint8_t* bp = bbase + ((int64_t)nrow * K) * ESZ + 32 * g;
+        const int64_t bs_row = bs_off + (int64_t)(tile * 16 / 128) * steps;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) { acc[mt] = (v4f){0.f, 0.f, 0.f, 0.f}; acci[mt] = (v4i){0, 0, 0, 0}; }
-    const int64_t bs_row = bs_off + (int64_t)(n0 / 128) * steps;
+        for (int u = 0; u < U; ++u) {
+            bool valid;
+            const int ksc = ks_of(ks0, u, valid);
+            t.bs[u] = 1.f;
+            if constexpr (BLOCKSCALE) t.bs[u] = valid ? ld_scale(p.b_s, bs_row + ksc, p.s_dtype) : 0.f;
+            t.b[u] = ld32(bp + (int64_t)ksc * 128);
+            if constexpr (!BLOCKSCALE) {
+                if (!valid) t.b[u] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+            }
+        }
+    };
+    auto load_a = [&](ABatch& t, int ks0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            bool valid;
+            const int ksc = ks_of(ks0, u, valid);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) t.a[u][mt] = ld32(ap[mt] + (int64_t)ksc * 128);
+        }
+    };
 
-#pragma unroll 2
-    for (int ks = wave; ks < steps; ks += NW) {
-        const v8i b = ld32(bp + (int64_t)ks * 128);
-        float bs = 1.f;
-        if constexpr (BLOCKSCALE) bs = ld_scale(p.b_s, bs_row + ks, p.s_dtype);
+    // activation scales of the tile rows for every K step -> LDS (requested before the first batch so that
+    // the wait for them does not drain the batch behind them)
+    constexpr int RB = MT == 4 ? 1 : 2;      // reduction buffers (one needs a second barrier per tile)
+    float* asl = red + RB * NW * MT * 256;
+    constexpr int SROWS = MT * 16;
+    float stage_as[4];
+    const int n_as = BLOCKSCALE ? SROWS * steps : 0;
+    if constexpr (BLOCKSCALE) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const v8i a = ld32(ap[mt] + (int64_t)ks * 128);
-            if constexpr (BLOCKSCALE) {
-                const v4f t = step_dot<KIND>(a, b);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float as = ld_scale(p.a_s, (int64_t)srow[mt][i] * steps + ks, p.s_dtype);
-                    acc[mt][i] += t[i] * (as * bs);
-                }
-            } else if constexpr (KIND == K_I8_ROWCOL) {
-                v4i a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]};
-                v4i b0 = {b[0], b[1], b[2], b[3]}, b1 = {b[4], b[5], b[6], b[7]};
-                acci[mt] = mfma_i8_16x16x64(a0, b0, acci[mt]);
-                acci[mt] = mfma_i8_16x16x64(a1, b1, acci[mt]);
-            } else if constexpr (KIND == K_F16) {
-                v8h a0, a1, b0, b1;
-                __builtin_memcpy(&a0, &a, 16); __builtin_memcpy(&a1, ((const char*)&a) + 16, 16);
-                __builtin_memcpy(&b0, &b, 16); __builtin_memcpy(&b1, ((const char*)&b) + 16, 16);
-                acc[mt] = mfma_f16_16x16x32(a0, b0, acc[mt]);
-                acc[mt] = mfma_f16_16x16x32(a1, b1, acc[mt]);
-            } else {
-                v8bf a0, a1, b0, b1;
-                __builtin_memcpy(&a0, &a, 16); __builtin_memcpy(&a1, ((const char*)&a) + 16, 16);
-                __builtin_memcpy(&b0, &b, 16); __builtin_memcpy(&b1, ((const char*)&b) + 16, 16);
-                acc[mt] = mfma_bf16_16x16x32(a0, b0, acc[mt]);
-                acc[mt] = mfma_bf16_16x16x32(a1, b1, acc[mt]);
+        for (int q = 0; q < 4; ++q) {
+            const int idx = (int)threadIdx.x + q * NW * 64;
+            stage_as[q] = 0.f;
+            if (idx < n_as) {
+                const int rr = idx / steps, kk = idx - rr * steps;
+                stage_as[q] = ld_scale(p.a_s, (int64_t)min(m_start + rr, m_end - 1) * steps + kk, p.s_dtype);
             }
         }
     }
-
-    // cross-wave reduction of the K split; integer accumulators travel as raw bits
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        float* dst = red + ((wave * MT + mt) * 64 + lane) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            dst[i] = (KIND == K_I8_ROWCOL) ? __int_as_float(acci[mt][i]) : acc[mt][i];
+    int tile = blockIdx.x;
+    ABatch acur, anxt;
+    BBatch bcur, bnxt;
+    if (steps > 0 && tile < ntiles) {
+        load_b(bcur, tile, wave);
+        load_a(acur, wave);
     }
-    __syncthreads();
-    for (int o = threadIdx.x; o < MT * 256; o += NW * 64) {
-        const int mt = o >> 8, row16 = (o & 255) >> 4, col = o & 15;
-        const int src = (mt * 64 + (row16 >> 2) * 16 + col) * 4 + (row16 & 3);
-        const int m = m_start + 16 * mt + row16, n = n0 + col;
-        if (m >= m_end || n >= N) continue;
-        if constexpr (KIND == K_I8_ROWCOL) {
-            int s = 0;
+    if constexpr (BLOCKSCALE) {
 #pragma unroll
-            for (int w = 0; w < NW; ++w) s += __float_as_int(red[w * MT * 256 + src]);
-            if (p.c_i32) p.c_i32[(int64_t)m * N + n] = s;
-            if (p.c) st_out(p.c, (int64_t)m * N + n, (float)s * ((const float*)p.a_s)[m] * ((const float*)p.b_s)[n], p.c_dtype);
-        } else {
-            float s = 0.f;
-#pragma unroll
-            for (int w = 0; w < NW; ++w) s += red[w * MT * 256 + src];
-            st_out(p.c, (int64_t)m * N + n, s, p.c_dtype);
+        for (int q = 0; q < 4; ++q) {
+            const int idx = (int)threadIdx.x + q * NW * 64;
+            if (idx < n_as) asl[idx] = stage_as[q];
         }
+        for (int idx = (int)threadIdx.x + 4 * NW * 64; idx < n_as; idx += NW * 64) {   // very long K only
+            const int rr = idx / steps, kk = idx - rr * steps;
+            asl[idx] = ld_scale(p.a_s, (int64_t)min(m_start + rr, m_end - 1) * steps + kk, p.s_dtype);
+        }
+        __syncthreads();
     }
+
+    auto mul_batch = [&](const ABatch& ta, const BBatch& tb, int ks0, v4f (&acc)[MT], v4i (&acci)[MT]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const v8i b = tb.b[u];
+            bool valid;
+            const int ksc = ks_of(ks0, u, valid);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const v8i a = ta.a[u][mt];
+                if constexpr (BLOCKSCALE) {
+                    const v4f t = step_dot<KIND>(a, b);
+                    const float bs = tb.bs[u];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float as = asl[(mt * 16 + 4 * g + i) * steps + ksc];
+                        acc[mt][i] += t[i] * (as * bs);
+                    }
+                } else if constexpr (KIND == K_I8_ROWCOL) {
+                    v4i a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]};
+                    v4i b0 = {b[0], b[1], b[2], b[3]}, b1 = {b[4], b[5], b[6], b[7]};
+                    acci[mt] = mfma_i8_16x16x64(a0, b0, acci[mt]);
+                    acci[mt] = mfma_i8_16x16x64(a1, b1, acci[mt]);
+                } else if constexpr (KIND == K_F16) {
+                    v8h a0, a1, b0, b1;
+                    __builtin_memcpy(&a0, &a, 16); __builtin_memcpy(&a1, ((const char*)&a) + 16, 16);
+                    __builtin_memcpy(&b0, &b, 16); __builtin_memcpy(&b1, ((const char*)&b) + 16, 16);
+                    acc[mt] = mfma_f16_16x16x32(a0, b0, acc[mt]);
+                    acc[mt] = mfma_f16_16x16x32(a1, b1, acc[mt]);
+                } else {
+                    v8bf a0, a1, b0, b1;
+                    __builtin_memcpy(&a0, &a, 16); __builtin_memcpy(&a1, ((const char*)&a) + 16, 16);
+                    __builtin_memcpy(&b0, &b, 16); __builtin_memcpy(&b1, ((const char*)&b) + 16, 16);
+                    acc[mt] = mfma_bf16_16x16x32(a0, b0, acc[mt]);
+                    acc[mt] = mfma_bf16_16x16x32(a1, b1, acc[mt]);
+                }
+            }
+        }
+    };
+
+    int parity = 0;
+    for (; tile < ntiles; tile += gridDim.x, parity ^= 1) {
+        v4f acc[MT];
+        v4i acci[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) { acc[mt] = (v4f){0.f, 0.f, 0.f, 0.f}; acci[mt] = (v4i){0, 0, 0, 0}; }
+        const int next_tile = tile + gridDim.x;
+        if constexpr (RESIDENT) {
+            if (next_tile < ntiles) load_b(bnxt, next_tile, wave);
+            mul_batch(acur, bcur, wave, acc, acci);
+            if (next_tile < ntiles) bcur = bnxt;
+        } else {
+            for (int ks0 = wave; ks0 < steps; ks0 += NW * U) {
+                const int nk = ks0 + NW * U;
+                const bool more = nk < steps;
+                if (more) { load_b(bnxt, tile, nk); load_a(anxt, nk); }
+                else if (next_tile < ntiles) { load_b(bnxt, next_tile, wave); load_a(anxt, wave); }
+                mul_batch(acur, bcur, ks0, acc, acci);
+                if (more || next_tile < ntiles) { bcur = bnxt; acur = anxt; }
+            }
+        }
+
+        // cross-wave reduction of the K split (two alternating buffers: one barrier per tile);
+        // integer accumulators travel as raw bits
+        float* rbuf = red + (RB == 2 ? parity : 0) * NW * MT * 256;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            float* dst = rbuf + ((wave * MT + mt) * 64 + lane) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                dst[i] = (KIND == K_I8_ROWCOL) ? __int_as_float(acci[mt][i]) : acc[mt][i];
+        }
+        __syncthreads();
+        const int n0 = tile * 16;
+        for (int o = threadIdx.x; o < MT * 256; o += NW * 64) {
+            const int mt = o >> 8, row16 = (o & 255) >> 4, col = o & 15;
+            const int src = (mt * 64 + (row16 >> 2) * 16 + col) * 4 + (row16 & 3);
+            const int m = m_start + 16 * mt + row16, n = n0 + col;
+            if (m >= m_end || n >= N) continue;
+            if constexpr (KIND == K_I8_ROWCOL) {
+                int s = 0;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) s += __float_as_int(rbuf[w * MT * 256 + src]);
+                if (p.c_i32) p.c_i32[(int64_t)m * N + n] = s;
+                if (p.c) st_out(p.c, (int64_t)m * N + n, (float)s * ((const float*)p.a_s)[m] * ((const float*)p.b_s)[n], p.c_dtype);
+            } else {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) s += rbuf[w * MT * 256 + src];
+                st_out(p.c, (int64_t)m * N + n, s, p.c_dtype);
+            }
+        }
+        if constexpr (RB == 1) __syncthreads();
+    }
+}
+
+template <int KIND, int MT, bool GROUPED>
+int launch_direct_mt(const DirectArgs& p, hipStream_t stream, const char* name) {
+    constexpr int NW = 8;
+    constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+    constexpr bool HALF = (KIND == K_F16 || KIND == K_BF16);
+    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
+    const int steps = p.K / (HALF ? 64 : 128);
+    const int ntiles = (p.N + 15) / 16;
+    const int mtiles = (p.M + 16 * MT - 1) / (16 * MT) + (GROUPED ? p.E : 0);
+    if (ntiles == 0 || mtiles == 0) return LLMK_OK;
+    const size_t smem = (size_t)(MT == 4 ? 1 : 2) * NW * MT * 256 * sizeof(float) + (SCALED ? (size_t)MT * 16 * steps * sizeof(float) : 0);
+    if (smem > 64 * 1024) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: K=%d too large for the weight-streaming kernel's scale table", name, p.K);
+    // column tiles are processed persistently: at most ~2 workgroups per CU and m-tile row
+    const int gx = min(ntiles, max(1, 512 / min(mtiles, 512)));
+    dim3 grid((unsigned)gx, (unsigned)mtiles), block(NW * 64);
+    if (steps <= NW * U) gemm_direct_kernel<KIND, MT, NW, GROUPED, true><<<grid, block, smem, stream>>>(p);
+    else gemm_direct_kernel<KIND, MT, NW, GROUPED, false><<<grid, block, smem, stream>>>(p);
+    LLMK_CHECK_LAUNCH(name);
+    return LLMK_OK;
 }
 
 template <int KIND, bool GROUPED>
 int launch_direct(const DirectArgs& p, int max_rows_per_segment_hint, hipStream_t stream, const char* name) {
     // m-tiles per workgroup: 1 for decode-sized M, up to 4 otherwise
-    const int M = p.M;
-    const int mt = (max_rows_per_segment_hint <= 16) ? 1 : (max_rows_per_segment_hint <= 32 ? 2 : 4);
-    constexpr int NW = 8;
-    dim3 block(NW * 64);
-    auto tiles = [&](int rows) { return (rows + 16 * mt - 1) / (16 * mt); };
-    dim3 grid((unsigned)((p.N + 15) / 16), (unsigned)(GROUPED ? tiles(M) + p.E : tiles(M)));
-    if (grid.y == 0 || grid.x == 0) return LLMK_OK;
-    const size_t smem = (size_t)NW * mt * 256 * sizeof(float);
-    if (mt == 1) gemm_direct_kernel<KIND, 1, NW, GROUPED><<<grid, block, smem, stream>>>(p);
-    else if (mt == 2) gemm_direct_kernel<KIND, 2, NW, GROUPED><<<grid, block, smem, stream>>>(p);
-    else gemm_direct_kernel<KIND, 4, NW, GROUPED><<<grid, block, smem, stream>>>(p);
-    LLMK_CHECK_LAUNCH(name);
-    return LLMK_OK;
+    if (max_rows_per_segment_hint <= 16) return launch_direct_mt<KIND, 1, GROUPED>(p, stream, name);
+    if (max_rows_per_segment_hint <= 32) return launch_direct_mt<KIND, 2, GROUPED>(p, stream, name);
+    return launch_direct_mt<KIND, 4, GROUPED>(p, stream, name);
 }
 
 }  // namespace llmk
