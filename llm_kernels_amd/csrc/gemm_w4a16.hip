@@ -86,6 +86,7 @@ __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
 
     int cur_grp0 = -1, cur_grp1 = -1;
     v8h s0 = {}, s1 = {};
+#pragma unroll 2
     for (int ks = ks_begin + wave; ks < ks_end; ks += NW) {
         const int st0 = 2 * ks, st1 = 2 * ks + 1;
         const bool have1 = st1 < strips;
@@ -122,22 +123,23 @@ __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
         }
     }
 
-    reduce_waves<NW, MT * 32>(acc, red, wave, lane);
-    if (wave != 0 || !chunk_ok) return;
+    // one-barrier reduction over the waves: slot e of lane l of wave w sits at red[(w * NE + e) * 64 + l]
+    constexpr int NE = MT * 32;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int e = 0; e < NE; ++e) red[(wave * NE + e) * 64 + lane] = acc[e];
+    __syncthreads();
+    for (int e = wave; e < NE; e += NW) {
+        float v = 0.f;
 #pragma unroll
-        for (int t = 0; t < 8; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int m = m0 + 16 * mt + 4 * g + i;
-                const int n = 64 * chunk + 16 * (t >> 1) + 8 * (t & 1) + c;
-                if (m < M) {
-                    const float v = acc[(mt * 8 + t) * 4 + i];
-                    if constexpr (TO_WS) ws[((int64_t)blockIdx.z * M + m) * N + n] = v;
-                    else C[(int64_t)m * N + n] = (_Float16)v;
-                }
-            }
+        for (int w = 0; w < NW; ++w) v += red[(w * NE + e) * 64 + lane];
+        const int mt = e >> 5, t = (e >> 2) & 7, i = e & 3;
+        const int m = m0 + 16 * mt + 4 * g + i;
+        const int n = 64 * chunk + 16 * (t >> 1) + 8 * (t & 1) + c;
+        if (chunk_ok && m < M) {
+            if constexpr (TO_WS) ws[((int64_t)blockIdx.z * M + m) * N + n] = v;
+            else C[(int64_t)m * N + n] = (_Float16)v;
+        }
+    }
 }
 
 __global__ void splitk_reduce_f16_kernel(const float* __restrict__ ws, _Float16* __restrict__ C, int64_t MN, int Z) {
@@ -211,19 +213,33 @@ __global__ __launch_bounds__(NW * 64) void w4a16_nk_kernel(
         }
 }
 
-// number of K slices (workgroups along z) used for decode-sized M
-int marlin_split_k(int col_groups, int total_steps) {
+// launch shape of the Marlin-layout kernel for a given problem
+struct MarlinPlan {
+    int mt, nw, mblocks, col_groups, z, steps_per_z;
+};
+
+MarlinPlan marlin_plan(int64_t M, int64_t N, int64_t K) {
+    MarlinPlan pl{};
+    pl.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    pl.nw = pl.mt == 1 ? 8 : (pl.mt == 2 ? 4 : 2);          // nw * mt * 8 KiB of reduction LDS <= 64 KiB
+    pl.mblocks = (int)cdiv64(M, 16 * pl.mt);
+    pl.col_groups = (int)((N / 64 + 1) / 2);
+    const int total_steps = (int)((K / 16 + 1) / 2);
+    // split K over workgroups until the grid covers the chip; every slice keeps >= nw steps
     int z = 1;
-    while (col_groups * z < 256 && total_steps / (z * 2) >= 8) z *= 2;
-    return z;
+    if (M <= 64)
+        while ((int64_t)pl.col_groups * pl.mblocks * z < 256 && total_steps / (z * 2) >= pl.nw) z *= 2;
+    pl.z = z;
+    pl.steps_per_z = (total_steps + z - 1) / z;
+    return pl;
 }
 
 }  // namespace
 
 extern "C" int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    if (M <= 0 || N <= 0 || K <= 0 || M > 16) return 0;
-    const int z = marlin_split_k((int)((N / 64 + 1) / 2), (int)((K / 16 + 1) / 2));
-    return z > 1 ? (int64_t)z * M * N * 4 : 0;
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const MarlinPlan pl = marlin_plan(M, N, K);
+    return pl.z > 1 ? (int64_t)pl.z * M * N * 4 : 0;
 }
 
 extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, const void* s, int64_t M, int64_t N,
@@ -242,37 +258,32 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)s) & 15) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a16_marlin: operands must be 16-byte aligned");
     if (M > 0x7fffffff / 2 || N > 0x7fffffff / 2 || K > 0x7fffffff / 2) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: dimension too large");
 
-    const int total_steps = (int)((K / 16 + 1) / 2);
-    const int col_groups = (int)((N / 64 + 1) / 2);
+    MarlinPlan pl = marlin_plan(M, N, K);
+    if (pl.z > 1 && (!workspace || workspace_bytes < (int64_t)pl.z * M * N * 4)) {
+        pl.z = 1;                                   // no scratch: every workgroup walks all of K
+        pl.steps_per_z = (int)((K / 16 + 1) / 2);
+    }
     hipStream_t st = (hipStream_t)stream;
     const _Float16* A = (const _Float16*)a;
     const v4i* B = (const v4i*)b;
     const _Float16* S = (const _Float16*)s;
     _Float16* C = (_Float16*)c;
-
-    if (M <= 16) {
-        constexpr int NW = 8;
-        // split K over workgroups until the grid covers the chip; each workgroup keeps >= NW steps
-        int z = marlin_split_k(col_groups, total_steps);
-        while (z > 1 && (!workspace || workspace_bytes < (int64_t)z * M * N * 4)) z >>= 1;
-        const int spz = (total_steps + z - 1) / z;
-        dim3 grid(col_groups, 1, z), blk(NW * 64);
-        const size_t smem = (size_t)(NW / 2) * 32 * 64 * sizeof(float);
-        if (z == 1) {
-            w4a16_marlin_kernel<1, NW, false><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, spz);
-            LLMK_CHECK_LAUNCH("gemm_w4a16_marlin");
-        } else {
-            w4a16_marlin_kernel<1, NW, true><<<grid, blk, smem, st>>>(A, B, S, C, (float*)workspace, (int)M, (int)N, (int)K, groupsize, spz);
-            LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(split)");
-            splitk_reduce_f16_kernel<<<(unsigned)cdiv64(M * N, 256), 256, 0, st>>>((const float*)workspace, C, M * N, z);
-            LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(reduce)");
-        }
-    } else {
-        constexpr int MT = 4, NW = 2;
-        dim3 grid(col_groups, (unsigned)cdiv64(M, 16 * MT), 1), blk(NW * 64);
-        const size_t smem = (size_t)(NW / 2) * MT * 32 * 64 * sizeof(float);
-        w4a16_marlin_kernel<MT, NW, false><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, total_steps);
-        LLMK_CHECK_LAUNCH("gemm_w4a16_marlin");
+    float* ws = (float*)workspace;
+    dim3 grid(pl.col_groups, pl.mblocks, pl.z), blk(pl.nw * 64);
+    const size_t smem = (size_t)pl.nw * pl.mt * 32 * 64 * sizeof(float);
+#define LLMK_MARLIN_LAUNCH(MT, NW)                                                                              \
+    do {                                                                                                        \
+        if (pl.z > 1) w4a16_marlin_kernel<MT, NW, true><<<grid, blk, smem, st>>>(A, B, S, C, ws, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
+        else w4a16_marlin_kernel<MT, NW, false><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
+    } while (0)
+    if (pl.mt == 1) LLMK_MARLIN_LAUNCH(1, 8);
+    else if (pl.mt == 2) LLMK_MARLIN_LAUNCH(2, 4);
+    else LLMK_MARLIN_LAUNCH(4, 2);
+#undef LLMK_MARLIN_LAUNCH
+    LLMK_CHECK_LAUNCH("gemm_w4a16_marlin");
+    if (pl.z > 1) {
+        splitk_reduce_f16_kernel<<<(unsigned)cdiv64(M * N, 256), 256, 0, st>>>((const float*)workspace, C, M * N, pl.z);
+        LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(reduce)");
     }
     return LLMK_OK;
 }

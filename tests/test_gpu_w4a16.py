@@ -117,3 +117,26 @@ def test_w4a16_nk_device_quantize_round_trip(dev):
     diff = (qd.cpu().int() - oq.int()).abs()
     assert diff.max() <= 1 and (diff != 0).sum() <= 64
     assert torch.equal(unpack_over_cols(packed, 4, 4096), qd)       # pack/unpack round trip, bit exact
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 1024, 4096), (64, 512, 8192), (16, 256, 14336)])
+def test_mul_split_k_is_deterministic_and_rearms(dev, M, N, K):
+    """Decode shapes split K over workgroups inside one launch; repeated launches must give identical bits
+    (fixed summation order) and leave the ticket counters re-armed."""
+    announce("marlin split-k repeat", M, N, K)
+    torch.manual_seed(7)
+    A = (torch.randn(M, K) * 0.3).half()
+    W = (torch.randn(K, N) * 0.05).half()
+    _, q, s = mr.fake_quantize(W, 128)
+    B, sp = mr.pack(q, s, 128)
+    Ag, Bg, sg = A.to(dev), B.to(dev), sp.to(dev)
+    ws = torch.zeros(64, dtype=torch.int32, device=dev)
+    outs = []
+    for _ in range(20):
+        C = torch.empty(M, N, dtype=torch.half, device=dev)
+        mul(Ag, Bg, C, sg, ws)
+        outs.append(C)
+    torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    assert_close_scaled(outs[0], g.w4a16_gemm(A, q, s, 128), what="marlin split-k")
