@@ -35,6 +35,7 @@ __device__ __forceinline__ void dma4(uint32_t lds_addr, uint32_t voff, const voi
 // s_waitcnt immediates for gfx9: vmcnt = imm[3:0] | imm[15:14] << 4, expcnt = imm[6:4] (7 = no wait),
 // lgkmcnt = imm[11:8] (15 = no wait)
 #define LLMK_WAIT_VMCNT_7 0x0F77
+#define LLMK_WAIT_VMCNT_6 0x0F76
 #define LLMK_WAIT_VMCNT_0 0x0F70
 
 
@@ -73,15 +74,24 @@ __device__ __forceinline__ void store_row16(void* c, int64_t off, const v4f (&v)
     }
 }
 
-template <int KIND, bool GROUPED>
+// MI = 16-row tiles per wave along M (4, 2 or 1): the workgroup tile is 64*MI rows x 128 columns.
+template <int KIND, bool GROUPED, int MI>
 __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
+    constexpr int BM = 64 * MI;              // tile rows
+    constexpr int WR = 16 * MI;              // rows per wave
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
-    const int K = p.K, N = p.N;
+    // SCALED: 8-bit operands with per-128-K block scales.  Otherwise fp16 / bf16 operands, no scales: a K
+    // step is still one 128-byte row segment (64 elements, two 16x16x32 MFMAs per tile) and the MFMAs
+    // accumulate directly.  Kb = bytes per operand row.
+    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
+    constexpr int ESZ = SCALED ? 1 : 2;
+    const int N = p.N;
+    const int K = p.K * ESZ;                 // row length in bytes
     const int KT = K >> 7;
     const int n0 = blockIdx.x * D_BN;
 
@@ -94,8 +104,8 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         bool found = false;
         for (; e < p.E; ++e) {
             const int64_t s1 = p.seg_indptr[e + 1];
-            const int t = (int)((s1 - s0 + D_BM - 1) / D_BM);
-            if (tile < cum + t) { found = true; m_start = (int)s0 + (tile - cum) * D_BM; m_end = min((int)s1, m_start + D_BM); break; }
+            const int t = (int)((s1 - s0 + BM - 1) / BM);
+            if (tile < cum + t) { found = true; m_start = (int)s0 + (tile - cum) * BM; m_end = min((int)s1, m_start + BM); break; }
             cum += t;
             s0 = s1;
         }
@@ -104,8 +114,8 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         bbase += widx * (int64_t)N * K;
         bs_off = widx * (int64_t)((N + 127) / 128) * KT;
     } else {
-        m_start = blockIdx.y * D_BM;
-        m_end = min(p.M, m_start + D_BM);
+        m_start = blockIdx.y * BM;
+        m_end = min(p.M, m_start + BM);
     }
 
     float* bsl = (float*)(lds + D_NSTAGE * D_STAGE);
@@ -117,11 +127,12 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // 16*((rho & 15) >> 2) + 4*(rho >> 4) + (rho & 3): MFMA j then produces, in lane group g, the four
     // columns 16g + 4j + (0..3), so that a lane ends up with 16 consecutive columns of one output row.
     const int row8 = lane >> 3;
-    uint32_t aoff[4], boff[2];
+    uint32_t aoff[MI], boff[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t chunk = (uint32_t)((lane & 7) ^ (((i & 1) * 4 + (row8 >> 1)) & 7)) * 16u;
-        aoff[i] = (uint32_t)min(m_start + 8 * (wave * 4 + i) + row8, m_end - 1) * (uint32_t)K + chunk;
+    for (int i = 0; i < MI; ++i) {
+        const int R = 8 * (wave * MI + i) + row8;
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ ((R >> 1) & 7)) * 16u;
+        aoff[i] = (uint32_t)min(m_start + R, m_end - 1) * (uint32_t)K + chunk;
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -130,7 +141,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const int col = (R & 64) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
-    const uint32_t soff = (uint32_t)min(m_start + (wave & 3) * 64 + lane, m_end - 1) * (uint32_t)KT * 4u;
+    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT * 4u;
 
     auto issue = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
@@ -138,16 +149,18 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const uint8_t* gb = bbase + (int64_t)kt * 128;
         const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(st + (uint32_t)(wave * 4 + i) * 1024u, aoff[i], ga);
+        for (int i = 0; i < MI; ++i) dma16(st + (uint32_t)(wave * MI + i) * 1024u, aoff[i], ga);
 #pragma unroll
         for (int i = 0; i < 2; ++i) dma16(st + D_A + (uint32_t)(wave * 2 + i) * 1024u, boff[i], gb);
-        dma4(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+        if constexpr (SCALED) dma4(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, soff, gs);
     };
+    // loads per stage per thread: MI (A) + 2 (B) + 1 (scale column); imm = vmcnt | no expcnt/lgkmcnt wait
+    constexpr int WAIT_ONE_STAGE = 0x0F70 | (MI + 2 + (SCALED ? 1 : 0));
 
     // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 64 x 64 tile
-    v4f acc[4][4];
+    v4f acc[MI][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
@@ -156,7 +169,8 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // weight scales of this tile for every K step -> LDS.  These are the only compiler-tracked vector
     // loads; they sit behind the first two stages in the memory queue, so waiting for them also waits
     // for stage 0 and 1 (an acceptable one-off: the pipeline is being filled anyway).
-    for (int i = tid; i < KT; i += D_THREADS) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
+    if constexpr (SCALED)
+        for (int i = tid; i < KT; i += D_THREADS) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
     __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
     __syncthreads();
 
@@ -172,60 +186,96 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // X (tile rows 0,1) and Y (tile rows 2,3).  While the MFMAs of one set run, the scale-and-accumulate
     // FMAs of the other set (finished half a step earlier) issue on the VALU: one MFMA (32 cycles) covers
     // the four FMAs (16 cycles) of one tile.
-    v4f tx[2][4], ty[2][4];
-    float sy[2] = {0.f, 0.f};
+    constexpr int H = MI >= 2 ? MI / 2 : 1;   // tile rows per register set (MI == 1: set X only, no overlap)
+    v4f tx[H][4], ty[H][4];
+    float sy[H];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < H; ++i) {
+        sy[i] = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) tx[i][j] = ty[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    }
 
     // fragments of the K step being multiplied (zero before the first load: multiplying them is a no-op)
-    v8i bf[4], af[4];
-    float sa[4];
+    v8i bf[4], af[MI];
+    float sa[MI];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        bf[i] = af[i] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+    for (int j = 0; j < 4; ++j) bf[j] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        af[i] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
         sa[i] = 0.f;
     }
     auto load_frags = [&](int kt) {
         const uint8_t* st = lds + (kt % D_NSTAGE) * D_STAGE;
-        const uint8_t* As = st + (wm * 64) * 128;
+        const uint8_t* As = st + (wm * WR) * 128;
         const uint8_t* Bs = st + D_A + (wn * 64) * 128;
-        const float* Ss = (const float*)(st + D_A + D_B) + wm * 64 + r;
-        const float bs = bsl[kt];
+        const float* Ss = (const float*)(st + D_A + D_B) + wm * WR + r;
 #pragma unroll
         for (int j = 0; j < 4; ++j) bf[j] = ldfrag(Bs + j * 2048);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[i] = ldfrag(As + i * 2048);
+        for (int i = 0; i < MI; ++i) af[i] = ldfrag(As + i * 2048);
+        if constexpr (SCALED) {
+            const float bs = bsl[kt];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sa[i] = Ss[i * 16] * bs;
+            for (int i = 0; i < MI; ++i) sa[i] = Ss[i * 16] * bs;
+        }
+    };
+    auto mma16 = [&](const v8i& x, const v8i& y, v4f c) {      // two 16x16x32 half-precision MFMAs
+        if constexpr (KIND == K_F16) {
+            v8h x0, x1, y0, y1;
+            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
+            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
+            c = mfma_f16_16x16x32(x0, y0, c);
+            return mfma_f16_16x16x32(x1, y1, c);
+        } else {
+            v8bf x0, x1, y0, y1;
+            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
+            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
+            c = mfma_bf16_16x16x32(x0, y0, c);
+            return mfma_bf16_16x16x32(x1, y1, c);
+        }
     };
     // The weight fragment is the MFMA row operand and the activation fragment the column operand, i.e.
     // the tile is produced transposed: a lane owns output row r and four consecutive columns per MFMA.
     // Branch-free so that the whole body is a single scheduling region.
     auto compute = [&]() {
-        // phase 1: X <- rows 0,1 of this step; retire Y of the previous step into acc rows 2,3
+        if constexpr (!SCALED) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                acc[2 + i][j] += ty[i][j] * sy[i];
-                tx[i][j] = step_dot<KIND>(bf[j], af[i]);
-                __builtin_amdgcn_sched_group_barrier(0x008, KIND == K_FP8_BLOCK ? 1 : 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, KIND == K_FP8_BLOCK ? 4 : 8, 0);
-            }
-        // phase 2: Y <- rows 2,3 of this step; retire X into acc rows 0,1
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
+                for (int j = 0; j < 4; ++j) acc[i][j] = mma16(bf[j], af[i], acc[i][j]);
+        } else if constexpr (MI == 1) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                ty[i][j] = step_dot<KIND>(bf[j], af[2 + i]);
-                acc[i][j] += tx[i][j] * sa[i];
-                __builtin_amdgcn_sched_group_barrier(0x008, KIND == K_FP8_BLOCK ? 1 : 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, KIND == K_FP8_BLOCK ? 4 : 8, 0);
+                acc[0][j] += tx[0][j] * sy[0];                  // retire the previous step while this one multiplies
+                tx[0][j] = step_dot<KIND>(bf[j], af[0]);
             }
-        sy[0] = sa[2];
-        sy[1] = sa[3];
+            sy[0] = sa[0];
+        } else {
+            // phase 1: X <- upper tile rows of this step; retire Y of the previous step into the lower acc rows
+#pragma unroll
+            for (int i = 0; i < H; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[H + i][j] += ty[i][j] * sy[i];
+                    tx[i][j] = step_dot<KIND>(bf[j], af[i]);
+                    __builtin_amdgcn_sched_group_barrier(0x008, KIND == K_FP8_BLOCK ? 1 : 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, KIND == K_FP8_BLOCK ? 4 : 8, 0);
+                }
+            // phase 2: Y <- lower tile rows of this step; retire X into the upper acc rows
+#pragma unroll
+            for (int i = 0; i < H; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    ty[i][j] = step_dot<KIND>(bf[j], af[H + i]);
+                    acc[i][j] += tx[i][j] * sa[i];
+                    __builtin_amdgcn_sched_group_barrier(0x008, KIND == K_FP8_BLOCK ? 1 : 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, KIND == K_FP8_BLOCK ? 4 : 8, 0);
+                }
+#pragma unroll
+            for (int i = 0; i < H; ++i) sy[i] = sa[H + i];
+        }
     };
 
     // Ping-pong between the two wave groups that share every SIMD (waves 0-3 and 4-7): group 0 reads the
@@ -239,7 +289,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             issue(kt + 2);
             load_frags(kt);
             compute();
-            __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_7);
+            __builtin_amdgcn_s_waitcnt(WAIT_ONE_STAGE);
             __syncthreads();
         }
         if (kt + 1 < KT) {
@@ -259,7 +309,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             compute();
             __builtin_amdgcn_sched_barrier(0);
             load_frags(kt);
-            __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_7);
+            __builtin_amdgcn_s_waitcnt(WAIT_ONE_STAGE);
             __syncthreads();
         }
         if (kt + 1 < KT) {
@@ -277,10 +327,16 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         }
         compute();
     }
+    if constexpr (SCALED && MI >= 2) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < H; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[2 + i][j] += ty[i][j] * sy[i];
+            for (int j = 0; j < 4; ++j) acc[H + i][j] += ty[i][j] * sy[i];
+    }
+    if constexpr (SCALED && MI == 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[0][j] += tx[0][j] * sy[0];
+    }
 
     // ---- epilogue: every lane writes 16 consecutive outputs of each of its four rows
     const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
@@ -288,8 +344,8 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     const int nb = n0 + wn * 64 + 16 * g;
     const int n_valid = N - nb;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m_start + wm * 64 + 16 * i + r;
+    for (int i = 0; i < MI; ++i) {
+        const int m = m_start + wm * WR + 16 * i + r;
         if (m >= m_end || n_valid <= 0) continue;
         const int64_t off = (int64_t)m * N + nb;
         if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
@@ -306,27 +362,42 @@ __global__ void scales_to_f32_kernel(const void* __restrict__ src, float* __rest
 }
 
 // true when the three-stage kernel can take this problem (32-bit source offsets, scale table size)
-inline bool dma_eligible(const DirectArgs& p) {
-    return (int64_t)p.M * p.K < (1ll << 32) && (int64_t)p.N * p.K < (1ll << 32) &&
-           (int64_t)p.M * (p.K >> 7) * 4 < (1ll << 32) && (p.K >> 7) <= D_MAX_KT && p.K > 0;
+inline bool dma_eligible(const DirectArgs& p, int esz = 1) {
+    const int64_t kb = (int64_t)p.K * esz;              // row bytes
+    return (int64_t)p.M * kb < (1ll << 32) && (int64_t)p.N * kb < (1ll << 32) && kb % 128 == 0 &&
+           (int64_t)p.M * (kb >> 7) * 4 < (1ll << 32) && (kb >> 7) <= D_MAX_KT && p.K > 0;
 }
 
 // a_s must be fp32 here (p.a_s); p.s_dtype describes b_s only.
-template <int KIND, bool GROUPED>
-int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
+template <int KIND, bool GROUPED, int MI>
+int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     static bool configured = false;
-    auto kern = gemm_dma_kernel<KIND, GROUPED>;
+    auto kern = gemm_dma_kernel<KIND, GROUPED, MI>;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, D_LDS);
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, D_LDS, hipGetErrorString(e));
         configured = true;
     }
-    const int tiles_m = (p.M + D_BM - 1) / D_BM + (GROUPED ? p.E : 0);
+    constexpr int BM = 64 * MI;
+    const int tiles_m = (p.M + BM - 1) / BM + (GROUPED ? p.E : 0);
     dim3 grid((unsigned)((p.N + D_BN - 1) / D_BN), (unsigned)tiles_m);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
     kern<<<grid, D_THREADS, D_LDS, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     return LLMK_OK;
+}
+
+// Tile height by occupancy: the tallest tile (least weight re-reading) that still gives every CU a
+// workgroup.  Segments of a grouped GEMM are judged by their average length.
+template <int KIND, bool GROUPED>
+int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
+    const int64_t ncol = (p.N + D_BN - 1) / D_BN;
+    const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
+    const int64_t groups = GROUPED ? p.E : 1;
+    auto wgs = [&](int bm) { return ncol * groups * ((rows + bm - 1) / bm); };
+    if (wgs(256) >= 256 || rows > 1024) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
+    if (wgs(128) >= 256 || rows > 512) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
+    return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
 }
 
 // Dispatch for the compute-bound block-scaled GEMM: three-stage kernel when eligible (converting 16-bit
@@ -343,6 +414,13 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
         LLMK_CHECK_LAUNCH(name);
         p.a_s = workspace;
     }
+    return launch_dma<KIND, GROUPED>(p, stream, name);
+}
+
+// fp16 / bf16 operands, no scales (K % 64 == 0)
+template <int KIND, bool GROUPED>
+int launch_big_half(const DirectArgs& p, hipStream_t stream, const char* name) {
+    if (!dma_eligible(p, 2)) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: shape not supported by the tiled half-precision kernel", name);
     return launch_dma<KIND, GROUPED>(p, stream, name);
 }
 

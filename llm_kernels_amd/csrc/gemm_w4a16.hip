@@ -2,7 +2,7 @@
 //
 // nibble -> fp16 without integer->float converts: (q | 0x6400) is the fp16 number 1024 + q,
 // ((q << 4) | 0x6400) is 1024 + 16 q; one packed subtract / fma gives q - 8 exactly.
-#include "common.hpp"
+#include "gemm_dma.hpp"
 
 namespace {
 
@@ -151,6 +151,42 @@ __global__ void splitk_reduce_f16_kernel(const float* __restrict__ ws, _Float16*
 }
 
 // ------------------------------------------------------------------------------------------
+// Marlin words -> dequantised fp16 W^T [N][K] (K contiguous), the operand layout of the tiled GEMM.
+// One workgroup converts 8 strips (128 K) of one 64-column chunk: every thread expands one 16-byte unit
+// (32 values, scaled in fp16 exactly as the fused kernels do), the tile is transposed through LDS and
+// written as 256-byte row segments.
+__global__ __launch_bounds__(256) void marlin_dequant_kernel(const v4i* __restrict__ B, const _Float16* __restrict__ S,
+                                                             _Float16* __restrict__ Wt, int N, int K, int groupsize) {
+    __shared__ __attribute__((aligned(16))) _Float16 tile[64][136];
+    const int tid = threadIdx.x, sl = tid >> 5, ml = tid & 31, c = ml >> 2, q = ml & 3;
+    const int nchunks = N >> 6, strips = K >> 4;
+    const int chunk = blockIdx.x, strip = blockIdx.y * 8 + sl;
+    if (strip < strips) {
+        const v4i w = B[((int64_t)strip * nchunks + chunk) * 32 + ml];
+        const v8h sc = *(const v8h*)(S + (int64_t)((16 * strip) / groupsize) * N + 64 * chunk + 8 * c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const unsigned u = ((unsigned)w[j]) >> (8 * b);
+                const v2h s2 = {sc[2 * j + b], sc[2 * j + b]};
+                const int n = 16 * j + 8 * b + c, k = 16 * sl + 2 * q;
+                *(v2h*)&tile[n][k] = deq_lo(u) * s2;
+                *(v2h*)&tile[n][k + 8] = deq_hi(u) * s2;
+            }
+    }
+    __syncthreads();
+    const int row = tid >> 2, seg = tid & 3;
+    const int k0 = blockIdx.y * 128;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        const int kl = seg * 32 + x * 8;
+        if (k0 + kl < K)
+            *(v8h*)(Wt + (int64_t)(64 * chunk + row) * K + k0 + kl) = *(const v8h*)&tile[row][kl];
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // [N, K/8] layout (pack_weights_over_cols: nibble i of word w of row n is k = 8w + i) with
 // scales [N, K/g].  Lane (r = column, g) loads one 16-byte unit = 32 consecutive k of its row per
 // 128-K step; word j feeds MFMA j, whose fragment order is k offsets [0,4,1,5,2,6,3,7] -- the A
@@ -238,6 +274,7 @@ MarlinPlan marlin_plan(int64_t M, int64_t N, int64_t K) {
 
 extern "C" int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (M > 64) return K % 64 == 0 ? N * K * 2 : 0;      // dequantised fp16 copy of W for the tiled GEMM
     const MarlinPlan pl = marlin_plan(M, N, K);
     return pl.z > 1 ? (int64_t)pl.z * M * N * 4 : 0;
 }
@@ -258,12 +295,24 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)s) & 15) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a16_marlin: operands must be 16-byte aligned");
     if (M > 0x7fffffff / 2 || N > 0x7fffffff / 2 || K > 0x7fffffff / 2) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: dimension too large");
 
+    hipStream_t st = (hipStream_t)stream;
+    if (M > 64 && K % 64 == 0 && workspace && workspace_bytes >= N * K * 2 && !((uintptr_t)workspace & 15)) {
+        // compute-bound: expand W once to fp16 [N, K], then run the tiled MFMA GEMM on it
+        llmk::DirectArgs p{};
+        p.a = (const uint8_t*)a; p.b = (const uint8_t*)workspace; p.c = c; p.c_dtype = LLMK_F16;
+        p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+        if (llmk::dma_eligible(p, 2)) {
+            dim3 dgrid((unsigned)(N / 64), (unsigned)cdiv64(K, 128));
+            marlin_dequant_kernel<<<dgrid, 256, 0, st>>>((const v4i*)b, (const _Float16*)s, (_Float16*)workspace, (int)N, (int)K, groupsize);
+            LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(dequant)");
+            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_marlin(tiled)");
+        }
+    }
     MarlinPlan pl = marlin_plan(M, N, K);
     if (pl.z > 1 && (!workspace || workspace_bytes < (int64_t)pl.z * M * N * 4)) {
         pl.z = 1;                                   // no scratch: every workgroup walks all of K
         pl.steps_per_z = (int)((K / 16 + 1) / 2);
     }
-    hipStream_t st = (hipStream_t)stream;
     const _Float16* A = (const _Float16*)a;
     const v4i* B = (const v4i*)b;
     const _Float16* S = (const _Float16*)s;

@@ -183,6 +183,8 @@ extern "C" int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind
     const bool big = M > 64 * (int64_t)E;            // average segment long enough for 256-row tiles
     if (big && kind == LLMK_KIND_I8) return launch_big<K_I8_BLOCK, true>(p, workspace, workspace_bytes, st, "grouped_gemm(i8, tiled)");
     if (big && kind == LLMK_KIND_FP8) return launch_big<K_FP8_BLOCK, true>(p, workspace, workspace_bytes, st, "grouped_gemm(fp8, tiled)");
+    if (big && kind == LLMK_KIND_F16 && dma_eligible(p, 2)) return launch_big_half<K_F16, true>(p, st, "grouped_gemm(f16, tiled)");
+    if (big && kind == LLMK_KIND_BF16 && dma_eligible(p, 2)) return launch_big_half<K_BF16, true>(p, st, "grouped_gemm(bf16, tiled)");
     switch (kind) {
         case LLMK_KIND_I8:   return launch_direct<K_I8_BLOCK, true>(p, (int)M, st, "grouped_gemm(i8)");
         case LLMK_KIND_FP8:  return launch_direct<K_FP8_BLOCK, true>(p, (int)M, st, "grouped_gemm(fp8)");

@@ -153,3 +153,25 @@ def test_w4a8_exact_and_wrap(dev):
                                   s4.to(dev), z4.to(dev))
     b8 = q.w4a8_dequant_int8(wq, s4, z4)
     assert torch.equal(c.cpu().long(), a.long() @ b8.long().T)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
+@pytest.mark.parametrize("M,N,K", [(65, 128, 128), (130, 200, 256), (300, 384, 512), (520, 256, 384), (1100, 130, 256)])
+def test_tiled_kernels_ragged_shapes(dev, kind, M, N, K):
+    """Shapes that exercise every tile height of the large-M kernel, with ragged M and N."""
+    announce("tiled ragged", kind, M, N, K)
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    if kind == "fp8":
+        a, a_s = q.act_quant_fp8(x)
+        b, b_s = q.weight_quant_fp8(w)
+        fn = fp8_kernel.fp8_gemm
+    else:
+        a, a_s = q.act_quant_int8(x)
+        b, b_s = q.weight_quant_int8(w)
+        fn = int8_kernel.int8_gemm
+    for out in (torch.bfloat16, torch.float32):
+        with default_dtype(out):
+            c = fn(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+        assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="tiled %s" % kind)
