@@ -68,6 +68,72 @@ class CopyCase:
         return time.perf_counter() - t0, 0
 
 
+class MoECase:
+    """Mixtral-8x7B shaped expert set on one GPU: permute -> grouped GEMM -> SwiGLU -> grouped GEMM -> un-permute.
+
+    8 experts, hidden 4096, intermediate 14336, fp8 128x128 block-scaled weights, 4096 bf16 tokens,
+    softmax top-2 routing.  A step is the whole forward of moe/ep_moe.py (activation quantisation included).
+    """
+
+    def __init__(self, name, kind="fp8", T=4096, H=4096, I=14336, E=8, topk=2):
+        self.name, self.op, self.kind = name, "moe", kind
+        self.T, self.H, self.I, self.E, self.topk = T, H, I, E, topk
+        self.M, self.N, self.K = T * topk, 2 * I, H
+        rows = T * topk
+        self.flops = 2.0 * rows * (2 * I) * H + 2.0 * rows * H * I
+        kb1, kb2 = H // 128, I // 128
+        self.bytes = (rows * H + E * 2 * I * H + 4 * rows * kb1 + 4 * E * (2 * I // 128) * kb1 + 2 * rows * 2 * I) + \
+                     (rows * I + E * H * I + 4 * rows * kb2 + 4 * E * (H // 128) * kb2 + 2 * rows * H)
+        self.bound, self.mfma_dtype, self.nbuf = "mfma", ("fp8" if kind == "fp8" else "int8"), 1
+        self.dtype = "fp8_e4m3" if kind == "fp8" else "int8"
+
+    def setup(self, dev):
+        from llm_kernels_amd.moe.ep_moe import ep_moe_forward, softmax_topk_router
+        from llm_kernels_amd.quantization import fp8_kernel, int8_kernel
+        torch.manual_seed(0)
+        T, H, I, E = self.T, self.H, self.I, self.E
+        wq = fp8_kernel.weight_quant if self.kind == "fp8" else int8_kernel.weight_quant
+        qdt = torch.float8_e4m3fn if self.kind == "fp8" else torch.int8
+        sdt = torch.float32 if self.kind == "fp8" else torch.float16
+        w13 = torch.empty(E, 2 * I, H, dtype=qdt, device=dev)
+        w13s = torch.empty(E, 2 * I // 128, H // 128, dtype=sdt, device=dev)
+        w2 = torch.empty(E, H, I, dtype=qdt, device=dev)
+        w2s = torch.empty(E, H // 128, I // 128, dtype=sdt, device=dev)
+        for e in range(E):                                    # per expert: bounds the fp32 staging memory
+            w13[e], w13s[e] = wq(torch.randn(2 * I, H, device=dev) * 0.02)
+            w2[e], w2s[e] = wq(torch.randn(H, I, device=dev) * 0.02)
+        x = torch.randn(T, H, device=dev).bfloat16()
+        ids, wts = softmax_topk_router(torch.randn(T, E, device=dev), self.topk)
+        self.tensors = (x, ids, wts, w13, w2, w13s, w2s)
+        self.counts = torch.bincount(ids.flatten(), minlength=E).tolist()
+        self.launch = lambda i: ep_moe_forward(x, ids, wts, w13, w2, w13s, w2s, block_shape=[128, 128])
+
+    def cpu_seconds(self, max_rows):
+        """Dense per-expert SwiGLU loop in fp32 on dequantised weights, for the first `max_rows` tokens."""
+        import torch.nn.functional as F
+        x, ids, wts, w13, w2, w13s, w2s = [t.cpu() for t in self.tensors]
+        rows = min(self.T, max_rows)
+        x, ids, wts = x[:rows].float(), ids[:rows], wts[:rows].float()
+
+        def deq(w, s):
+            wf = w.float() if w.dtype == torch.int8 else w.to(torch.float32)
+            return wf * s.float().repeat_interleave(128, 0).repeat_interleave(128, 1)
+
+        def run():
+            out = torch.zeros(rows, self.H, dtype=torch.float32)
+            for e in range(self.E):
+                tok, slot = torch.where(ids == e)
+                if tok.numel() == 0:
+                    continue
+                h = x[tok] @ deq(w13[e], w13s[e]).T
+                y = (F.silu(h[:, :self.I]) * h[:, self.I:]) @ deq(w2[e], w2s[e]).T
+                out.index_add_(0, tok, y * wts[tok, slot][:, None])
+            return out
+        t0 = time.perf_counter()
+        run()
+        return time.perf_counter() - t0, rows
+
+
 class Case:
     """One GEMM workload: device buffers (rotated), a launcher, algorithmic cost and a CPU restatement."""
 
@@ -173,9 +239,10 @@ for _op in ("fp8", "int8", "w4a8", "w4a16", "w4a16_nk"):
         for _N, _K in ((4096, 4096), (6144, 4096), (14336, 4096), (28672, 4096), (4096, 14336)):
             WORKLOADS["%s_m%d_n%d_k%d" % (_op, _M, _N, _K)] = (_op, _M, _N, _K)
 
+MOE_WORKLOADS = {"moe_mixtral_fp8_t4096": "fp8", "moe_mixtral_int8_t4096": "int8"}
 DEFAULT_WORKLOAD = "fp8_m4096_n4096_k4096"
 HEADLINE_SET = ["w4a16_m16_n4096_k4096", "fp8_m16_n4096_k4096", "fp8_m16_n28672_k4096", "fp8_m16_n4096_k14336",
-                "w4a16_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "w4a8_m16_n4096_k4096"]
+                "w4a16_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "w4a8_m16_n4096_k4096", "moe_mixtral_fp8_t4096"]
 
 
 def run_case(case, dev, steps, warmup, eager=False):
@@ -259,6 +326,9 @@ def main():
     if args.workload == "copy_256m":
         op, M, N, K = "copy", 0, 0, 0
         case = CopyCase(args.workload, 256 << 20)
+    elif args.workload in MOE_WORKLOADS:
+        case = MoECase(args.workload, MOE_WORKLOADS[args.workload])
+        op, M, N, K = "moe", case.M, case.N, case.K
     else:
         op, M, N, K = WORKLOADS[args.workload]
         case = Case(args.workload, op, M, N, K)
@@ -270,7 +340,7 @@ def main():
         for name in HEADLINE_SET:
             if name == args.workload:
                 continue
-            c = Case(name, *WORKLOADS[name])
+            c = MoECase(name, MOE_WORKLOADS[name]) if name in MOE_WORKLOADS else Case(name, *WORKLOADS[name])
             w2, e2 = run_case(c, dev, args.steps, args.warmup, args.eager)
             cases.append(record(c, w2, e2, args.steps))
             del c
@@ -287,7 +357,8 @@ def main():
             cpu = {"value": round(case.bytes / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
                    "sample": "host memcpy of the same size"}
         else:
-            cpu = {"value": round(2.0 * rows * N * K / dt / 1e12, 4), "unit": "TFLOP/s",
+            cpu_flops = case.flops * rows / case.T if op == "moe" else 2.0 * rows * N * K
+            cpu = {"value": round(cpu_flops / dt / 1e12, 4), "unit": "TFLOP/s",
                    "cores": torch.get_num_threads(), "kind": "port",
                    "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
                              "1 warm-up + 1 timed pass, weight dequantisation included (%.2f s)" % (rows, M, dt)}
