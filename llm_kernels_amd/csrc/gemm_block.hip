@@ -1,5 +1,5 @@
 // Dense block-scaled fp8 / int8 GEMM entry points.
-#include "gemm_dma.hpp"
+#include "gemm_wide.hpp"
 
 using namespace llmk;
 

@@ -387,41 +387,4 @@ int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     return LLMK_OK;
 }
 
-// Tile height by occupancy: the tallest tile (least weight re-reading) that still gives every CU a
-// workgroup.  Segments of a grouped GEMM are judged by their average length.
-template <int KIND, bool GROUPED>
-int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
-    const int64_t ncol = (p.N + D_BN - 1) / D_BN;
-    const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
-    const int64_t groups = GROUPED ? p.E : 1;
-    auto wgs = [&](int bm) { return ncol * groups * ((rows + bm - 1) / bm); };
-    if (wgs(256) >= 256 || rows > 1024) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
-    if (wgs(128) >= 256 || rows > 512) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
-    return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
-}
-
-// Dispatch for the compute-bound block-scaled GEMM: three-stage kernel when eligible (converting 16-bit
-// activation scales into `workspace` first), register-staged two-stage kernel otherwise.
-template <int KIND, bool GROUPED>
-int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream_t stream, const char* name) {
-    if (!dma_eligible(p)) return launch_tiled<KIND, GROUPED>(p, stream, name);
-    if (p.s_dtype != LLMK_F32) {
-        const int64_t n = (int64_t)p.M * (p.K >> 7);
-        if (!workspace || workspace_bytes < n * 4) return launch_tiled<KIND, GROUPED>(p, stream, name);
-        const unsigned blocks = (unsigned)cdiv64(n, 256);
-        if (p.s_dtype == LLMK_F16) scales_to_f32_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
-        else scales_to_f32_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
-        LLMK_CHECK_LAUNCH(name);
-        p.a_s = workspace;
-    }
-    return launch_dma<KIND, GROUPED>(p, stream, name);
-}
-
-// fp16 / bf16 operands, no scales (K % 64 == 0)
-template <int KIND, bool GROUPED>
-int launch_big_half(const DirectArgs& p, hipStream_t stream, const char* name) {
-    if (!dma_eligible(p, 2)) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: shape not supported by the tiled half-precision kernel", name);
-    return launch_dma<KIND, GROUPED>(p, stream, name);
-}
-
 }  // namespace llmk

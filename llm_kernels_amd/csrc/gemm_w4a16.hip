@@ -2,7 +2,7 @@
 //
 // nibble -> fp16 without integer->float converts: (q | 0x6400) is the fp16 number 1024 + q,
 // ((q << 4) | 0x6400) is 1024 + 16 q; one packed subtract / fma gives q - 8 exactly.
-#include "gemm_dma.hpp"
+#include "gemm_wide.hpp"
 
 namespace {
 

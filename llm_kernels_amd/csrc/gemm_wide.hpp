@@ -1,0 +1,270 @@
+// 256 x 256 output tile variant of the direct-to-LDS pipeline, for problems large enough to fill the
+// chip with such tiles.  Per K step a workgroup moves (256 + 256) x 128 bytes from L2 to LDS for
+// 256 x 256 x 128 multiply-adds: a third less L2 and a quarter less LDS traffic per flop than the
+// 256 x 128 tile, which is what bounds that kernel.
+//
+// Workgroup: 512 threads = 8 waves, 2 along M x 4 along N; wave tile 128 rows x 64 columns =
+// 8 x 4 MFMA tiles (128 accumulator registers per lane).  Two LDS stages of 66560 bytes
+// (A 32 KB, B 32 KB, activation-scale column 1 KB): the loads of K step kt+1 fly while step kt is
+// multiplied, one barrier per step.
+//
+// Inside a step a wave keeps its four weight fragments in registers for the whole step and streams
+// the eight activation fragments through a two-deep register buffer.  The product of tile n is
+// scaled and accumulated (VALU) while the MFMAs of tiles n+1 and n+2 run, through a four-entry ring
+// of partial-product registers that carries over from one K step to the next.
+#pragma once
+#include "gemm_dma.hpp"
+
+namespace llmk {
+
+constexpr int W_BM = 256, W_BN = 256, W_THREADS = 512;
+constexpr int W_A = W_BM * 128, W_B = W_BN * 128, W_S = W_BM * 4;
+constexpr int W_STAGE = W_A + W_B + W_S;                   // 66560
+constexpr int W_LDS = 2 * W_STAGE + 2 * D_MAX_KT * 4;      // 135168 bytes
+
+template <int KIND, bool GROUPED>
+__global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int wm = wave >> 2, wn = wave & 3;
+    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
+    constexpr int ESZ = SCALED ? 1 : 2;
+    const int N = p.N;
+    const int K = p.K * ESZ;                 // row length in bytes
+    const int KT = K >> 7;
+    const int n0 = blockIdx.x * W_BN;
+
+    int m_start, m_end;
+    const uint8_t* bbase = p.b;
+    int64_t bs_off = 0;
+    if constexpr (GROUPED) {
+        int tile = blockIdx.y, e = 0, cum = 0;
+        int64_t s0 = p.seg_indptr[0];
+        bool found = false;
+        for (; e < p.E; ++e) {
+            const int64_t s1 = p.seg_indptr[e + 1];
+            const int t = (int)((s1 - s0 + W_BM - 1) / W_BM);
+            if (tile < cum + t) { found = true; m_start = (int)s0 + (tile - cum) * W_BM; m_end = min((int)s1, m_start + W_BM); break; }
+            cum += t;
+            s0 = s1;
+        }
+        if (!found) return;
+        const int64_t widx = p.weight_indices ? p.weight_indices[e] : e;
+        bbase += widx * (int64_t)N * K;
+        bs_off = widx * (int64_t)((N + 127) / 128) * KT;
+    } else {
+        m_start = blockIdx.y * W_BM;
+        m_end = min(p.M, m_start + W_BM);
+    }
+
+    // weight scales of the tile's two 128-column blocks, for every K step
+    float* bsl = (float*)(lds + 2 * W_STAGE);
+    const int nblk = (N + 127) / 128;
+
+    // ---- source offsets of the 9 loads of a stage.  Load i of a wave fills LDS rows 8q .. 8q+7,
+    // q = 4*wave + i.  A: LDS row R holds tile row R.  B: within each 64-row group, LDS row rho holds
+    // tile column 16*((rho & 15) >> 2) + 4*(rho >> 4) + (rho & 3), so that MFMA j yields, in lane group
+    // g, the four columns 16g + 4j + (0..3) and a lane ends up with 16 consecutive columns of a row.
+    // The 16-byte chunk index is XOR-swizzled with ((R >> 1) & 7) on the global side.
+    const int row8 = lane >> 3;
+    uint32_t aoff[4], boff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int R = 8 * (wave * 4 + i) + row8;
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ ((R >> 1) & 7)) * 16u;
+        aoff[i] = (uint32_t)min(m_start + R, m_end - 1) * (uint32_t)K + chunk;
+        const int rho = R & 63;
+        const int col = (R & 192) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
+        boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
+    }
+    const uint32_t soff = (uint32_t)min(m_start + (wave & 3) * 64 + lane, m_end - 1) * (uint32_t)KT * 4u;
+
+    auto issue = [&](int kt) {
+        const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
+        const uint8_t* ga = p.a + (int64_t)kt * 128;
+        const uint8_t* gb = bbase + (int64_t)kt * 128;
+        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(st + (uint32_t)(wave * 4 + i) * 1024u, aoff[i], ga);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(st + W_A + (uint32_t)(wave * 4 + i) * 1024u, boff[i], gb);
+        if constexpr (SCALED) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+    };
+
+    // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 128 x 64 tile
+    v4f acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    if (KT > 0) issue(0);
+    if constexpr (SCALED) {
+        for (int i = tid; i < 2 * KT; i += W_THREADS) {
+            const int c = i >= KT ? 1 : 0, kk = i - c * KT;
+            const int64_t blk = min(blockIdx.x * 2 + c, nblk - 1);
+            bsl[c * D_MAX_KT + kk] = ld_scale(p.b_s, bs_off + blk * KT + kk, p.s_dtype);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
+    __syncthreads();
+
+    const int lo = r * 128 + (((2 * g) ^ ((r >> 1) & 7)) * 16);
+    const int hi = r * 128 + (((2 * g + 1) ^ ((r >> 1) & 7)) * 16);
+    auto ldfrag = [&](const uint8_t* base) {
+        const v4i x = *(const v4i*)(base + lo), y = *(const v4i*)(base + hi);
+        return (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+    };
+    auto mma16 = [&](const v8i& x, const v8i& y, v4f c) {      // two 16x16x32 half-precision MFMAs
+        if constexpr (KIND == K_F16) {
+            v8h x0, x1, y0, y1;
+            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
+            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
+            c = mfma_f16_16x16x32(x0, y0, c);
+            return mfma_f16_16x16x32(x1, y1, c);
+        } else {
+            v8bf x0, x1, y0, y1;
+            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
+            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
+            c = mfma_bf16_16x16x32(x0, y0, c);
+            return mfma_bf16_16x16x32(x1, y1, c);
+        }
+    };
+
+    // ring of partial products: tile n = 4i + j of a step lives in t[j]; it is retired two tiles later.
+    // Tiles 30 and 31 of a step are retired by the first two tiles of the next one, with the scale of
+    // their own step (sprev).
+    v4f t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    float sprev = 0.f;
+
+    auto step = [&](int kt) {
+        const uint8_t* st = lds + (kt & 1) * W_STAGE;
+        const uint8_t* As = st + (wm * 128) * 128;
+        const uint8_t* Bs = st + W_A + (wn * 64) * 128;
+        v8i bf[4], af[2];
+        float sa[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bf[j] = ldfrag(Bs + j * 2048);
+        af[0] = ldfrag(As);
+        if constexpr (SCALED) {
+            const float* Ss = (const float*)(st + W_A + W_B) + wm * 128 + r;
+            const float bs = bsl[(wn >> 1) * D_MAX_KT + kt];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sa[i] = Ss[i * 16] * bs;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (i < 7) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (SCALED) {
+                    const int n = 4 * i + j;
+                    if (n >= 2) {
+                        const int m = n - 2;
+                        acc[m >> 2][m & 3] += t[m & 3] * sa[m >> 2];
+                    } else {
+                        acc[7][2 + n] += t[2 + n] * sprev;
+                    }
+                    t[j] = step_dot<KIND>(bf[j], af[i & 1]);
+                } else {
+                    acc[i][j] = mma16(bf[j], af[i & 1], acc[i][j]);
+                }
+                // Nothing moves across a tile boundary: the FMAs above retire the product of two tiles
+                // ago, never the one whose MFMA has just been issued, and each activation fragment is
+                // requested a whole tile row before its first use.
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if constexpr (SCALED) sprev = sa[7];
+    };
+
+    int kt = 0;
+    for (; kt + 1 < KT; ++kt) {
+        issue(kt + 1);
+        step(kt);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
+        __syncthreads();
+    }
+    if (kt < KT) step(kt);
+    if constexpr (SCALED) {
+        acc[7][2] += t[2] * sprev;
+        acc[7][3] += t[3] * sprev;
+    }
+
+    // ---- epilogue: every lane writes 16 consecutive outputs of each of its eight rows
+    const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
+    const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
+    const int nb = n0 + wn * 64 + 16 * g;
+    const int n_valid = N - nb;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int m = m_start + wm * 128 + 16 * i + r;
+        if (m >= m_end || n_valid <= 0) continue;
+        const int64_t off = (int64_t)m * N + nb;
+        if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
+        else if (p.c_dtype == LLMK_F16) store_row16<LLMK_F16>(p.c, off, acc[i], n_valid, vec_ok);
+        else store_row16<LLMK_F32>(p.c, off, acc[i], n_valid, vec_ok);
+    }
+}
+
+template <int KIND, bool GROUPED>
+int launch_wide(const DirectArgs& p, hipStream_t stream, const char* name) {
+    static bool configured = false;
+    auto kern = gemm_wide_kernel<KIND, GROUPED>;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, W_LDS);
+        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, W_LDS, hipGetErrorString(e));
+        configured = true;
+    }
+    const int tiles_m = (p.M + W_BM - 1) / W_BM + (GROUPED ? p.E : 0);
+    dim3 grid((unsigned)((p.N + W_BN - 1) / W_BN), (unsigned)tiles_m);
+    if (grid.x == 0 || grid.y == 0) return LLMK_OK;
+    kern<<<grid, W_THREADS, W_LDS, stream>>>(p);
+    LLMK_CHECK_LAUNCH(name);
+    return LLMK_OK;
+}
+
+// Tile shape by occupancy: the largest tile (least operand re-reading) that still gives every CU a
+// workgroup.  Segments of a grouped GEMM are judged by their average length.
+template <int KIND, bool GROUPED>
+int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
+    const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
+    const int64_t groups = GROUPED ? p.E : 1;
+    auto wgs = [&](int bm, int bn) { return ((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm); };
+    if (wgs(256, 256) >= 240) return launch_wide<KIND, GROUPED>(p, stream, name);
+    if (wgs(256, 128) >= 256 || rows > 1024) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
+    if (wgs(128, 128) >= 256 || rows > 512) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
+    return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
+}
+
+// Dispatch for the compute-bound block-scaled GEMM: direct-to-LDS kernels when eligible (converting
+// 16-bit activation scales into `workspace` first), register-staged two-stage kernel otherwise.
+template <int KIND, bool GROUPED>
+int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream_t stream, const char* name) {
+    if (!dma_eligible(p)) return launch_tiled<KIND, GROUPED>(p, stream, name);
+    if (p.s_dtype != LLMK_F32) {
+        const int64_t n = (int64_t)p.M * (p.K >> 7);
+        if (!workspace || workspace_bytes < n * 4) return launch_tiled<KIND, GROUPED>(p, stream, name);
+        const unsigned blocks = (unsigned)cdiv64(n, 256);
+        if (p.s_dtype == LLMK_F16) scales_to_f32_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
+        else scales_to_f32_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
+        LLMK_CHECK_LAUNCH(name);
+        p.a_s = workspace;
+    }
+    return launch_dma<KIND, GROUPED>(p, stream, name);
+}
+
+// fp16 / bf16 operands, no scales (K % 64 == 0)
+template <int KIND, bool GROUPED>
+int launch_big_half(const DirectArgs& p, hipStream_t stream, const char* name) {
+    if (!dma_eligible(p, 2)) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: shape not supported by the tiled half-precision kernel", name);
+    return launch_dma<KIND, GROUPED>(p, stream, name);
+}
+
+}  // namespace llmk

@@ -1,6 +1,6 @@
 // Single-GPU expert-parallel MoE path: segment bookkeeping, token permute / un-permute,
 // gated activation, and the grouped GEMM over one GPU's experts.
-#include "gemm_dma.hpp"
+#include "gemm_wide.hpp"
 
 using namespace llmk;
 

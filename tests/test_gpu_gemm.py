@@ -84,7 +84,7 @@ def test_int8_gemm(dev, M, N, K):
     assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="int8_gemm")
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 128, 128), (16, 256, 4096), (37, 130, 512), (128, 512, 14336)])
+@pytest.mark.parametrize("M,N,K", [(1, 128, 128), (16, 256, 4096), (37, 130, 512), (128, 512, 14336), (3850, 4110, 640)])
 def test_int8_block_accumulators_bit_exact(dev, M, N, K):
     """Unit scales and fp32 output: the result is the exact integer product (every 128-K int32 partial
     and their sum stay below 2^24 for |values| <= 15)."""
@@ -175,3 +175,28 @@ def test_tiled_kernels_ragged_shapes(dev, kind, M, N, K):
         with default_dtype(out):
             c = fn(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
         assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="tiled %s" % kind)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8", "int8_f32scales"])
+@pytest.mark.parametrize("M,N,K", [(4000, 4100, 256), (4096, 4096, 384), (3900, 4352, 128)])
+def test_wide_tile_kernel_ragged_shapes(dev, kind, M, N, K):
+    """Shapes large enough for the 256 x 256 tile, with ragged M and N, odd and single K step counts."""
+    announce("wide ragged", kind, M, N, K)
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    if kind == "fp8":
+        a, a_s = q.act_quant_fp8(x)
+        b, b_s = q.weight_quant_fp8(w)
+        fn = fp8_kernel.fp8_gemm
+    else:
+        a, a_s = q.act_quant_int8(x)
+        b, b_s = q.weight_quant_int8(w)
+        if kind == "int8_f32scales":
+            a_s, b_s = a_s.float(), b_s.float()
+        fn = int8_kernel.int8_gemm
+    ref = g.gemm_blockwise(a, a_s, b, b_s)
+    for out in (torch.bfloat16, torch.float32):
+        with default_dtype(out):
+            c = fn(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+        assert_close_scaled(c, ref, what="wide %s" % kind)
