@@ -174,9 +174,10 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
     __syncthreads();
 
-    // fragment read offsets inside a 16-row slab: chunks 2g and 2g+1 of row r, swizzled
-    const int lo = r * 128 + (((2 * g) ^ ((r >> 1) & 7)) * 16);
-    const int hi = r * 128 + (((2 * g + 1) ^ ((r >> 1) & 7)) * 16);
+    // fragment read offsets inside a 16-row slab: chunks g and g + 4 of row r, swizzled (same K order for
+    // both operands; the four lane groups of a b128 read then hit disjoint bank sets)
+    const int lo = r * 128 + ((g ^ ((r >> 1) & 7)) * 16);
+    const int hi = r * 128 + (((g + 4) ^ ((r >> 1) & 7)) * 16);
     auto ldfrag = [&](const uint8_t* base) {
         const v4i x = *(const v4i*)(base + lo), y = *(const v4i*)(base + hi);
         return (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};

@@ -10,8 +10,8 @@
 //
 // Inside a step a wave keeps its four weight fragments in registers for the whole step and streams
 // the eight activation fragments through a two-deep register buffer.  The product of tile n is
-// scaled and accumulated (VALU) while the MFMAs of tiles n+1 and n+2 run, through a four-entry ring
-// of partial-product registers that carries over from one K step to the next.
+// scaled and accumulated (VALU) while the MFMAs of the next tile row run, through two register sets
+// of partial products that carry over from one K step to the next.
 #pragma once
 #include "gemm_dma.hpp"
 
@@ -112,8 +112,11 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
     __syncthreads();
 
-    const int lo = r * 128 + (((2 * g) ^ ((r >> 1) & 7)) * 16);
-    const int hi = r * 128 + (((2 * g + 1) ^ ((r >> 1) & 7)) * 16);
+    // fragment read offsets inside a 16-row slab: lane group g takes 16-byte chunks g and g + 4 of row r
+    // (swizzled).  Both operands use the same K order, so the products are unchanged; with this order the
+    // four lane groups of a b128 read hit disjoint bank sets.
+    const int lo = r * 128 + ((g ^ ((r >> 1) & 7)) * 16);
+    const int hi = r * 128 + (((g + 4) ^ ((r >> 1) & 7)) * 16);
     auto ldfrag = [&](const uint8_t* base) {
         const v4i x = *(const v4i*)(base + lo), y = *(const v4i*)(base + hi);
         return (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
@@ -134,12 +137,12 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         }
     };
 
-    // ring of partial products: tile n = 4i + j of a step lives in t[j]; it is retired two tiles later.
-    // Tiles 30 and 31 of a step are retired by the first two tiles of the next one, with the scale of
-    // their own step (sprev).
-    v4f t[4];
+    // Partial products of a tile row live in one of two register sets: while the MFMAs of row i fill
+    // set i & 1, the FMAs scale and accumulate row i - 1 from the other set, four MFMAs after it was
+    // produced.  Row 7 of a step is retired by row 0 of the next one, with the scale of its own step.
+    v4f t[2][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) t[j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 4; ++j) t[0][j] = t[1][j] = (v4f){0.f, 0.f, 0.f, 0.f};
     float sprev = 0.f;
 
     auto step = [&](int kt) {
@@ -163,20 +166,15 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if constexpr (SCALED) {
-                    const int n = 4 * i + j;
-                    if (n >= 2) {
-                        const int m = n - 2;
-                        acc[m >> 2][m & 3] += t[m & 3] * sa[m >> 2];
-                    } else {
-                        acc[7][2 + n] += t[2 + n] * sprev;
-                    }
-                    t[j] = step_dot<KIND>(bf[j], af[i & 1]);
+                    t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
+                    if (i > 0) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
+                    else acc[7][j] += t[1][j] * sprev;
                 } else {
                     acc[i][j] = mma16(bf[j], af[i & 1], acc[i][j]);
                 }
-                // Nothing moves across a tile boundary: the FMAs above retire the product of two tiles
-                // ago, never the one whose MFMA has just been issued, and each activation fragment is
-                // requested a whole tile row before its first use.
+                // Nothing moves across a tile boundary: the FMAs retire a product finished four MFMAs
+                // ago, never the one just issued, and each activation fragment is requested a whole
+                // tile row before its first use.
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -193,8 +191,8 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     }
     if (kt < KT) step(kt);
     if constexpr (SCALED) {
-        acc[7][2] += t[2] * sprev;
-        acc[7][3] += t[3] * sprev;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[7][j] += t[1][j] * sprev;
     }
 
     // ---- epilogue: every lane writes 16 consecutive outputs of each of its eight rows
