@@ -36,6 +36,17 @@ __device__ __forceinline__ v8i ld32(const uint8_t* p) {
     return r;
 }
 
+// 32 bytes of a 128-byte K step for lane group g, taken as the 16-byte chunks g and g + 4 (pointer already
+// offset by 16 g): the four lane groups of a row then read 64 contiguous bytes per instruction.  The K order
+// inside an MFMA is free as long as both operands use the same one.
+__device__ __forceinline__ v8i ld_split(const uint8_t* p) {
+    const v4i lo = *(const v4i*)p, hi = *(const v4i*)(p + 64);
+    v8i r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
+}
+
 // product of one 32-byte-per-lane K step, returned as fp32 (exact for the integer kinds)
 template <int KIND>
 __device__ __forceinline__ v4f step_dot(const v8i& a, const v8i& b) {
@@ -76,7 +87,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     constexpr bool BLOCKSCALE = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
     extern __shared__ float red[];            // [NW][MT][64][4]
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: K-step indices stay scalar
     const int r = lane & 15, g = lane >> 4;
     const int K = p.K, N = p.N;
     const int steps = K / KSTEP;
@@ -109,7 +121,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int arow = min(m_start + 16 * mt + r, m_end - 1);
-        ap[mt] = p.a + ((int64_t)arow * K) * ESZ + 32 * g;
+        ap[mt] = p.a + ((int64_t)arow * K) * ESZ + 16 * g;
     }
 
     // A batch is U K-steps of this wave; all its loads are issued before any of them is consumed.  Steps
@@ -133,7 +145,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     };
     auto load_b = [&](BBatch& t, int tile, int ks0) {
         const int nrow = min(tile * 16 + r, N - 1);
-        const uint8_t* bp = bbase + ((int64_t)nrow * K) * ESZ + 32 * g;
+        const uint8_t* bp = bbase + ((int64_t)nrow * K) * ESZ + 16 * g;
         const int64_t bs_row = bs_off + (int64_t)(tile * 16 / 128) * steps;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -141,7 +153,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
             const int ksc = ks_of(ks0, u, valid);
             t.bs[u] = 1.f;
             if constexpr (BLOCKSCALE) t.bs[u] = valid ? ld_scale(p.b_s, bs_row + ksc, p.s_dtype) : 0.f;
-            t.b[u] = ld32(bp + (int64_t)ksc * 128);
+            t.b[u] = ld_split(bp + (int64_t)ksc * 128);
             if constexpr (!BLOCKSCALE) {
                 if (!valid) t.b[u] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
             }
@@ -153,7 +165,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
             bool valid;
             const int ksc = ks_of(ks0, u, valid);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) t.a[u][mt] = ld32(ap[mt] + (int64_t)ksc * 128);
+            for (int mt = 0; mt < MT; ++mt) t.a[u][mt] = ld_split(ap[mt] + (int64_t)ksc * 128);
         }
     };
 
@@ -177,7 +189,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     }
     int tile = blockIdx.x;
     ABatch acur, anxt;
-    BBatch bcur, bnxt;
+    BBatch bcur, bnxt, bnx2;
+    bool first = true;
     if (steps > 0 && tile < ntiles) {
         load_b(bcur, tile, wave);
         load_a(acur, wave);
@@ -242,9 +255,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         for (int mt = 0; mt < MT; ++mt) { acc[mt] = (v4f){0.f, 0.f, 0.f, 0.f}; acci[mt] = (v4i){0, 0, 0, 0}; }
         const int next_tile = tile + gridDim.x;
         if constexpr (RESIDENT) {
-            if (next_tile < ntiles) load_b(bnxt, next_tile, wave);
+            // two column tiles ahead: bnxt was requested while the previous tile was multiplied
+            const int next2 = next_tile + gridDim.x;
+            if (first && next_tile < ntiles) load_b(bnxt, next_tile, wave);
+            if (next2 < ntiles) load_b(bnx2, next2, wave);
+            first = false;
             mul_batch(acur, bcur, wave, acc, acci);
             if (next_tile < ntiles) bcur = bnxt;
+            if (next2 < ntiles) bnxt = bnx2;
         } else {
             for (int ks0 = wave; ks0 < steps; ks0 += NW * U) {
                 const int nk = ks0 + NW * U;
@@ -302,10 +320,23 @@ int launch_direct_mt(const DirectArgs& p, hipStream_t stream, const char* name) 
     if (ntiles == 0 || mtiles == 0) return LLMK_OK;
     const size_t smem = (size_t)(MT == 4 ? 1 : 2) * NW * MT * 256 * sizeof(float) + (SCALED ? (size_t)MT * 16 * steps * sizeof(float) : 0);
     if (smem > 64 * 1024) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: K=%d too large for the weight-streaming kernel's scale table", name, p.K);
-    // column tiles are processed persistently: at most ~2 workgroups per CU and m-tile row
-    const int gx = min(ntiles, max(1, 512 / min(mtiles, 512)));
+    // Column tiles are processed persistently by as many workgroups as are resident at once (so that every
+    // workgroup streams tile after tile with its next tiles already requested), split over the m-tile rows.
+    const bool resident = steps <= NW * U;
+    static int slots[2] = {0, 0};             // resident workgroups on the whole device, per kernel variant
+    if (slots[resident] == 0) {
+        int dev = 0, cus = 0, per_cu = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e == hipSuccess)
+            e = resident ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, MT, NW, GROUPED, true>, NW * 64, 64 * 1024)
+                         : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, MT, NW, GROUPED, false>, NW * 64, 64 * 1024);
+        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
+        slots[resident] = max(1, cus * max(1, per_cu));
+    }
+    const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
     dim3 grid((unsigned)gx, (unsigned)mtiles), block(NW * 64);
-    if (steps <= NW * U) gemm_direct_kernel<KIND, MT, NW, GROUPED, true><<<grid, block, smem, stream>>>(p);
+    if (resident) gemm_direct_kernel<KIND, MT, NW, GROUPED, true><<<grid, block, smem, stream>>>(p);
     else gemm_direct_kernel<KIND, MT, NW, GROUPED, false><<<grid, block, smem, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     return LLMK_OK;

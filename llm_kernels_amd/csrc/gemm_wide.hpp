@@ -5,14 +5,15 @@
 //
 // Workgroup: 512 threads = 8 waves, 2 along M x 4 along N; wave tile 128 rows x 64 columns =
 // 8 x 4 MFMA tiles (128 accumulator registers per lane).  Two LDS stages of 66560 bytes
-// (A 32 KB, B 32 KB, activation-scale column 1 KB): the loads of K step kt+1 fly while step kt is
-// multiplied, one barrier per step.
+// (A 32 KB, B 32 KB, activation-scale column 1 KB): the loads of K step kt+2 are issued behind the
+// one barrier of step kt, which sits before its last tile row; they fly while step kt+1 is multiplied.
 //
 // Inside a step a wave keeps its four weight fragments in registers for the whole step and streams
 // the eight activation fragments through a two-deep register buffer.  The product of tile n is
 // scaled and accumulated (VALU) while the MFMAs of the next tile row run, through two register sets
 // of partial products that carry over from one K step to the next.
 #pragma once
+#include <type_traits>
 #include "gemm_dma.hpp"
 
 namespace llmk {
@@ -145,17 +146,22 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     for (int j = 0; j < 4; ++j) t[0][j] = t[1][j] = (v4f){0.f, 0.f, 0.f, 0.f};
     float sprev = 0.f;
 
-    auto step = [&](int kt) {
-        const uint8_t* st = lds + (kt & 1) * W_STAGE;
-        const uint8_t* As = st + (wm * 128) * 128;
-        const uint8_t* Bs = st + W_A + (wn * 64) * 128;
-        v8i bf[4], af[2];
+    // Fragments of the step being multiplied.  bf and af[0] of step kt + 1 are fetched during the last
+    // tile row of step kt, so that a step starts with its operands already in registers.
+    v8i bf[4], af[2];
+    auto stage_a = [&](int kt) { return lds + (kt & 1) * W_STAGE + (wm * 128) * 128; };
+    auto stage_b = [&](int kt) { return lds + (kt & 1) * W_STAGE + W_A + (wn * 64) * 128; };
+
+    // One K step.  SYNC: another step follows; before the last tile row the wave waits for its share of
+    // the next stage and for its own LDS reads, and meets the others at the barrier.  Behind the barrier
+    // the next stage is complete and nobody reads the current one any more, so the loads of step kt + 2
+    // (ISSUE) may overwrite it, and the fragments of step kt + 1 are fetched while row 7 is multiplied.
+    auto step = [&](int kt, auto sync_c, auto issue_c) {
+        constexpr bool SYNC = decltype(sync_c)::value, ISSUE = decltype(issue_c)::value;
+        const uint8_t* As = stage_a(kt);
         float sa[8];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) bf[j] = ldfrag(Bs + j * 2048);
-        af[0] = ldfrag(As);
         if constexpr (SCALED) {
-            const float* Ss = (const float*)(st + W_A + W_B) + wm * 128 + r;
+            const float* Ss = (const float*)(lds + (kt & 1) * W_STAGE + W_A + W_B) + wm * 128 + r;
             const float bs = bsl[(wn >> 1) * D_MAX_KT + kt];
 #pragma unroll
             for (int i = 0; i < 8; ++i) sa[i] = Ss[i * 16] * bs;
@@ -163,6 +169,12 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             if (i < 7) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+            if (i == 7 && SYNC) {
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if constexpr (SCALED) {
@@ -171,6 +183,11 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                     else acc[7][j] += t[1][j] * sprev;
                 } else {
                     acc[i][j] = mma16(bf[j], af[i & 1], acc[i][j]);
+                }
+                if (i == 7 && SYNC) {
+                    if (j == 0 && ISSUE) issue(kt + 2);
+                    bf[j] = ldfrag(stage_b(kt + 1) + j * 2048);
+                    if (j == 3) af[0] = ldfrag(stage_a(kt + 1));
                 }
                 // Nothing moves across a tile boundary: the FMAs retire a product finished four MFMAs
                 // ago, never the one just issued, and each activation fragment is requested a whole
@@ -181,15 +198,18 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         if constexpr (SCALED) sprev = sa[7];
     };
 
-    int kt = 0;
-    for (; kt + 1 < KT; ++kt) {
-        issue(kt + 1);
-        step(kt);
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
-        __syncthreads();
+    if (KT > 1) issue(1);
+    if (KT > 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bf[j] = ldfrag(stage_b(0) + j * 2048);
+        af[0] = ldfrag(stage_a(0));
     }
-    if (kt < KT) step(kt);
+    const std::true_type yes;
+    const std::false_type no;
+    int kt = 0;
+    for (; kt + 2 < KT; ++kt) step(kt, yes, yes);
+    if (kt + 1 < KT) { step(kt, yes, no); ++kt; }
+    if (kt < KT) step(kt, no, no);
     if constexpr (SCALED) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[7][j] += t[1][j] * sprev;
