@@ -21,6 +21,21 @@ __device__ __forceinline__ float ld_scale(const void* p, int64_t i, int dt) {
     return bf16_to_f32(((const unsigned short*)p)[i]);
 }
 
+// raw scale element (fp32 bits or 16-bit pattern) -> fp32; SDT is a dtype code known at compile time
+template <int SDT> struct ScaleIO;
+template <> struct ScaleIO<LLMK_F32> {
+    typedef float Raw;
+    static __device__ __forceinline__ float cvt(Raw v) { return v; }
+};
+template <> struct ScaleIO<LLMK_F16> {
+    typedef unsigned short Raw;
+    static __device__ __forceinline__ float cvt(Raw v) { return f16_to_f32(v); }
+};
+template <> struct ScaleIO<LLMK_BF16> {
+    typedef unsigned short Raw;
+    static __device__ __forceinline__ float cvt(Raw v) { return bf16_to_f32(v); }
+};
+
 __device__ __forceinline__ void st_out(void* p, int64_t i, float v, int dt) {
     if (dt == LLMK_F32) ((float*)p)[i] = v;
     else if (dt == LLMK_F16) ((unsigned short*)p)[i] = f32_to_f16(v);
@@ -79,8 +94,11 @@ struct DirectArgs {
     int M, N, K, E;
 };
 
-template <int KIND, int MT, int NW, bool GROUPED, bool RESIDENT>
+// SDT: dtype code of the block scales, fixed at compile time so that a scale load is a plain typed load with
+// no branch (and hence no wait for memory) between it and the loads around it.
+template <int KIND, int MT, int NW, bool GROUPED, bool RESIDENT, int SDT>
 __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
+    typedef typename ScaleIO<SDT>::Raw SRaw;
     constexpr bool HALF = (KIND == K_F16 || KIND == K_BF16);
     constexpr int ESZ = HALF ? 2 : 1;
     constexpr int KSTEP = 128 / ESZ;          // elements covered by one 128-byte step
@@ -132,7 +150,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
     struct BBatch {
         v8i b[U];
-        float bs[U];
+        SRaw bs[U];           // raw weight scales, converted when the batch is multiplied
     };
     struct ABatch {
         v8i a[U][MT];
@@ -147,16 +165,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         const int nrow = min(tile * 16 + r, N - 1);
         const uint8_t* bp = bbase + ((int64_t)nrow * K) * ESZ + 16 * g;
         const int64_t bs_row = bs_off + (int64_t)(tile * 16 / 128) * steps;
+        // all data loads first, then the scales as raw bits: nothing in here waits for memory
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             bool valid;
             const int ksc = ks_of(ks0, u, valid);
-            t.bs[u] = 1.f;
-            if constexpr (BLOCKSCALE) t.bs[u] = valid ? ld_scale(p.b_s, bs_row + ksc, p.s_dtype) : 0.f;
             t.b[u] = ld_split(bp + (int64_t)ksc * 128);
             if constexpr (!BLOCKSCALE) {
                 if (!valid) t.b[u] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
             }
+        }
+        if constexpr (BLOCKSCALE) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) { bool valid; t.bs[u] = ((const SRaw*)p.b_s)[bs_row + ks_of(ks0, u, valid)]; }
         }
     };
     auto load_a = [&](ABatch& t, int ks0) {
@@ -169,24 +190,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         }
     };
 
-    // activation scales of the tile rows for every K step -> LDS (requested before the first batch so that
-    // the wait for them does not drain the batch behind them)
+    // activation scales of the tile rows for every K step -> LDS table
     constexpr int RB = MT == 4 ? 1 : 2;      // reduction buffers (one needs a second barrier per tile)
     float* asl = red + RB * NW * MT * 256;
     constexpr int SROWS = MT * 16;
-    float stage_as[4];
+    // The scale rows of a tile are contiguous in a_s, so table entry idx is element m_start*steps + idx
+    // (entries of rows past the segment end repeat the last valid element; those rows are never stored).
+    // Requested behind the first weight / activation batch and written once the whole batch has landed.
     const int n_as = BLOCKSCALE ? SROWS * steps : 0;
-    if constexpr (BLOCKSCALE) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int idx = (int)threadIdx.x + q * NW * 64;
-            stage_as[q] = 0.f;
-            if (idx < n_as) {
-                const int rr = idx / steps, kk = idx - rr * steps;
-                stage_as[q] = ld_scale(p.a_s, (int64_t)min(m_start + rr, m_end - 1) * steps + kk, p.s_dtype);
-            }
-        }
-    }
+    const int n_as_valid = (m_end - m_start) * steps;
+    const int64_t as_base = (int64_t)m_start * steps;
     int tile = blockIdx.x;
     ABatch acur, anxt;
     BBatch bcur, bnxt, bnx2;
@@ -196,15 +209,20 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         load_a(acur, wave);
     }
     if constexpr (BLOCKSCALE) {
+        SRaw stage_as[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int idx = (int)threadIdx.x + q * NW * 64;
-            if (idx < n_as) asl[idx] = stage_as[q];
+            stage_as[q] = 0;
+            if (idx < n_as) stage_as[q] = ((const SRaw*)p.a_s)[as_base + min(idx, n_as_valid - 1)];
         }
-        for (int idx = (int)threadIdx.x + 4 * NW * 64; idx < n_as; idx += NW * 64) {   // very long K only
-            const int rr = idx / steps, kk = idx - rr * steps;
-            asl[idx] = ld_scale(p.a_s, (int64_t)min(m_start + rr, m_end - 1) * steps + kk, p.s_dtype);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int idx = (int)threadIdx.x + q * NW * 64;
+            if (idx < n_as) asl[idx] = ScaleIO<SDT>::cvt(stage_as[q]);
         }
+        for (int idx = (int)threadIdx.x + 4 * NW * 64; idx < n_as; idx += NW * 64)   // very long K only
+            asl[idx] = ScaleIO<SDT>::cvt(((const SRaw*)p.a_s)[as_base + min(idx, n_as_valid - 1)]);
         __syncthreads();
     }
 
@@ -219,7 +237,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
                 const v8i a = ta.a[u][mt];
                 if constexpr (BLOCKSCALE) {
                     const v4f t = step_dot<KIND>(a, b);
-                    const float bs = tb.bs[u];
+                    const float bs = valid ? ScaleIO<SDT>::cvt(tb.bs[u]) : 0.f;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const float as = asl[(mt * 16 + 4 * g + i) * steps + ksc];
@@ -308,8 +326,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     }
 }
 
-template <int KIND, int MT, bool GROUPED>
-int launch_direct_mt(const DirectArgs& p, hipStream_t stream, const char* name) {
+template <int KIND, int MT, bool GROUPED, int SDT>
+int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name) {
     constexpr int NW = 8;
     constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
     constexpr bool HALF = (KIND == K_F16 || KIND == K_BF16);
@@ -329,17 +347,33 @@ int launch_direct_mt(const DirectArgs& p, hipStream_t stream, const char* name) 
         hipError_t e = hipGetDevice(&dev);
         if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (e == hipSuccess)
-            e = resident ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, MT, NW, GROUPED, true>, NW * 64, 64 * 1024)
-                         : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, MT, NW, GROUPED, false>, NW * 64, 64 * 1024);
+            e = resident ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, MT, NW, GROUPED, true, SDT>, NW * 64, 64 * 1024)
+                         : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, MT, NW, GROUPED, false, SDT>, NW * 64, 64 * 1024);
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
         slots[resident] = max(1, cus * max(1, per_cu));
     }
     const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
     dim3 grid((unsigned)gx, (unsigned)mtiles), block(NW * 64);
-    if (resident) gemm_direct_kernel<KIND, MT, NW, GROUPED, true><<<grid, block, smem, stream>>>(p);
-    else gemm_direct_kernel<KIND, MT, NW, GROUPED, false><<<grid, block, smem, stream>>>(p);
+    if (resident) gemm_direct_kernel<KIND, MT, NW, GROUPED, true, SDT><<<grid, block, smem, stream>>>(p);
+    else gemm_direct_kernel<KIND, MT, NW, GROUPED, false, SDT><<<grid, block, smem, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     return LLMK_OK;
+}
+
+// the scale dtype only matters for the int8 block kind (fp8 scales are fp32, the other kinds carry none)
+template <int KIND, int MT, bool GROUPED>
+int launch_direct_mt(const DirectArgs& p, hipStream_t stream, const char* name) {
+    if constexpr (KIND == K_I8_BLOCK) {
+        switch (p.s_dtype) {
+            case LLMK_F32:  return launch_direct_sdt<KIND, MT, GROUPED, LLMK_F32>(p, stream, name);
+            case LLMK_F16:  return launch_direct_sdt<KIND, MT, GROUPED, LLMK_F16>(p, stream, name);
+            case LLMK_BF16: return launch_direct_sdt<KIND, MT, GROUPED, LLMK_BF16>(p, stream, name);
+            default: LLMK_FAIL(LLMK_ERR_DTYPE, "%s: s_dtype %d", name, p.s_dtype);
+        }
+    } else {
+        if (KIND == K_FP8_BLOCK && p.s_dtype != LLMK_F32) LLMK_FAIL(LLMK_ERR_DTYPE, "%s: fp8 block scales must be fp32", name);
+        return launch_direct_sdt<KIND, MT, GROUPED, LLMK_F32>(p, stream, name);
+    }
 }
 
 template <int KIND, bool GROUPED>

@@ -21,21 +21,6 @@ constexpr int T_B_BYTES = T_BN * T_ROW;            // 18432
 constexpr int T_STAGE = T_A_BYTES + T_B_BYTES + T_BM * 4;   // + the scale column of this K step
 constexpr int T_LDS = 2 * T_STAGE;                 // 112640 bytes
 
-// raw scale element (fp32 bits or 16-bit pattern) -> fp32; SDT is a dtype code known at compile time
-template <int SDT> struct ScaleIO;
-template <> struct ScaleIO<LLMK_F32> {
-    typedef float Raw;
-    static __device__ __forceinline__ float cvt(Raw v) { return v; }
-};
-template <> struct ScaleIO<LLMK_F16> {
-    typedef unsigned short Raw;
-    static __device__ __forceinline__ float cvt(Raw v) { return f16_to_f32(v); }
-};
-template <> struct ScaleIO<LLMK_BF16> {
-    typedef unsigned short Raw;
-    static __device__ __forceinline__ float cvt(Raw v) { return bf16_to_f32(v); }
-};
-
 template <int KIND, bool GROUPED, int SDT>
 __global__ __launch_bounds__(T_THREADS) void gemm_tiled_kernel(DirectArgs p) {
     typedef typename ScaleIO<SDT>::Raw SRaw;
