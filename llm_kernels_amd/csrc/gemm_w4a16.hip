@@ -84,40 +84,56 @@ __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
 #pragma unroll
     for (int i = 0; i < MT * 32; ++i) acc[i] = 0.f;
 
-    int cur_grp0 = -1, cur_grp1 = -1;
-    v8h s0 = {}, s1 = {};
-#pragma unroll 2
-    for (int ks = ks_begin + wave; ks < ks_end; ks += NW) {
-        const int st0 = 2 * ks, st1 = 2 * ks + 1;
-        const bool have1 = st1 < strips;
-        const int st1c = have1 ? st1 : st0;
-        const v4i w0 = B[((int64_t)st0 * nchunks + chunk) * 32 + 4 * c + g];
-        const v4i w1 = B[((int64_t)st1c * nchunks + chunk) * 32 + 4 * c + g];
-        const int grp0 = (16 * st0) / groupsize, grp1 = (16 * st1c) / groupsize;
-        if (grp0 != cur_grp0) { s0 = *(const v8h*)(S + (int64_t)grp0 * N + 64 * chunk + 8 * c); cur_grp0 = grp0; }
-        if (grp1 != cur_grp1) { s1 = *(const v8h*)(S + (int64_t)grp1 * N + 64 * chunk + 8 * c); cur_grp1 = grp1; }
-
-        v8h a[MT];
+    // Batches of U steps: every load of a batch (weights, scales, activations) is issued before the first
+    // one is used, with clamped indices and no branch in between, so that a batch costs one memory round
+    // trip.  Steps past the end of the range multiply by a zero activation fragment.
+    constexpr int U = MT == 4 ? 1 : 2;
+    const v4i* bptr = B + (int64_t)chunk * 32 + 4 * c + g;
+    const int64_t strip_stride = (int64_t)nchunks * 32;
+    const _Float16* sptr = S + 64 * chunk + 8 * c;
+    for (int ks0 = ks_begin + wave; ks0 < ks_end; ks0 += U * NW) {
+        v4i w0[U], w1[U], x[U][MT];
+        v8h s0[U], s1[U];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const unsigned* ap = (const unsigned*)(arow[mt] + 32 * ks);
-            unsigned x0 = ap[0], x1 = ap[4], x2 = have1 ? ap[8] : 0u, x3 = have1 ? ap[12] : 0u;
-            a[mt] = make8(as_h2(x0), as_h2(x1), as_h2(x2), as_h2(x3));
+        for (int u = 0; u < U; ++u) {
+            const int ks = min(ks0 + u * NW, ks_end - 1);
+            const int st0 = 2 * ks, st1 = min(2 * ks + 1, strips - 1);
+            w0[u] = bptr[st0 * strip_stride];
+            w1[u] = bptr[st1 * strip_stride];
+            s0[u] = *(const v8h*)(sptr + (int64_t)((16 * st0) / groupsize) * N);
+            s1[u] = *(const v8h*)(sptr + (int64_t)((16 * st1) / groupsize) * N);
+            const int o1 = 2 * ks + 1 < strips ? 8 : 0;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const unsigned* ap = (const unsigned*)(arow[mt] + 32 * ks);
+                x[u][mt] = (v4i){(int)ap[0], (int)ap[4], (int)ap[o1], (int)ap[o1 + 4]};
+            }
         }
+        __builtin_amdgcn_sched_barrier(0);       // keep every load above ahead of the first use below
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int u = 0; u < U; ++u) {
+            const int ks = ks0 + u * NW;
+            const bool valid = ks < ks_end, valid1 = valid && 2 * ks + 1 < strips;
+            v8h a[MT];
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const int t = 2 * j + b;
-                const unsigned u0 = ((unsigned)w0[j]) >> (8 * b), u1 = ((unsigned)w1[j]) >> (8 * b);
-                const v2h sc0 = {s0[t], s0[t]}, sc1 = {s1[t], s1[t]};
-                const v8h bf = make8(deq_lo(u0) * sc0, deq_hi(u0) * sc0, deq_lo(u1) * sc1, deq_hi(u1) * sc1);
+            for (int mt = 0; mt < MT; ++mt)
+                a[mt] = make8(as_h2(valid ? (unsigned)x[u][mt][0] : 0u), as_h2(valid ? (unsigned)x[u][mt][1] : 0u),
+                              as_h2(valid1 ? (unsigned)x[u][mt][2] : 0u), as_h2(valid1 ? (unsigned)x[u][mt][3] : 0u));
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    v4f d = {acc[(mt * 8 + t) * 4 + 0], acc[(mt * 8 + t) * 4 + 1], acc[(mt * 8 + t) * 4 + 2], acc[(mt * 8 + t) * 4 + 3]};
-                    d = mfma_f16_16x16x32(a[mt], bf, d);
-                    acc[(mt * 8 + t) * 4 + 0] = d[0]; acc[(mt * 8 + t) * 4 + 1] = d[1];
-                    acc[(mt * 8 + t) * 4 + 2] = d[2]; acc[(mt * 8 + t) * 4 + 3] = d[3];
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    const int t = 2 * j + b;
+                    const unsigned u0 = ((unsigned)w0[u][j]) >> (8 * b), u1 = ((unsigned)w1[u][j]) >> (8 * b);
+                    const v2h sc0 = {s0[u][t], s0[u][t]}, sc1 = {s1[u][t], s1[u][t]};
+                    const v8h bf = make8(deq_lo(u0) * sc0, deq_hi(u0) * sc0, deq_lo(u1) * sc1, deq_hi(u1) * sc1);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        v4f d = {acc[(mt * 8 + t) * 4 + 0], acc[(mt * 8 + t) * 4 + 1], acc[(mt * 8 + t) * 4 + 2], acc[(mt * 8 + t) * 4 + 3]};
+                        d = mfma_f16_16x16x32(a[mt], bf, d);
+                        acc[(mt * 8 + t) * 4 + 0] = d[0]; acc[(mt * 8 + t) * 4 + 1] = d[1];
+                        acc[(mt * 8 + t) * 4 + 2] = d[2]; acc[(mt * 8 + t) * 4 + 3] = d[3];
+                    }
                 }
             }
         }
