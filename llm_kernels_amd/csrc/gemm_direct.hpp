@@ -203,7 +203,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     int tile = blockIdx.x;
     ABatch acur, anxt;
     BBatch bcur, bnxt, bnx2;
-    bool first = true;
     if (steps > 0 && tile < ntiles) {
         load_b(bcur, tile, wave);
         load_a(acur, wave);
@@ -265,36 +264,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         }
     };
 
+    // cross-wave reduction of the K split and store of one finished tile (alternating buffers: one barrier
+    // per tile); integer accumulators travel as raw bits
     int parity = 0;
-    for (; tile < ntiles; tile += gridDim.x, parity ^= 1) {
-        v4f acc[MT];
-        v4i acci[MT];
+    v4f acc[MT];
+    v4i acci[MT];
+    auto clear_acc = [&]() {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) { acc[mt] = (v4f){0.f, 0.f, 0.f, 0.f}; acci[mt] = (v4i){0, 0, 0, 0}; }
-        const int next_tile = tile + gridDim.x;
-        if constexpr (RESIDENT) {
-            // two column tiles ahead: bnxt was requested while the previous tile was multiplied
-            const int next2 = next_tile + gridDim.x;
-            if (first && next_tile < ntiles) load_b(bnxt, next_tile, wave);
-            if (next2 < ntiles) load_b(bnx2, next2, wave);
-            first = false;
-            mul_batch(acur, bcur, wave, acc, acci);
-            if (next_tile < ntiles) bcur = bnxt;
-            if (next2 < ntiles) bnxt = bnx2;
-        } else {
-            for (int ks0 = wave; ks0 < steps; ks0 += NW * U) {
-                const int nk = ks0 + NW * U;
-                const bool more = nk < steps;
-                if (more) { load_b(bnxt, tile, nk); load_a(anxt, nk); }
-                else if (next_tile < ntiles) { load_b(bnxt, next_tile, wave); load_a(anxt, wave); }
-                mul_batch(acur, bcur, ks0, acc, acci);
-                if (more || next_tile < ntiles) { bcur = bnxt; acur = anxt; }
-            }
-        }
-
-        // cross-wave reduction of the K split (two alternating buffers: one barrier per tile);
-        // integer accumulators travel as raw bits
+    };
+    auto finish = [&](int tl) __attribute__((always_inline)) {
         float* rbuf = red + (RB == 2 ? parity : 0) * NW * MT * 256;
+        parity ^= 1;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             float* dst = rbuf + ((wave * MT + mt) * 64 + lane) * 4;
@@ -303,26 +284,70 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
                 dst[i] = (KIND == K_I8_ROWCOL) ? __int_as_float(acci[mt][i]) : acc[mt][i];
         }
         __syncthreads();
-        const int n0 = tile * 16;
+        const int n0 = tl * 16;
         for (int o = threadIdx.x; o < MT * 256; o += NW * 64) {
             const int mt = o >> 8, row16 = (o & 255) >> 4, col = o & 15;
             const int src = (mt * 64 + (row16 >> 2) * 16 + col) * 4 + (row16 & 3);
             const int m = m_start + 16 * mt + row16, n = n0 + col;
             if (m >= m_end || n >= N) continue;
             if constexpr (KIND == K_I8_ROWCOL) {
-                int s = 0;
+                int sum = 0;
 #pragma unroll
-                for (int w = 0; w < NW; ++w) s += __float_as_int(rbuf[w * MT * 256 + src]);
-                if (p.c_i32) p.c_i32[(int64_t)m * N + n] = s;
-                if (p.c) st_out(p.c, (int64_t)m * N + n, (float)s * ((const float*)p.a_s)[m] * ((const float*)p.b_s)[n], p.c_dtype);
+                for (int w = 0; w < NW; ++w) sum += __float_as_int(rbuf[w * MT * 256 + src]);
+                if (p.c_i32) p.c_i32[(int64_t)m * N + n] = sum;
+                if (p.c) st_out(p.c, (int64_t)m * N + n, (float)sum * ((const float*)p.a_s)[m] * ((const float*)p.b_s)[n], p.c_dtype);
             } else {
-                float s = 0.f;
+                float sum = 0.f;
 #pragma unroll
-                for (int w = 0; w < NW; ++w) s += rbuf[w * MT * 256 + src];
-                st_out(p.c, (int64_t)m * N + n, s, p.c_dtype);
+                for (int w = 0; w < NW; ++w) sum += rbuf[w * MT * 256 + src];
+                st_out(p.c, (int64_t)m * N + n, sum, p.c_dtype);
             }
         }
         if constexpr (RB == 1) __syncthreads();
+        clear_acc();
+    };
+    clear_acc();
+    const int stride = gridDim.x;
+
+    // The batches form a ring that is never copied: a register copy of a batch whose loads are still in
+    // flight would have to wait for them, which would undo the look-ahead.
+    if constexpr (RESIDENT) {
+        // bcur holds `tile`, bnxt is loaded here with the next tile, bnx2 inside the loop with the one after
+        if (tile + stride < ntiles) load_b(bnxt, tile + stride, wave);
+        auto one = [&](BBatch& cur, BBatch& fill) __attribute__((always_inline)) {
+            const int t2 = tile + 2 * stride;
+            if (t2 < ntiles) load_b(fill, t2, wave);
+            mul_batch(acur, cur, wave, acc, acci);
+            finish(tile);
+            tile += stride;
+        };
+        while (tile < ntiles) {
+            one(bcur, bnx2);
+            if (tile >= ntiles) break;
+            one(bnxt, bcur);
+            if (tile >= ntiles) break;
+            one(bnx2, bnxt);
+        }
+    } else {
+        // flattened sequence of (tile, K batch) positions, two batch pairs in ping-pong
+        int ks0 = wave;
+        auto one = [&](ABatch& ca, BBatch& cb, ABatch& fa, BBatch& fb) __attribute__((always_inline)) {
+            const int nk = ks0 + NW * U;
+            const bool more = nk < steps;
+            const int nt = more ? tile : tile + stride;
+            const bool any = nt < ntiles;
+            const int fk = more ? nk : wave;
+            if (any) { load_b(fb, nt, fk); load_a(fa, fk); }
+            mul_batch(ca, cb, ks0, acc, acci);
+            if (!more) finish(tile);
+            tile = nt;
+            ks0 = more ? nk : wave;
+        };
+        while (tile < ntiles) {
+            one(acur, bcur, anxt, bnxt);
+            if (tile >= ntiles) break;
+            one(anxt, bnxt, acur, bcur);
+        }
     }
 }
 

@@ -265,6 +265,214 @@ __global__ __launch_bounds__(NW * 64) void w4a16_nk_kernel(
         }
 }
 
+// Weight-streaming variant of the [N, K/8] kernel for groupsize % 128 == 0 (every 128-K step lies in one
+// scale group): persistent workgroups of 8 waves walk 16-column tiles; the waves split K by interleaved
+// 128-K steps in batches of U, all loads of a batch issued before its first use and the weights of the next
+// two tiles requested ahead.  When a wave's K share fits one batch (RESIDENT) its activation fragments are
+// loaded and permuted once and stay in registers for every tile.  The group scale multiplies the fp32
+// partial of the step (one FMA per output) instead of the eight fp16 weights.
+template <int MT, int NT, bool RESIDENT>
+__global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
+    const _Float16* __restrict__ A, const int32_t* __restrict__ B, const _Float16* __restrict__ S,
+    _Float16* __restrict__ C, int M, int N, int K, int groupsize) {
+    constexpr int NW = 8;
+    constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+    extern __shared__ float red[];                       // [2][NW][NT][MT][64][4]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int steps = K >> 7, ngroups = K / groupsize, kwords = K >> 3;
+    const int m0 = blockIdx.y * 16 * MT;
+    const int ntiles = (N + 16 * NT - 1) / (16 * NT);    // a tile is NT adjacent 16-column blocks
+
+    const _Float16* arow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (int64_t)min(m0 + 16 * mt + r, M - 1) * K + 32 * g;
+
+    struct BBatch {
+        v4i w[NT][U];
+        unsigned short s[NT][U];
+    };
+    struct ABatch {
+        v4i a[U][MT][4];
+    };
+    auto clamp_step = [&](int ks) { return min(ks, steps - 1); };
+    auto load_b = [&](BBatch& t, int tile, int ks0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int nrow = min((tile * NT + nt) * 16 + r, N - 1);
+            const int32_t* brow = B + (int64_t)nrow * kwords + 4 * g;
+#pragma unroll
+            for (int u = 0; u < U; ++u) t.w[nt][u] = *(const v4i*)(brow + clamp_step(ks0 + u * NW) * 16);
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int nrow = min((tile * NT + nt) * 16 + r, N - 1);
+            const unsigned short* srow = (const unsigned short*)S + (int64_t)nrow * ngroups;
+#pragma unroll
+            for (int u = 0; u < U; ++u) t.s[nt][u] = srow[(clamp_step(ks0 + u * NW) * 128) / groupsize];
+        }
+    };
+    auto load_a = [&](ABatch& t, int ks0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) t.a[u][mt][j] = *(const v4i*)(arow[mt] + clamp_step(ks0 + u * NW) * 128 + 8 * j);
+    };
+    // k order of a dequantised word is [0,4,1,5,2,6,3,7]: bring the activation fragment into the same order
+    auto perm_a = [&](ABatch& t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const v4i x = t.a[u][mt][j];
+                    v4i y;
+                    y[0] = (int)__builtin_amdgcn_perm((unsigned)x[2], (unsigned)x[0], 0x05040100u);
+                    y[1] = (int)__builtin_amdgcn_perm((unsigned)x[2], (unsigned)x[0], 0x07060302u);
+                    y[2] = (int)__builtin_amdgcn_perm((unsigned)x[3], (unsigned)x[1], 0x05040100u);
+                    y[3] = (int)__builtin_amdgcn_perm((unsigned)x[3], (unsigned)x[1], 0x07060302u);
+                    t.a[u][mt][j] = y;
+                }
+    };
+    auto mul = [&](const ABatch& ta, const BBatch& tb, int ks0, v4f (&acc)[NT][MT]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool valid = ks0 + u * NW < steps;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float sc = valid ? f16_to_f32(tb.s[nt][u]) : 0.f;
+                v4f t[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) t[mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const unsigned w = (unsigned)tb.w[nt][u][j], w8 = w >> 8;
+                    const v8h bf = make8(deq_lo(w), deq_hi(w), deq_lo(w8), deq_hi(w8));
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        v8h a;
+                        __builtin_memcpy(&a, &ta.a[u][mt][j], 16);
+                        t[mt] = mfma_f16_16x16x32(a, bf, t[mt]);
+                    }
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += t[mt] * sc;
+            }
+        }
+    };
+
+    int tile = blockIdx.x;
+    const int stride = gridDim.x;
+    ABatch acur, anxt;
+    BBatch bcur, bnxt, bnx2;
+    if (tile < ntiles) {
+        load_b(bcur, tile, wave);
+        load_a(acur, wave);
+        if (RESIDENT && tile + stride < ntiles) load_b(bnxt, tile + stride, wave);
+        __builtin_amdgcn_sched_barrier(0);
+        if (RESIDENT) perm_a(acur);
+    }
+    constexpr int NB = NT * MT;                          // 16x16 blocks per tile
+    int parity = 0;
+    v4f acc[NT][MT];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+    };
+    // cross-wave reduction of the K split, two alternating buffers: one barrier per tile
+    auto finish = [&](int tl) __attribute__((always_inline)) {
+        float* rbuf = red + parity * NW * NB * 256;
+        parity ^= 1;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) *(v4f*)(rbuf + ((wave * NB + nt * MT + mt) * 64 + lane) * 4) = acc[nt][mt];
+        __syncthreads();
+        for (int o = threadIdx.x; o < NB * 256; o += NW * 64) {
+            const int blk = o >> 8, nt = blk / MT, mt = blk - nt * MT, row16 = (o & 255) >> 4, col = o & 15;
+            const int src = (blk * 64 + (row16 >> 2) * 16 + col) * 4 + (row16 & 3);
+            const int m = m0 + 16 * mt + row16, n = (tl * NT + nt) * 16 + col;
+            if (m >= M || n >= N) continue;
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) v += rbuf[w * NB * 256 + src];
+            C[(int64_t)m * N + n] = (_Float16)v;
+        }
+        clear_acc();
+    };
+    clear_acc();
+    // The batches form a ring that is never copied (a register copy of a batch whose loads are in flight
+    // would wait for them).
+    if constexpr (RESIDENT) {
+        auto one = [&](BBatch& cur, BBatch& fill) __attribute__((always_inline)) {
+            const int t2 = tile + 2 * stride;
+            if (t2 < ntiles) load_b(fill, t2, wave);
+            mul(acur, cur, wave, acc);
+            finish(tile);
+            tile += stride;
+        };
+        while (tile < ntiles) {
+            one(bcur, bnx2);
+            if (tile >= ntiles) break;
+            one(bnxt, bcur);
+            if (tile >= ntiles) break;
+            one(bnx2, bnxt);
+        }
+    } else {
+        int ks0 = wave;
+        auto one = [&](ABatch& ca, BBatch& cb, ABatch& fa, BBatch& fb) __attribute__((always_inline)) {
+            const int nk = ks0 + NW * U;
+            const bool more = nk < steps;
+            const int nt = more ? tile : tile + stride;
+            const bool any = nt < ntiles;
+            const int fk = more ? nk : wave;
+            if (any) { load_b(fb, nt, fk); load_a(fa, fk); }
+            perm_a(ca);                                  // permuted when it becomes current, not while in flight
+            mul(ca, cb, ks0, acc);
+            if (!more) finish(tile);
+            tile = nt;
+            ks0 = more ? nk : wave;
+        };
+        while (tile < ntiles) {
+            one(acur, bcur, anxt, bnxt);
+            if (tile >= ntiles) break;
+            one(anxt, bnxt, acur, bcur);
+        }
+    }
+}
+
+template <int MT, int NT>
+int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Float16* C, int M, int N, int K, int groupsize,
+                     hipStream_t st) {
+    constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
+    const int steps = K >> 7, ntiles = (N + 16 * NT - 1) / (16 * NT), mtiles = (M + 16 * MT - 1) / (16 * MT);
+    const bool resident = steps <= 8 * U;
+    const size_t smem = (size_t)2 * 8 * NT * MT * 256 * sizeof(float);
+    static int slots[2] = {0, 0};
+    if (slots[resident] == 0) {
+        int dev = 0, cus = 0, per_cu = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e == hipSuccess)
+            e = resident ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, w4a16_nk_stream_kernel<MT, NT, true>, 512, smem)
+                         : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, w4a16_nk_stream_kernel<MT, NT, false>, 512, smem);
+        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a16_nk: occupancy query failed: %s", hipGetErrorString(e));
+        slots[resident] = max(1, cus * max(1, per_cu));
+    }
+    const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
+    dim3 grid((unsigned)gx, (unsigned)mtiles);
+    if (resident) w4a16_nk_stream_kernel<MT, NT, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
+    else w4a16_nk_stream_kernel<MT, NT, false><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
+    LLMK_CHECK_LAUNCH("gemm_w4a16_nk(stream)");
+    return LLMK_OK;
+}
+
 // launch shape of the Marlin-layout kernel for a given problem
 struct MarlinPlan {
     int mt, nw, mblocks, col_groups, z, steps_per_z;
@@ -371,6 +579,12 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
     const _Float16* A = (const _Float16*)a;
     const _Float16* S = (const _Float16*)s;
     _Float16* C = (_Float16*)c;
+    if (groupsize % 128 == 0 && M <= 64) {
+        // one 16-column block per tile: two blocks per tile (NT = 2) measured slower at every shape tried
+        if (M <= 16) return launch_nk_stream<1, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
+        if (M <= 32) return launch_nk_stream<2, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
+        return launch_nk_stream<4, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
+    }
     const unsigned gx = (unsigned)cdiv64(N, 16);
     if (M <= 16) {
         constexpr int NW = 8;
