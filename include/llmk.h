@@ -155,6 +155,20 @@ int llmk_moe_act_and_mul(const void* gateup, int in_dtype, void* out, int out_dt
                          const void* reorder_topk_ids, int ids_bytes, const float* scales,
                          int start_expert, int end_expert, int64_t M, int64_t two_i, int act,
                          void* stream);
+/* Fused variants (the reference marks them as TODO: moe/sglang_moe_all_gather_all_reduce.py:295-296,365,
+ * 407-408): the gated activation, resp. the token permutation, followed by the 1 x 128 activation quantizer
+ * of the grouped GEMM in one pass.  kind: LLMK_KIND_FP8 (q e4m3, s fp32) or LLMK_KIND_I8 (q int8, s fp16,
+ * round_mode as in llmk_act_quant_i8).  q_out [M, I] resp. [T*topk, hidden]; s_out one scale per 128
+ * elements of a row.  Results equal llmk_moe_act_and_mul / llmk_moe_pre_reorder followed by
+ * llmk_act_quant_fp8 / _i8 bit for bit.  fp16 / bf16 inputs; I resp. hidden a multiple of 128. */
+int llmk_moe_act_and_mul_quant(const void* gateup, int in_dtype, void* q_out, void* s_out, int kind,
+                               int round_mode, const void* reorder_topk_ids, int ids_bytes,
+                               const float* scales, int start_expert, int end_expert, int64_t M,
+                               int64_t two_i, int act, void* stream);
+int llmk_moe_pre_reorder_quant(const void* x, int x_dtype, void* q_out, void* s_out, int kind,
+                               int round_mode, const int32_t* src2dst, const void* topk_ids,
+                               int ids_bytes, const float* a1_scales, int start_expert, int end_expert,
+                               int topk, int64_t T, int64_t hidden, void* stream);
 /* w_dtype: dtype code of topk_weights. */
 int llmk_moe_post_reorder(const void* down_out, void* out, int dtype, const int32_t* src2dst,
                           const void* topk_ids, int ids_bytes, const void* topk_weights, int w_dtype,

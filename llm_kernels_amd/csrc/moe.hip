@@ -1,6 +1,7 @@
 // Single-GPU expert-parallel MoE path: segment bookkeeping, token permute / un-permute,
 // gated activation, and the grouped GEMM over one GPU's experts.
 #include "gemm_wide.hpp"
+#include "quant_util.hpp"
 
 using namespace llmk;
 
@@ -52,6 +53,24 @@ template <int DT> __device__ __forceinline__ float rnd(float v) {
     else return v;
 }
 
+// gated activation of one element with the reference's rounding points (activation in fp32, rounded to the
+// tensor dtype, product in the tensor dtype, optional per-expert scale in the tensor dtype)
+template <int IDT>
+__device__ __forceinline__ float gated_act(float gv, float up, int act, bool has_scale, float scale) {
+    if (act == 0) {
+        gv = gv * (1.0f / (1.0f + expf(-gv)));
+    } else {
+        const float kAlpha = 0.7978845608028654f;
+        const float u = kAlpha * (gv + 0.044715f * gv * gv * gv);
+        const float th = 2.0f * (1.0f / (1.0f + expf(-2.0f * u))) - 1.0f;
+        gv = 0.5f * gv * (1.0f + th);
+    }
+    gv = rnd<IDT>(gv);
+    float r = rnd<IDT>(gv * up);
+    if (has_scale) r = rnd<IDT>(r * scale);
+    return r;
+}
+
 template <int IDT, int ODT>
 __global__ void act_and_mul_kernel(const void* __restrict__ gateup, void* __restrict__ out,
                                    const void* __restrict__ reorder_topk_ids, int ids_bytes,
@@ -63,20 +82,76 @@ __global__ void act_and_mul_kernel(const void* __restrict__ gateup, void* __rest
     const bool has_scale = scales != nullptr;
     const float scale = has_scale ? rnd<IDT>(1.0f / scales[e - start_e]) : 1.0f;
     for (int64_t c = threadIdx.x; c < I; c += blockDim.x) {
-        float gv = FloatIO<IDT>::ld(gateup, row * two_i + c);
+        const float gv = FloatIO<IDT>::ld(gateup, row * two_i + c);
         const float up = FloatIO<IDT>::ld(gateup, row * two_i + I + c);
-        if (act == 0) {
-            gv = gv * (1.0f / (1.0f + expf(-gv)));
-        } else {
-            const float kAlpha = 0.7978845608028654f;
-            const float u = kAlpha * (gv + 0.044715f * gv * gv * gv);
-            const float th = 2.0f * (1.0f / (1.0f + expf(-2.0f * u))) - 1.0f;
-            gv = 0.5f * gv * (1.0f + th);
-        }
-        gv = rnd<IDT>(gv);
-        float r = rnd<IDT>(gv * up);
-        if (has_scale) r = rnd<IDT>(r * scale);
+        const float r = gated_act<IDT>(gv, up, act, has_scale, scale);
         FloatIO<ODT>::st(out, row * I + c, r);
+    }
+}
+
+// Gated activation and 1 x 128 activation quantisation in one pass: 16 lanes own one group of 128 outputs,
+// 8 each.  The values quantised are exactly those the separate activation kernel would have stored in the
+// tensor dtype, so q and s equal those of the two-kernel sequence bit for bit.
+template <int IDT, bool FP8>
+__global__ void act_mul_quant_kernel(const void* __restrict__ gateup, void* __restrict__ q_out, void* __restrict__ s_out,
+                                     const void* __restrict__ reorder_topk_ids, int ids_bytes,
+                                     const float* __restrict__ scales, int start_e, int end_e, int64_t M, int64_t two_i,
+                                     int act, int mode) {
+    const int64_t I = two_i / 2, gpr = I / 128;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t grp = tid >> 4;
+    const bool live = grp < M * gpr;
+    const int64_t gs = live ? grp : 0;
+    const int64_t row = gs / gpr, col = (gs - row * gpr) * 128 + (tid & 15) * EPL;
+    const int64_t e = ld_id(reorder_topk_ids, row, ids_bytes);
+    const bool local = e >= start_e && e <= end_e;
+    const bool has_scale = scales != nullptr && local;
+    const float scale = has_scale ? rnd<IDT>(1.0f / scales[e - start_e]) : 1.0f;
+    float gv[EPL], up[EPL], r[EPL];
+    load8<IDT>(gateup, row * two_i + col, gv);
+    load8<IDT>(gateup, row * two_i + I + col, up);
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+        r[j] = gated_act<IDT>(gv[j], up[j], act, has_scale, scale);
+        m = fmaxf(m, fabsf(r[j]));
+    }
+    m = group_max<16>(m);
+    if (!live || !local) return;
+    quant_store8<FP8>(r, m, q_out, row * I + col, s_out, grp, (tid & 15) == 0, mode);
+}
+
+// Token permutation and 1 x 128 activation quantisation in one pass: a token's row is read once, quantised
+// (after the optional per-expert scale, rounded to the tensor dtype as the separate kernels do) and written
+// to the destination row of each of its local experts.
+template <int IDT, bool FP8>
+__global__ void pre_reorder_quant_kernel(const void* __restrict__ x, void* __restrict__ q_out, void* __restrict__ s_out,
+                                         const int32_t* __restrict__ src2dst, const void* __restrict__ topk_ids,
+                                         int ids_bytes, const float* __restrict__ a1_scales, int start_e, int end_e,
+                                         int topk, int64_t T, int64_t hidden, int mode) {
+    const int64_t gpr = hidden / 128;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t grp = tid >> 4;
+    const bool live = grp < T * gpr;
+    const int64_t gs = live ? grp : 0;
+    const int64_t t = gs / gpr, gi = gs - t * gpr, col = gi * 128 + (tid & 15) * EPL;
+    float v[EPL];
+    load8<IDT>(x, t * hidden + col, v);
+    for (int j = 0; j < topk; ++j) {
+        const int64_t e = ld_id(topk_ids, t * topk + j, ids_bytes);
+        const bool local = e >= start_e && e <= end_e;
+        const float scale = (a1_scales && local) ? 1.0f / a1_scales[e - start_e] : 1.0f;
+        float w[EPL];
+        float m = 0.f;
+#pragma unroll
+        for (int k = 0; k < EPL; ++k) {
+            w[k] = rnd<IDT>(v[k] * scale);
+            m = fmaxf(m, fabsf(w[k]));
+        }
+        m = group_max<16>(m);
+        if (!live || !local) continue;
+        const int64_t dst = src2dst[t * topk + j];
+        quant_store8<FP8>(w, m, q_out, dst * hidden + col, s_out, dst * gpr + gi, (tid & 15) == 0, mode);
     }
 }
 
@@ -144,6 +219,51 @@ extern "C" int llmk_moe_act_and_mul(const void* gateup, int in_dtype, void* out,
     LLMK_DISPATCH_FLOAT(in_dtype, IDT, LLMK_DISPATCH_FLOAT(out_dtype, ODT,
         (act_and_mul_kernel<IDT, ODT><<<(unsigned)M, 256, 0, (hipStream_t)stream>>>(gateup, out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, two_i, act))));
     LLMK_CHECK_LAUNCH("moe_act_and_mul");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_moe_act_and_mul_quant(const void* gateup, int in_dtype, void* q_out, void* s_out, int kind,
+                                          int round_mode, const void* reorder_topk_ids, int ids_bytes,
+                                          const float* scales, int start_expert, int end_expert, int64_t M,
+                                          int64_t two_i, int act, void* stream) {
+    if (M < 0 || two_i < 0 || two_i % 256) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_act_and_mul_quant: 2I=%lld must be a multiple of 256", (long long)two_i);
+    if (ids_bytes != 4 && ids_bytes != 8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul_quant: ids_bytes %d", ids_bytes);
+    if (act != 0 && act != 1) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul_quant: act %d", act);
+    if (kind != LLMK_KIND_I8 && kind != LLMK_KIND_FP8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul_quant: kind %d", kind);
+    if (round_mode != LLMK_ROUND_HALF_AWAY && round_mode != LLMK_ROUND_HALF_UP) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul_quant: round_mode %d", round_mode);
+    if (in_dtype == LLMK_F32) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul_quant: fp16 / bf16 inputs only");
+    if (M == 0 || two_i == 0) return LLMK_OK;
+    if (!gateup || !q_out || !s_out || !reorder_topk_ids) LLMK_FAIL(LLMK_ERR_ARG, "moe_act_and_mul_quant: null pointer");
+    if (((uintptr_t)gateup | (uintptr_t)q_out) & 15) LLMK_FAIL(LLMK_ERR_ARG, "moe_act_and_mul_quant: buffers must be 16-byte aligned");
+    const int64_t threads = M * (two_i / 256) * 16;
+    const unsigned grid = (unsigned)cdiv64(threads, 256);
+    LLMK_DISPATCH_FLOAT(in_dtype, IDT, {
+        if (kind == LLMK_KIND_FP8) act_mul_quant_kernel<IDT, true><<<grid, 256, 0, (hipStream_t)stream>>>(gateup, q_out, s_out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, M, two_i, act, round_mode);
+        else act_mul_quant_kernel<IDT, false><<<grid, 256, 0, (hipStream_t)stream>>>(gateup, q_out, s_out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, M, two_i, act, round_mode);
+    });
+    LLMK_CHECK_LAUNCH("moe_act_and_mul_quant");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_moe_pre_reorder_quant(const void* x, int x_dtype, void* q_out, void* s_out, int kind, int round_mode,
+                                          const int32_t* src2dst, const void* topk_ids, int ids_bytes,
+                                          const float* a1_scales, int start_expert, int end_expert, int topk,
+                                          int64_t T, int64_t hidden, void* stream) {
+    if (T < 0 || hidden < 0 || topk < 0 || hidden % 128) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_pre_reorder_quant: hidden=%lld must be a multiple of 128", (long long)hidden);
+    if (ids_bytes != 4 && ids_bytes != 8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_pre_reorder_quant: ids_bytes %d", ids_bytes);
+    if (kind != LLMK_KIND_I8 && kind != LLMK_KIND_FP8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_pre_reorder_quant: kind %d", kind);
+    if (round_mode != LLMK_ROUND_HALF_AWAY && round_mode != LLMK_ROUND_HALF_UP) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_pre_reorder_quant: round_mode %d", round_mode);
+    if (x_dtype == LLMK_F32) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_pre_reorder_quant: fp16 / bf16 inputs only");
+    if (T == 0 || hidden == 0 || topk == 0) return LLMK_OK;
+    if (!x || !q_out || !s_out || !src2dst || !topk_ids) LLMK_FAIL(LLMK_ERR_ARG, "moe_pre_reorder_quant: null pointer");
+    if (((uintptr_t)x | (uintptr_t)q_out) & 15) LLMK_FAIL(LLMK_ERR_ARG, "moe_pre_reorder_quant: buffers must be 16-byte aligned");
+    const int64_t threads = T * (hidden / 128) * 16;
+    const unsigned grid = (unsigned)cdiv64(threads, 256);
+    LLMK_DISPATCH_FLOAT(x_dtype, IDT, {
+        if (kind == LLMK_KIND_FP8) pre_reorder_quant_kernel<IDT, true><<<grid, 256, 0, (hipStream_t)stream>>>(x, q_out, s_out, src2dst, topk_ids, ids_bytes, a1_scales, start_expert, end_expert, topk, T, hidden, round_mode);
+        else pre_reorder_quant_kernel<IDT, false><<<grid, 256, 0, (hipStream_t)stream>>>(x, q_out, s_out, src2dst, topk_ids, ids_bytes, a1_scales, start_expert, end_expert, topk, T, hidden, round_mode);
+    });
+    LLMK_CHECK_LAUNCH("moe_pre_reorder_quant");
     return LLMK_OK;
 }
 

@@ -2,56 +2,9 @@
 //
 // Arithmetic follows the reference kernels exactly: fp32 math, IEEE division by the
 // un-rounded fp32 scale, then the scale is stored in its (possibly narrower) type.
-#include "common.hpp"
+#include "quant_util.hpp"
 
 namespace {
-
-constexpr int EPL = 8;   // elements per lane in the 1 x block kernels
-
-template <int DT>
-__device__ __forceinline__ void load8(const void* p, int64_t i, float (&v)[EPL]) {
-    if constexpr (DT == LLMK_F32) {
-        const float4* q = (const float4*)((const float*)p + i);
-        float4 a = q[0], b = q[1];
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    } else {
-        uint4 u = *(const uint4*)((const unsigned short*)p + i);
-        unsigned w[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            unsigned short lo = (unsigned short)(w[j] & 0xffff), hi = (unsigned short)(w[j] >> 16);
-            v[2 * j]     = (DT == LLMK_F16) ? f16_to_f32(lo) : bf16_to_f32(lo);
-            v[2 * j + 1] = (DT == LLMK_F16) ? f16_to_f32(hi) : bf16_to_f32(hi);
-        }
-    }
-}
-
-__device__ __forceinline__ float round_mode(float v, int mode) {
-    // half-away: roundf is exact; half-up: floor(v + 0.5f) with the fp32 add as the reference states it
-    return mode == LLMK_ROUND_HALF_AWAY ? roundf(v) : floorf(v + 0.5f);
-}
-
-__device__ __forceinline__ unsigned pack_fp8x4(float a, float b, float c, float d) {
-    // saturate finite values to +-448 (comparisons leave NaN untouched), then RNE hardware convert
-    auto sat = [](float x) { return x > 448.f ? 448.f : (x < -448.f ? -448.f : x); };
-    int w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(a), sat(b), 0, false);
-    w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(c), sat(d), w, true);
-    return (unsigned)w;
-}
-
-// group max over the LPG lanes that share a group (LPG power of two <= 64)
-template <int LPG>
-__device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-    for (int o = LPG / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-template <int LPG>
-__device__ __forceinline__ float group_min(float v) {
-#pragma unroll
-    for (int o = LPG / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
-    return v;
-}
 
 // ---------------------------------------------------------------- 1 x block activation quant
 // LPG lanes cooperate on one group of LPG*8 contiguous elements.
@@ -70,27 +23,7 @@ __global__ void act_quant_kernel(const void* __restrict__ x, void* __restrict__ 
     for (int j = 0; j < EPL; ++j) m = fmaxf(m, fabsf(v[j]));
     m = group_max<LPG>(m);
     if (!live) return;
-    if constexpr (FP8) {
-        const float sc = m / 448.f;
-        float q[EPL];
-#pragma unroll
-        for (int j = 0; j < EPL; ++j) q[j] = v[j] / sc;
-        uint2 o;
-        o.x = pack_fp8x4(q[0], q[1], q[2], q[3]);
-        o.y = pack_fp8x4(q[4], q[5], q[6], q[7]);
-        *(uint2*)((uint8_t*)y + off) = o;
-        if (tid % LPG == 0) ((float*)s)[grp] = sc;
-    } else {
-        const float sc = m / 127.f;
-        unsigned w[2] = {0, 0};
-#pragma unroll
-        for (int j = 0; j < EPL; ++j) {
-            int qi = (int)round_mode(v[j] / sc, mode);
-            w[j >> 2] |= ((unsigned)(qi & 0xff)) << (8 * (j & 3));
-        }
-        *(uint2*)((int8_t*)y + off) = make_uint2(w[0], w[1]);
-        if (tid % LPG == 0) ((unsigned short*)s)[grp] = f32_to_f16(sc);
-    }
+    quant_store8<FP8>(v, m, y, off, s, grp, tid % LPG == 0, mode);
 }
 
 // ---------------------------------------------------------------- block x block weight quant

@@ -9,7 +9,7 @@ from typing import List, Optional
 import torch
 
 from .group_gemm_kernel import (grouped_gemm_triton, post_reorder, pre_reorder, run_moe_ep_preproess,
-                                silu_and_mul, gelu_and_mul)
+                                silu_and_mul, gelu_and_mul, pre_reorder_quant, act_and_mul_quant)
 
 
 def softmax_topk_router(router_logits: torch.Tensor, top_k: int = 2, renormalize: bool = True):
@@ -24,8 +24,12 @@ def ep_moe_forward(hidden_states: torch.Tensor, topk_ids: torch.Tensor, topk_wei
                    w13_weight: torch.Tensor, w2_weight: torch.Tensor,
                    w13_weight_scale: Optional[torch.Tensor] = None, w2_weight_scale: Optional[torch.Tensor] = None,
                    block_shape: Optional[List[int]] = None, activation: str = "silu",
-                   start_expert_id: int = 0, end_expert_id: Optional[int] = None):
-    """hidden_states [T, H]; w13 [E, 2I, H] (gate rows first, then up), w2 [E, H, I]. Returns [T, H]."""
+                   start_expert_id: int = 0, end_expert_id: Optional[int] = None, fuse_quant: bool = True):
+    """hidden_states [T, H]; w13 [E, 2I, H] (gate rows first, then up), w2 [E, H, I]. Returns [T, H].
+
+    With block-quantised weights and `fuse_quant`, the permutation and the gated activation write the
+    1 x 128 quantised activations of the following grouped GEMM directly (same results bit for bit as the
+    separate kernels, two activation round trips through HBM fewer)."""
     T, H = hidden_states.shape
     E = w13_weight.shape[0]
     top_k = topk_ids.shape[1]
@@ -37,23 +41,33 @@ def ep_moe_forward(hidden_states: torch.Tensor, topk_ids: torch.Tensor, topk_wei
     topk_weights = topk_weights.contiguous()
 
     reorder_topk_ids, src2dst, seg_indptr = run_moe_ep_preproess(topk_ids, num_experts)
-    gateup_input = torch.empty((T * top_k, H), device=dev, dtype=dt)
-    pre_reorder(hidden_states, gateup_input, src2dst, topk_ids, None, start_expert_id, end_expert_id, top_k, H)
-
     seg_cur = seg_indptr[start_expert_id:end_expert_id + 2]
     widx = torch.arange(0, E, device=dev, dtype=torch.int64)
+    quantised = block_shape is not None and w13_weight.dtype in (torch.int8, torch.float8_e4m3fn)
+    fused = bool(fuse_quant and quantised and H % 128 == 0 and (w13_weight.shape[1] // 2) % 128 == 0
+                 and dt in (torch.float16, torch.bfloat16))
+
+    if fused:
+        gateup_input, a1_s = pre_reorder_quant(hidden_states, src2dst, topk_ids, None, start_expert_id, end_expert_id,
+                                               top_k, H, w13_weight.dtype)
+    else:
+        gateup_input, a1_s = torch.empty((T * top_k, H), device=dev, dtype=dt), None
+        pre_reorder(hidden_states, gateup_input, src2dst, topk_ids, None, start_expert_id, end_expert_id, top_k, H)
     gateup_output = torch.empty(gateup_input.shape[0], w13_weight.shape[1], device=dev, dtype=dt)
     grouped_gemm_triton(a=gateup_input, b=w13_weight, c=gateup_output, batch_size=E, weight_column_major=True,
-                        seg_indptr=seg_cur, weight_indices=widx, use_fp8_w8a8=False, scale_a=None,
+                        seg_indptr=seg_cur, weight_indices=widx, use_fp8_w8a8=False, scale_a=a1_s,
                         scale_b=w13_weight_scale, block_shape=block_shape)
 
-    down_input = torch.empty(gateup_output.shape[0], gateup_output.shape[1] // 2, device=dev, dtype=dt)
-    act = {"silu": silu_and_mul, "gelu": gelu_and_mul}[activation]
-    act(gateup_output, down_input, gateup_output.shape[1], reorder_topk_ids, None, start_expert_id, end_expert_id)
-
+    if fused:
+        down_input, a2_s = act_and_mul_quant(gateup_output, gateup_output.shape[1], reorder_topk_ids, None,
+                                             start_expert_id, end_expert_id, w2_weight.dtype, activation)
+    else:
+        down_input, a2_s = torch.empty(gateup_output.shape[0], gateup_output.shape[1] // 2, device=dev, dtype=dt), None
+        act = {"silu": silu_and_mul, "gelu": gelu_and_mul}[activation]
+        act(gateup_output, down_input, gateup_output.shape[1], reorder_topk_ids, None, start_expert_id, end_expert_id)
     down_output = torch.empty(down_input.shape[0], w2_weight.shape[1], device=dev, dtype=dt)
     grouped_gemm_triton(a=down_input, b=w2_weight, c=down_output, batch_size=E, weight_column_major=True,
-                        seg_indptr=seg_cur, weight_indices=widx, use_fp8_w8a8=False, scale_a=None,
+                        seg_indptr=seg_cur, weight_indices=widx, use_fp8_w8a8=False, scale_a=a2_s,
                         scale_b=w2_weight_scale, block_shape=block_shape)
 
     output = torch.empty((T, H), device=dev, dtype=dt)

@@ -93,6 +93,52 @@ def post_reorder(down_output, output, src2dst, topk_ids, topk_weights, start_exp
     return output
 
 
+def _quant_buffers(rows, cols, quant_dtype, device):
+    """(q, s, kind, round_mode) for the 1 x 128 activation format that goes with a weight dtype."""
+    assert cols % 128 == 0, 'row length must be a multiple of 128'
+    if quant_dtype == torch.float8_e4m3fn:
+        return (torch.empty(rows, cols, device=device, dtype=torch.float8_e4m3fn),
+                torch.empty(rows, cols // 128, device=device, dtype=torch.float32), _lib.KIND_FP8, 0)
+    assert quant_dtype == torch.int8, 'quant_dtype must be torch.int8 or torch.float8_e4m3fn'
+    return (torch.empty(rows, cols, device=device, dtype=torch.int8),
+            torch.empty(rows, cols // 128, device=device, dtype=torch.float16), _lib.KIND_I8, 0)
+
+
+def pre_reorder_quant(input, src2dst, topk_ids, a1_scales, start_expert_id, end_expert_id, topk, hidden_size,
+                      quant_dtype):
+    """pre_reorder followed by the 1 x 128 activation quantizer, in one pass (the reference's TODO at
+    sglang_moe_all_gather_all_reduce.py:295-296).  Returns (q [T*topk, hidden], s [T*topk, hidden/128]); equal
+    bit for bit to act_quant(pre_reorder(...)).  Rows of non-local experts are left unwritten."""
+    _lib.require_gpu(input, src2dst, topk_ids)
+    assert input.is_contiguous() and src2dst.is_contiguous() and topk_ids.is_contiguous()
+    assert input.dtype in (torch.float16, torch.bfloat16)
+    T = input.numel() // hidden_size
+    q, s, kind, mode = _quant_buffers(T * topk, hidden_size, quant_dtype, input.device)
+    sc = _f32_or_none(a1_scales)
+    _lib.call("llmk_moe_pre_reorder_quant", _lib.ptr(input), _lib.dt(input.dtype), _lib.ptr(q), _lib.ptr(s), kind, mode,
+              _lib.ptr(src2dst), _lib.ptr(topk_ids), _ids_bytes(topk_ids), _lib.ptr(sc), int(start_expert_id),
+              int(end_expert_id), int(topk), T, int(hidden_size), _lib.stream(input))
+    return q, s
+
+
+def act_and_mul_quant(gateup_output, hidden_size, reorder_topk_ids, scales, start_expert_id, end_expert_id, quant_dtype,
+                      activation="silu"):
+    """silu_and_mul / gelu_and_mul followed by the 1 x 128 activation quantizer, in one pass (the reference's TODO
+    at sglang_moe_all_gather_all_reduce.py:365,407-408).  `hidden_size` is the gate+up width 2I as in
+    silu_and_mul.  Returns (q [M, I], s [M, I/128]); equal bit for bit to act_quant(silu_and_mul(...))."""
+    _lib.require_gpu(gateup_output, reorder_topk_ids)
+    assert gateup_output.is_contiguous() and reorder_topk_ids.is_contiguous()
+    assert gateup_output.dtype in (torch.float16, torch.bfloat16)
+    M = gateup_output.numel() // hidden_size
+    q, s, kind, mode = _quant_buffers(M, hidden_size // 2, quant_dtype, gateup_output.device)
+    sc = _f32_or_none(scales)
+    _lib.call("llmk_moe_act_and_mul_quant", _lib.ptr(gateup_output), _lib.dt(gateup_output.dtype), _lib.ptr(q),
+              _lib.ptr(s), kind, mode, _lib.ptr(reorder_topk_ids), _ids_bytes(reorder_topk_ids), _lib.ptr(sc),
+              int(start_expert_id), int(end_expert_id), M, int(hidden_size), {"silu": 0, "gelu": 1}[activation],
+              _lib.stream(gateup_output))
+    return q, s
+
+
 class _GridCall:
     """Accepts `obj[grid](*args, BLOCK_SIZE=...)`; the grid and the tile size are chosen by the HIP launcher."""
 
@@ -143,11 +189,17 @@ def grouped_gemm_triton(
         assert len(block_shape) == 2
         block_n, block_k = block_shape[0], block_shape[1]
         assert block_n == 128 and block_k == 128, 'block-scaled grouped GEMM uses 128 x 128 weight blocks'
-        if b.dtype == torch.int8:
-            from ..quantization.int8_kernel import act_quant as per_token_group_quant
+        if a.dtype == b.dtype:
+            # extension: activations already in the 1 x block_k format of the weights (from pre_reorder_quant /
+            # act_and_mul_quant); scale_a is theirs
+            assert scale_a is not None, 'quantised activations need scale_a'
+            scale_a = scale_a.contiguous()
         else:
-            from ..quantization.fp8_kernel import act_quant as per_token_group_quant
-        a, scale_a = per_token_group_quant(a.contiguous(), block_k)
+            if b.dtype == torch.int8:
+                from ..quantization.int8_kernel import act_quant as per_token_group_quant
+            else:
+                from ..quantization.fp8_kernel import act_quant as per_token_group_quant
+            a, scale_a = per_token_group_quant(a.contiguous(), block_k)
         assert _cdiv(a.shape[-1], block_k) == scale_a.shape[-1]
         assert _cdiv(b.shape[-2], block_n) == scale_b.shape[-2]
         assert _cdiv(b.shape[-1], block_k) == scale_b.shape[-1]

@@ -207,3 +207,58 @@ def test_ep_moe_forward_mixtral_dims_full_size(dev):
     ref = m.ep_moe_forward(x[sub].cpu(), ids[sub].cpu(), wts[sub].cpu(), w13.cpu(), w13s.cpu(), w2.cpu(), w2s.cpu(),
                            q.act_quant_fp8, dtype=torch.bfloat16)
     assert_close_scaled(out_sub, ref, rtol=5e-2, atol=5e-2, what="subset vs oracle")
+
+
+# ------------------------------------------------------------------ fused permute / activation + quantisation
+@pytest.mark.parametrize("qdt", [torch.float8_e4m3fn, torch.int8])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("with_scales", [False, True])
+def test_fused_quant_kernels_equal_the_two_kernel_sequence(dev, qdt, dtype, with_scales):
+    """pre_reorder_quant == act_quant(pre_reorder) and act_and_mul_quant == act_quant(silu/gelu_and_mul), bit for
+    bit, on the rows of local experts (start/end expert window narrower than the expert set)."""
+    announce("fused quant", qdt, dtype, with_scales)
+    torch.manual_seed(3)
+    T, H, I, E, topk = 70, 384, 256, 8, 2
+    start_e, end_e = 1, 6
+    act_quant = fp8_kernel.act_quant if qdt == torch.float8_e4m3fn else int8_kernel.act_quant
+    x = (torch.randn(T, H) * 3).to(dtype).to(dev)
+    ids = torch.stack([torch.randperm(E)[:topk] for _ in range(T)]).to(dev)
+    reorder_ids, src2dst, seg = gk.run_moe_ep_preproess(ids, E)
+    a1 = (torch.rand(end_e - start_e + 1) + 0.5).to(dev) if with_scales else None
+    local_rows = ((reorder_ids >= start_e) & (reorder_ids <= end_e)).cpu()
+
+    plain = torch.zeros(T * topk, H, dtype=dtype, device=dev)
+    gk.pre_reorder(x, plain, src2dst, ids, a1, start_e, end_e, topk, H)
+    q0, s0 = act_quant(plain)
+    q1, s1 = gk.pre_reorder_quant(x, src2dst, ids, a1, start_e, end_e, topk, H, qdt)
+    assert q1.dtype == qdt and s1.dtype == s0.dtype and s1.shape == s0.shape
+    assert torch.equal(q1.view(torch.uint8).cpu()[local_rows], q0.view(torch.uint8).cpu()[local_rows])
+    assert torch.equal(s1.cpu()[local_rows], s0.cpu()[local_rows])
+
+    gateup = (torch.randn(T * topk, 2 * I) * 2).to(dtype).to(dev)
+    for name, fn in (("silu", gk.silu_and_mul), ("gelu", gk.gelu_and_mul)):
+        down = torch.zeros(T * topk, I, dtype=dtype, device=dev)
+        fn(gateup, down, 2 * I, reorder_ids, a1, start_e, end_e)
+        q0, s0 = act_quant(down)
+        q1, s1 = gk.act_and_mul_quant(gateup, 2 * I, reorder_ids, a1, start_e, end_e, qdt, name)
+        assert torch.equal(q1.view(torch.uint8).cpu()[local_rows], q0.view(torch.uint8).cpu()[local_rows]), name
+        assert torch.equal(s1.cpu()[local_rows], s0.cpu()[local_rows]), name
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+def test_ep_moe_forward_fused_equals_unfused(dev, kind):
+    announce("ep_moe fused vs unfused", kind)
+    torch.manual_seed(9)
+    T, H, I, E, topk = 200, 256, 384, 8, 2
+    dt = torch.bfloat16
+    x = torch.randn(T, H).to(dt).to(dev)
+    ids, w = softmax_topk_router(torch.randn(T, E).to(dev), topk)
+    wq = int8_kernel.weight_quant if kind == "int8" else fp8_kernel.weight_quant
+    w13 = [wq((torch.randn(2 * I, H) * 0.05).to(dev)) for _ in range(E)]
+    w2 = [wq((torch.randn(H, I) * 0.05).to(dev)) for _ in range(E)]
+    cat = lambda xs: torch.stack([t.view(torch.uint8) for t in xs]).view(xs[0].dtype)
+    args = (x, ids, w, cat([t[0] for t in w13]), cat([t[0] for t in w2]), torch.stack([t[1] for t in w13]),
+            torch.stack([t[1] for t in w2]))
+    a = ep_moe_forward(*args, block_shape=[128, 128], fuse_quant=True)
+    b = ep_moe_forward(*args, block_shape=[128, 128], fuse_quant=False)
+    assert torch.equal(a, b)
