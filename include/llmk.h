@@ -115,6 +115,8 @@ int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, cons
                         void* stream);
 /* b packed [N/8, K] int32, nibble (n % 8) of word [n/8, k]; b8 = int8((q - z4[n,kg]) * s4[n,kg]).
  * ref: quantization/w4a8_kernel.py:317-448 */
+/* workspace: at least N*K bytes (the expanded int8 weights); with round16(N*K) +
+ * llmk_gemm_workspace_bytes(M,N,K) bytes large M runs on the fast tile kernels. */
 int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, const void* b_s,
                    int s_dtype, const int8_t* b_s4, const int8_t* b_z4, void* c, int c_dtype,
                    int64_t M, int64_t N, int64_t K, int group_int4,
@@ -138,6 +140,26 @@ int llmk_gemm_w4a16_marlin(const void* a_f16, const int32_t* b, void* c_f16, con
 int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s_f16,
                        int ac_dtype, int64_t M, int64_t N, int64_t K, int groupsize,
                        void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ converters and the one-tile MFMA GEMM
+ * ref: fast_dequant/fast_dtype_convert/fast_uint4_to_fp16.cu:21-109,112-127 (out[i] = nibble_i - 8, nibble i
+ *      of word w at bits 4i; the natural order of the reference's "simple" kernel),
+ *      fast_uint8_to_fp16.cu:8-73 and fast_uint8_to_bf16.cu:8-70 (out[i] = in[i] - 128),
+ *      fast_dequant/simple_marlin/mma_fp16.cu (C fp16 [M,N] = A fp16 [M,K] x B fp16 [K,N], row-major). */
+int llmk_convert_u4_to_f16(const uint32_t* packed, void* out_f16, int64_t n, void* stream);
+int llmk_convert_u8_to_f16(const uint8_t* in, void* out_f16, int64_t n, void* stream);
+int llmk_convert_u8_to_bf16(const uint8_t* in, void* out_bf16, int64_t n, void* stream);
+int llmk_gemm_f16_simple(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K,
+                         void* stream);
+
+/* ------------------------------------------------------------------ communication payload quantizers
+ * ref: quant_communication/quant_utils.py:9-58 (int8, block 32: llmk_act_quant_i8 with
+ *      LLMK_ROUND_HALF_UP), :61-113 and :158-205 (dequant: the product is formed and rounded in the
+ *      scale dtype), :116-155 (e4m3, block 128, scale stored as fp16). */
+int llmk_comm_quant_fp8(const void* x, int x_dtype, void* y_e4m3, void* s, int s_dtype,
+                        int64_t n_groups, int block, void* stream);
+int llmk_comm_dequant(const void* y, int kind, const void* s, int s_dtype, void* x, int x_dtype,
+                      int64_t n_groups, int block, void* stream);
 
 /* ------------------------------------------------------------------ MoE (one GPU's experts)
  * ref: moe/group_gemm_kernel.py:19-45 (segment pointers, src2dst), :81-117 (pre_reorder),

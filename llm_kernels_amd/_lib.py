@@ -44,6 +44,12 @@ SIGNATURES = {
     "llmk_gemm_w4a16_marlin_workspace_bytes": [_l, _l, _l],
     "llmk_gemm_w4a16_marlin": [_p, _p, _p, _p, _l, _l, _l, _i, _p, _l, _p],
     "llmk_gemm_w4a16_nk": [_p, _p, _p, _p, _i, _l, _l, _l, _i, _p, _l, _p],
+    "llmk_convert_u4_to_f16": [_p, _p, _l, _p],
+    "llmk_convert_u8_to_f16": [_p, _p, _l, _p],
+    "llmk_convert_u8_to_bf16": [_p, _p, _l, _p],
+    "llmk_gemm_f16_simple": [_p, _p, _p, _l, _l, _l, _p],
+    "llmk_comm_quant_fp8": [_p, _i, _p, _p, _i, _l, _i, _p],
+    "llmk_comm_dequant": [_p, _i, _p, _i, _p, _i, _l, _i, _p],
     "llmk_moe_seg_indptr": [_p, _p, _l, _i, _p],
     "llmk_moe_src2dst": [_p, _p, _l, _p],
     "llmk_moe_pre_reorder": [_p, _i, _p, _i, _p, _p, _i, _p, _i, _i, _i, _l, _l, _p],

@@ -48,5 +48,9 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
         w4a8_expand_kernel<<<grid, blk, 0, (hipStream_t)stream>>>(b_packed, b_s4, b_z4, (int8_t*)workspace, N, K, group_int4);
         LLMK_CHECK_LAUNCH("gemm_w4a8(expand)");
     }
-    return llmk_gemm_i8_block(a, a_s, (const int8_t*)workspace, b_s, s_dtype, c, c_dtype, M, N, K, nullptr, 0, stream);
+    // what is left of the workspace behind the expanded weights (16-byte aligned) serves the int8 GEMM
+    const int64_t used = (N * K + 15) & ~(int64_t)15;
+    void* rest = workspace_bytes > used ? (void*)((uint8_t*)workspace + used) : nullptr;
+    const int64_t rest_bytes = rest ? workspace_bytes - used : 0;
+    return llmk_gemm_i8_block(a, a_s, (const int8_t*)workspace, b_s, s_dtype, c, c_dtype, M, N, K, rest, rest_bytes, stream);
 }

@@ -10,7 +10,7 @@ namespace {
 // LPG lanes cooperate on one group of LPG*8 contiguous elements.
 template <int DT, int LPG, bool FP8>
 __global__ void act_quant_kernel(const void* __restrict__ x, void* __restrict__ y, void* __restrict__ s,
-                                 int64_t n_groups, int mode) {
+                                 int64_t n_groups, int mode, bool fp8_scale_f16 = false) {
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t grp = tid / LPG;
     const bool live = grp < n_groups;
@@ -23,7 +23,43 @@ __global__ void act_quant_kernel(const void* __restrict__ x, void* __restrict__ 
     for (int j = 0; j < EPL; ++j) m = fmaxf(m, fabsf(v[j]));
     m = group_max<LPG>(m);
     if (!live) return;
-    quant_store8<FP8>(v, m, y, off, s, grp, tid % LPG == 0, mode);
+    quant_store8<FP8>(v, m, y, off, s, grp, tid % LPG == 0, mode, fp8_scale_f16);
+}
+
+// ---------------------------------------------------------------- 1 x block dequant of a communication payload
+// x = cast(y -> scale dtype) * s, the product rounded in the scale dtype (fp16 in the reference), then cast
+// to the output dtype.  LPG lanes per group, 8 elements each.
+template <int SDT, int ODT, int LPG, bool FP8>
+__global__ void block_dequant_kernel(const uint8_t* __restrict__ y, const void* __restrict__ s, void* __restrict__ x,
+                                     int64_t n_groups) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t grp = tid / LPG;
+    if (grp >= n_groups) return;
+    const int64_t off = grp * (LPG * EPL) + (tid % LPG) * EPL;
+    const float sc = FloatIO<SDT>::ld(s, grp);
+    const uint2 raw = *(const uint2*)(y + off);
+    const unsigned w[2] = {raw.x, raw.y};
+    float v[EPL];
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+        const unsigned b = (w[j >> 2] >> (8 * (j & 3))) & 0xff;
+        float q;
+        if constexpr (FP8) {
+            // e4m3fn decode (exact in fp16 and fp32): NaN patterns 0x7f / 0xff stay NaN
+            const unsigned e = (b >> 3) & 0xf, mnt = b & 7;
+            float mag = e ? __uint_as_float(((e + 120u) << 23) | (mnt << 20)) : (float)mnt * 0.001953125f;
+            if ((b & 0x7f) == 0x7f) mag = __uint_as_float(0x7fc00000u);
+            q = (b & 0x80) ? -mag : mag;
+        } else {
+            q = (float)(int)(int8_t)b;
+        }
+        float pr = q * sc;
+        if constexpr (SDT == LLMK_F16) pr = f16_to_f32(f32_to_f16(pr));
+        else if constexpr (SDT == LLMK_BF16) pr = bf16_to_f32(f32_to_bf16(pr));
+        v[j] = pr;
+    }
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) FloatIO<ODT>::st(x, off + j, v[j]);
 }
 
 // ---------------------------------------------------------------- block x block weight quant
@@ -179,6 +215,40 @@ extern "C" int llmk_act_quant_fp8(const void* x, int x_dtype, void* y, float* s,
     LPG_SWITCH(block, CALL)
 #undef CALL
     LLMK_CHECK_LAUNCH("act_quant_fp8");
+    return LLMK_OK;
+}
+
+/* 1 x block e4m3 quantizer with the scale stored as fp16 or fp32 (communication payload format) */
+extern "C" int llmk_comm_quant_fp8(const void* x, int x_dtype, void* y, void* s, int s_dtype, int64_t n_groups,
+                                   int block, void* stream) {
+    if (!lpg_ok(block)) LLMK_FAIL(LLMK_ERR_SHAPE, "comm_quant_fp8: block %d unsupported (power of two in 8..512)", block);
+    if (s_dtype != LLMK_F16 && s_dtype != LLMK_F32) LLMK_FAIL(LLMK_ERR_DTYPE, "comm_quant_fp8: s_dtype %d", s_dtype);
+    if (n_groups == 0) return LLMK_OK;
+    if (!x || !y || !s || n_groups < 0) LLMK_FAIL(LLMK_ERR_ARG, "comm_quant_fp8: bad argument");
+    const int64_t threads = n_groups * (block / EPL);
+    dim3 grid((unsigned)cdiv64(threads, 256)), blk(256);
+    const bool f16s = s_dtype == LLMK_F16;
+#define CALL(L) LLMK_DISPATCH_FLOAT(x_dtype, DT, (act_quant_kernel<DT, L, true><<<grid, blk, 0, (hipStream_t)stream>>>(x, y, s, n_groups, 0, f16s)))
+    LPG_SWITCH(block, CALL)
+#undef CALL
+    LLMK_CHECK_LAUNCH("comm_quant_fp8");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_comm_dequant(const void* y, int kind, const void* s, int s_dtype, void* x, int x_dtype,
+                                 int64_t n_groups, int block, void* stream) {
+    if (!lpg_ok(block)) LLMK_FAIL(LLMK_ERR_SHAPE, "comm_dequant: block %d unsupported (power of two in 8..512)", block);
+    if (kind != LLMK_KIND_I8 && kind != LLMK_KIND_FP8) LLMK_FAIL(LLMK_ERR_DTYPE, "comm_dequant: kind %d", kind);
+    if (n_groups == 0) return LLMK_OK;
+    if (!x || !y || !s || n_groups < 0) LLMK_FAIL(LLMK_ERR_ARG, "comm_dequant: bad argument");
+    const int64_t threads = n_groups * (block / EPL);
+    dim3 grid((unsigned)cdiv64(threads, 256)), blk(256);
+#define CALL(L) LLMK_DISPATCH_FLOAT(s_dtype, SDT, LLMK_DISPATCH_FLOAT(x_dtype, ODT, {                                              \
+        if (kind == LLMK_KIND_FP8) block_dequant_kernel<SDT, ODT, L, true><<<grid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)y, s, x, n_groups); \
+        else block_dequant_kernel<SDT, ODT, L, false><<<grid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)y, s, x, n_groups); }))
+    LPG_SWITCH(block, CALL)
+#undef CALL
+    LLMK_CHECK_LAUNCH("comm_dequant");
     return LLMK_OK;
 }
 

@@ -57,7 +57,7 @@ __device__ __forceinline__ float group_min(float v) {
 // lane, the scale): exactly the arithmetic of the 1 x 128 activation quantizers
 template <bool FP8>
 __device__ __forceinline__ void quant_store8(const float (&v)[EPL], float m, void* y, int64_t off, void* s, int64_t grp,
-                                             bool first_lane, int mode) {
+                                             bool first_lane, int mode, bool fp8_scale_f16 = false) {
     if constexpr (FP8) {
         const float sc = m / 448.f;
         float q[EPL];
@@ -67,7 +67,10 @@ __device__ __forceinline__ void quant_store8(const float (&v)[EPL], float m, voi
         o.x = pack_fp8x4(q[0], q[1], q[2], q[3]);
         o.y = pack_fp8x4(q[4], q[5], q[6], q[7]);
         *(uint2*)((uint8_t*)y + off) = o;
-        if (first_lane) ((float*)s)[grp] = sc;
+        if (first_lane) {
+            if (fp8_scale_f16) ((unsigned short*)s)[grp] = f32_to_f16(sc);
+            else ((float*)s)[grp] = sc;
+        }
     } else {
         const float sc = m / 127.f;
         unsigned w[2] = {0, 0};

@@ -87,7 +87,8 @@ def w4a8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor,
     N = b.size(0) * elements_per_sample
     assert a_s.dtype == b_s.dtype, 'activation and weight scales must share a dtype'
     c = a.new_empty(*a.size()[:-1], N, dtype=torch.get_default_dtype())
-    ws = _lib.workspace(a.device, N * K)
+    # expanded int8 weights, then the scratch of the int8 GEMM behind them
+    ws = _lib.workspace(a.device, ((N * K + 15) // 16) * 16 + max(0, _lib.load().llmk_gemm_workspace_bytes(M, N, K)))
     _lib.call("llmk_gemm_w4a8", _lib.ptr(a), _lib.ptr(a_s), _lib.ptr(b), _lib.ptr(b_s), _lib.dt(a_s.dtype),
               _lib.ptr(b_s4), _lib.ptr(b_z4), _lib.ptr(c), _lib.dt(c.dtype), M, N, K, GROUP_SIZE_INT4,
               _lib.ptr(ws), ws.numel(), _lib.stream(a), exc=AssertionError)
