@@ -203,8 +203,24 @@ def grouped_gemm_triton(
         assert _cdiv(a.shape[-1], block_k) == scale_a.shape[-1]
         assert _cdiv(b.shape[-2], block_n) == scale_b.shape[-2]
         assert _cdiv(b.shape[-1], block_k) == scale_b.shape[-1]
+    elif quantised_w and use_fp8_w8a8:
+        # per-expert scalar scales (the branch the reference keeps commented out, group_gemm_kernel.py:417-420):
+        # c = (a . b^T) * scale_a[e] * scale_b[e] with operands already quantised.  Run as block scales that are
+        # constant per expert: a scalar factor commutes with the per-block accumulation.
+        assert a.dtype == b.dtype, 'per-expert scaling takes activations already in the weight dtype'
+        assert a.shape[-1] % 128 == 0, 'K must be a multiple of 128'
+        kb = a.shape[-1] // 128
+        sdt = torch.float32 if b.dtype == torch.float8_e4m3fn else torch.float16
+        seg64 = seg_indptr.to(torch.int64)
+        rows = (seg64[1:batch_size + 1] - seg64[:batch_size])
+        sa = scale_a.to(torch.float32).flatten()[:batch_size]
+        row_scale = torch.zeros(a.shape[0], device=a.device, dtype=torch.float32)
+        row_scale[seg64[0]:seg64[batch_size]] = torch.repeat_interleave(sa, rows)
+        scale_a = row_scale.to(sdt).unsqueeze(1).expand(-1, kb).contiguous()
+        nb = _cdiv(b.shape[1], 128)
+        scale_b = scale_b.to(sdt).flatten().view(-1, 1, 1).expand(-1, nb, kb).contiguous()
     elif quantised_w:
-        raise AssertionError('quantised weights need block_shape=[128, 128] and scale_b')
+        raise AssertionError('quantised weights need block_shape=[128, 128] and scale_b, or use_fp8_w8a8 with per-expert scales')
     assert a.is_contiguous() and b.is_contiguous() and c.is_contiguous(), 'Input tensors must be contiguous'
     assert b.dim() == 3 and a.shape[-1] == b.shape[-1] and c.shape[-1] == b.shape[1] and c.shape[0] == a.shape[0]
     assert a.dtype == b.dtype, 'a and b must share a dtype after activation quantisation'

@@ -262,3 +262,22 @@ def test_ep_moe_forward_fused_equals_unfused(dev, kind):
     a = ep_moe_forward(*args, block_shape=[128, 128], fuse_quant=True)
     b = ep_moe_forward(*args, block_shape=[128, 128], fuse_quant=False)
     assert torch.equal(a, b)
+
+
+def test_grouped_gemm_per_expert_scalar_scales(dev):
+    """use_fp8_w8a8 without block_shape: c = (a . b^T) * scale_a[e] * scale_b[e] (reference :417-420, commented out there)."""
+    announce("grouped gemm per-expert scales")
+    torch.manual_seed(4)
+    E, N, K = 4, 192, 256
+    seg = torch.tensor([0, 5, 5, 40, 64], dtype=torch.int64)
+    a = (torch.randn(64, K) * 0.5).to(torch.float8_e4m3fn)
+    b = (torch.randn(E, N, K) * 0.5).to(torch.float8_e4m3fn)
+    sa, sb = torch.rand(E) + 0.5, torch.rand(E) + 0.5
+    c = torch.zeros(64, N, dtype=torch.bfloat16, device=dev)
+    gk.grouped_gemm_triton(a.to(dev), b.to(dev), c, E, True, seg.to(dev), torch.arange(E, device=dev), True,
+                           sa.to(dev), sb.to(dev), None)
+    ref = torch.zeros(64, N, dtype=torch.float64)
+    for e in range(E):
+        r0, r1 = int(seg[e]), int(seg[e + 1])
+        ref[r0:r1] = a[r0:r1].double() @ b[e].double().T * float(sa[e]) * float(sb[e])
+    assert_close_scaled(c, ref, what="per-expert scales")
