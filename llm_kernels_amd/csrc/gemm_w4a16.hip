@@ -265,6 +265,26 @@ __global__ __launch_bounds__(NW * 64) void w4a16_nk_kernel(
         }
 }
 
+// [N, K/8] words -> dequantised fp16 W [N][K] (the operand layout of the tiled GEMM): one thread expands one
+// word (8 consecutive k of a row) and stores 16 bytes.
+__global__ void nk_dequant_kernel(const int32_t* __restrict__ B, const _Float16* __restrict__ S, _Float16* __restrict__ W,
+                                  int64_t N, int64_t K, int groupsize) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t kw = K >> 3;
+    if (idx >= N * kw) return;
+    const int64_t n = idx / kw, k = (idx - n * kw) * 8;
+    const unsigned w = (unsigned)B[idx], w8 = w >> 8;
+    const _Float16 sv = S[n * (K / groupsize) + k / groupsize];
+    const v2h sc = {sv, sv};
+    const unsigned p04 = as_u32(deq_lo(w) * sc), p15 = as_u32(deq_hi(w) * sc), p26 = as_u32(deq_lo(w8) * sc), p37 = as_u32(deq_hi(w8) * sc);
+    v4i o;
+    o[0] = (int)__builtin_amdgcn_perm(p15, p04, 0x05040100u);
+    o[1] = (int)__builtin_amdgcn_perm(p37, p26, 0x05040100u);
+    o[2] = (int)__builtin_amdgcn_perm(p15, p04, 0x07060302u);
+    o[3] = (int)__builtin_amdgcn_perm(p37, p26, 0x07060302u);
+    *(v4i*)(W + n * K + k) = o;
+}
+
 // Weight-streaming variant of the [N, K/8] kernel for groupsize % 128 == 0 (every 128-K step lies in one
 // scale group): persistent workgroups of 8 waves walk 16-column tiles; the waves split K by interleaved
 // 128-K steps in batches of U, all loads of a batch issued before its first use and the weights of the next
@@ -564,7 +584,6 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
 extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s, int ac_dtype,
                                   int64_t M, int64_t N, int64_t K, int groupsize, void* workspace,
                                   int64_t workspace_bytes, void* stream) {
-    (void)workspace; (void)workspace_bytes;
     if (ac_dtype != LLMK_F16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a16_nk: only fp16 activations/outputs are supported (dtype code %d)", ac_dtype);
     if (M < 0 || N < 0 || K < 0 || K % 128) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_nk: K=%lld must be a multiple of 128", (long long)K);
     if (M == 0 || N == 0) return LLMK_OK;
@@ -579,6 +598,17 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
     const _Float16* A = (const _Float16*)a;
     const _Float16* S = (const _Float16*)s;
     _Float16* C = (_Float16*)c;
+    if (M > 64 && K % 64 == 0 && workspace && workspace_bytes >= N * K * 2 && !((uintptr_t)workspace & 15)) {
+        // compute-bound: expand W once to fp16 [N, K], then run the tiled MFMA GEMM on it
+        llmk::DirectArgs p{};
+        p.a = (const uint8_t*)a; p.b = (const uint8_t*)workspace; p.c = c; p.c_dtype = LLMK_F16;
+        p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+        if (llmk::dma_eligible(p, 2)) {
+            nk_dequant_kernel<<<(unsigned)cdiv64(N * (K / 8), 256), 256, 0, st>>>(b_packed, S, (_Float16*)workspace, N, K, groupsize);
+            LLMK_CHECK_LAUNCH("gemm_w4a16_nk(dequant)");
+            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_nk(tiled)");
+        }
+    }
     if (groupsize % 128 == 0 && M <= 64) {
         // one 16-column block per tile: two blocks per tile (NT = 2) measured slower at every shape tried
         if (M <= 16) return launch_nk_stream<1, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
