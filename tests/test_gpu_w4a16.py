@@ -142,3 +142,30 @@ def test_mul_split_k_is_deterministic_and_rearms(dev, M, N, K):
     for o in outs[1:]:
         assert torch.equal(o, outs[0])
     assert_close_scaled(outs[0], g.w4a16_gemm(A, q, s, 128), what="marlin split-k")
+
+
+# ------------------------------------------------- compute-bound shapes: dequantise to fp16, then the 256 x 256 tile kernel
+@pytest.mark.parametrize("M,N,K,gs", [(4096, 4096, 256, 128), (4000, 4032, 192, 64), (3856, 4160, 64, 16), (4096, 4096, 128, -1)])
+def test_mul_large_tile_shapes(dev, M, N, K, gs):
+    announce("marlin large tiles", M, N, K, gs)
+    torch.manual_seed(M + K)
+    A = (torch.randn(M, K) * 0.3).half()
+    W = (torch.randn(K, N) * 0.05).half()
+    _, q4, s = mr.fake_quantize(W, gs)
+    B, sp = mr.pack(q4, s, K if gs == -1 else gs)          # the kernel reads scales in the grouped permutation
+    C = torch.zeros(M, N, dtype=torch.half, device=dev)
+    mul(A.to(dev), B.to(dev), C, sp.to(dev), torch.zeros(64, dtype=torch.int32, device=dev))
+    assert_close_scaled(C, g.w4a16_gemm(A, q4, s, gs), what="marlin large tiles")
+
+
+@pytest.mark.parametrize("M,N,K,gs", [(4096, 4096, 256, 128), (3990, 4100, 384, 64), (4096, 3848, 128, 32)])
+def test_w4a16_nk_large_tile_shapes(dev, M, N, K, gs):
+    announce("w4a16 nk large tiles", M, N, K, gs)
+    torch.manual_seed(N + K)
+    x = torch.randn(M, K).half()
+    w = torch.randn(N, K) * 0.02
+    qn, s = q.w4a16_quant_nk(w, gs)
+    packed, _ = bp.pack_cols(qn.numpy(), 4, 32)
+    y = w4a16.w4a16_gemm(x.to(dev), torch.from_numpy(packed).to(dev), s.to(dev), gs)
+    ref = g.w4a16_gemm(x, qn.t().int().contiguous(), s.t().contiguous(), gs)
+    assert_close_scaled(y, ref, what="w4a16 nk large tiles")
