@@ -11,6 +11,7 @@ import argparse
 import json
 import os
 import sys
+import re
 import time
 
 import torch
@@ -342,6 +343,12 @@ def main():
         case = MoECase(args.workload, MOE_WORKLOADS[args.workload])
         op, M, N, K = "moe", case.M, case.N, case.K
     else:
+        if args.workload not in WORKLOADS:
+            # any other shape of a known operator, spelt like the registered names: <op>_m<M>_n<N>_k<K>
+            m = re.fullmatch(r"(fp8|int8|w4a8|w4a16|w4a16_nk)_m(\d+)_n(\d+)_k(\d+)", args.workload)
+            if not m:
+                raise SystemExit("unknown workload %r" % args.workload)
+            WORKLOADS[args.workload] = (m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4)))
         op, M, N, K = WORKLOADS[args.workload]
         case = Case(args.workload, op, M, N, K)
     wall, ev_ms = run_case(case, dev, args.steps, args.warmup, args.eager)

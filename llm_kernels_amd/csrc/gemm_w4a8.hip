@@ -1,5 +1,5 @@
 // W4A8 GEMM: int8 activations x row-packed uint4 weights with two-level scales.
-#include "gemm_direct.hpp"
+#include "gemm_wide.hpp"
 
 using namespace llmk;
 
@@ -32,6 +32,306 @@ __global__ void w4a8_expand_kernel(const int32_t* __restrict__ packed, const int
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------------------
+// Fused decode-size kernel (M <= 64, K <= 4096, 128-wide second-level groups).  The packed words are streamed
+// HBM -> registers -> LDS fully coalesced; each lane then picks the nibble of its column out of the words it
+// needs, and the dequantisation (q - z4) * s4 is moved out of the inner product:
+//     sum_k a_k (q_k - z) s = s (sum_k a_k q_k - z sum_k a_k)      per 128-K group,
+// exact whenever (q - z) s fits int8 for q in 0..15 (weight_quant's output nearly always does).  A wave whose
+// lanes hold out-of-range (z4, s4) for a step dequantises that step nibble by nibble with the int8 wrap.
+//
+// Workgroup = 8 waves on 16 MT rows x 16 columns (two packed rows), persistent over column tiles; each wave
+// takes a run of consecutive 128-K steps; activation fragments, their per-group sums and scales stay resident.  The
+// loads of tiles i+1 and i+2 are in flight while tile i is multiplied; past the last tile the same number of
+// loads is still issued (all lanes on one hot line) so that the wait counts stay exact.
+struct W4A8Args {
+    const int8_t* a; const void* a_s; const int32_t* packed; const void* b_s; const int8_t* s4; const int8_t* z4;
+    void* c; int c_dtype; int M, N, K;
+};
+
+template <int MT, int SDT, int ROUNDS>
+__global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
+    constexpr int NW = 8, U = 4, D = 3;
+    constexpr bool TAB_REGS = MT == 1;                    // per-row sums and scales in registers, else in LDS
+    constexpr int ROWSTRIDE = ROUNDS * 8192 + 64;         // +64: the two packed rows of a tile start in different banks
+    constexpr int TB = 2 * ROWSTRIDE;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4, col8 = r & 7, half = r >> 3;
+    const int M = p.M, N = p.N, K = p.K, steps = K >> 7;
+    const int m0 = blockIdx.y * 16 * MT;
+    const int ntiles = (N + 15) >> 4, np = N >> 3;
+    // wave w multiplies the `cs` consecutive 128-K steps from w * cs: its zero points and second-level scales
+    // of a column are then the bytes of one dword
+    const int cs = (steps + NW - 1) / NW, ks0 = wave * cs;
+    auto step_ok = [&](int u) { return u < cs && ks0 + u < steps; };
+
+    float* red = (float*)smem;                            // [2][NW][MT][256]
+    float2* tab = (float2*)(red + 2 * NW * MT * 256);     // [MT*16][steps]: {activation scale, activation byte sum}
+    uint8_t* tbuf = (uint8_t*)(tab + MT * 16 * steps);    // two staged tiles
+
+    // z / s: the four zero points and second-level scales of this lane's column, one byte per step of the wave;
+    // bs: the block scale of step (lane & 3)
+    struct TileRegs { unsigned z, s, bs; v4i w[2 * ROUNDS]; };
+    auto issue_tile = [&](TileRegs& t, int tile) __attribute__((always_inline)) {
+        const bool live = tile < ntiles;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const int prow = live ? min(tile * 2 + hh, np - 1) : 0;
+            const uint8_t* rowp = (const uint8_t*)p.packed + (int64_t)prow * K * 4;
+#pragma unroll
+            for (int rd = 0; rd < ROUNDS; ++rd) {
+                const uint32_t off = (uint32_t)(rd * 8192 + wave * 1024 + lane * 16);
+                t.w[hh * ROUNDS + rd] = *(const v4i*)(rowp + (live ? min(off, (uint32_t)(K * 4 - 16)) : 0u));
+            }
+        }
+        const int n = live ? min(tile * 16 + r, N - 1) : 0;
+        // dword at byte n * steps + ks0 of each table, pulled back inside the table at its very end
+        const int64_t want = (int64_t)n * steps + ks0, last = (int64_t)N * steps - 4;
+        const int64_t at = min(want, last);
+        const int sh = (int)(want - at) * 8;
+        unsigned zw, sw;
+        __builtin_memcpy(&zw, p.z4 + at, 4);
+        __builtin_memcpy(&sw, p.s4 + at, 4);
+        t.z = sh < 32 ? zw >> sh : 0u;
+        t.s = sh < 32 ? sw >> sh : 0u;
+        const int64_t bsrow = (int64_t)((min(tile, ntiles - 1) * 16) >> 7) * steps;
+        const int kb = min(ks0 + (lane & 3), steps - 1);
+        if constexpr (SDT == LLMK_F32) t.bs = __float_as_uint(((const float*)p.b_s)[bsrow + kb]);
+        else t.bs = ((const unsigned short*)p.b_s)[bsrow + kb];
+    };
+    auto stage_tile = [&](const TileRegs& t, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+            for (int rd = 0; rd < ROUNDS; ++rd)
+                *(v4i*)(tbuf + buf * TB + hh * ROWSTRIDE + rd * 8192 + wave * 1024 + lane * 16) = t.w[hh * ROUNDS + rd];
+    };
+
+    // resident activation fragments (chunks g and g + 4 of every 128-byte step) and their scales first, so that
+    // the per-step sums below are computed while the first weight tiles are still on their way
+    v8i afrag[U][MT];
+    float ascale[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int ks = min(ks0 + u, steps - 1);
+            const int arow = min(m0 + 16 * mt + r, M - 1);
+            afrag[u][mt] = ld_split((const uint8_t*)p.a + (int64_t)arow * K + 16 * g + (int64_t)ks * 128);
+            ascale[u][mt] = ScaleIO<SDT>::cvt(((const typename ScaleIO<SDT>::Raw*)p.a_s)[(int64_t)arow * steps + ks]);
+        }
+
+    int tile = blockIdx.x;
+    const int stride = gridDim.x;
+    TileRegs tr[D];
+#pragma unroll
+    for (int j = 0; j < D - 1; ++j) issue_tile(tr[j], tile + j * stride);
+
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            int sum = 0;
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                const int x = afrag[u][mt][w];
+                sum += (x << 24 >> 24) + (x << 16 >> 24) + (x << 8 >> 24) + (x >> 24);
+            }
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            if (g == 0 && step_ok(u)) tab[(mt * 16 + r) * steps + ks0 + u] = make_float2(ascale[u][mt], (float)sum);
+        }
+    stage_tile(tr[0], 0);
+    __syncthreads();
+    float2 rtab[TAB_REGS ? U : 1][4];
+    if constexpr (TAB_REGS) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) rtab[u][i] = tab[(4 * g + i) * steps + min(ks0 + u, steps - 1)];
+    }
+
+    const unsigned byte_sel = (unsigned)(col8 >> 1);
+    const unsigned sel = byte_sel | ((4u + byte_sel) << 8) | 0x0c0c0000u;     // byte of this column from two words
+    const int nsh = 4 * (col8 & 1);
+    auto nib4 = [&](const v4i& w) {                        // this column's nibble of four consecutive words -> 4 bytes
+        const unsigned t01 = __builtin_amdgcn_perm((unsigned)w[1], (unsigned)w[0], sel);
+        const unsigned t23 = __builtin_amdgcn_perm((unsigned)w[3], (unsigned)w[2], sel);
+        return (int)((__builtin_amdgcn_perm(t23, t01, 0x05040100u) >> nsh) & 0x0f0f0f0fu);
+    };
+
+    v4f acc[MT];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+    };
+    clear_acc();
+    int parity = 0;
+
+    auto load_q = [&](const uint8_t* row, int ksc, v4i& ql, v4i& qh) __attribute__((always_inline)) {
+        const v4i* wl = (const v4i*)(row + (ksc * 128 + 16 * g) * 4);
+        const v4i* wh = (const v4i*)(row + (ksc * 128 + 64 + 16 * g) * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { ql[i] = nib4(wl[i]); qh[i] = nib4(wh[i]); }
+    };
+    auto row_entry = [&](int u, int mt, int i, int ksc) __attribute__((always_inline)) {
+        if constexpr (TAB_REGS) return rtab[u][i];
+        else return tab[(mt * 16 + 4 * g + i) * steps + ksc];
+    };
+    // raw nibbles through the MFMA, zero point and scale applied to the 128-K partial sums: every partial
+    // is an integer below 2^24, so the fp32 arithmetic up to the scale product is exact
+    auto step_fast = [&](int u, int ksc, const v4i& ql, const v4i& qh, int z, int sc4, float bs) __attribute__((always_inline)) {
+        const float zf = (float)z, c1 = bs * (float)sc4;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const v8i a = afrag[u][mt];
+            v4i pr = {0, 0, 0, 0};
+            pr = mfma_i8_16x16x64((v4i){a[0], a[1], a[2], a[3]}, ql, pr);
+            pr = mfma_i8_16x16x64((v4i){a[4], a[5], a[6], a[7]}, qh, pr);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float2 e = row_entry(u, mt, i, ksc);
+                const float part = fmaf(-zf, e.y, (float)pr[i]);
+                acc[mt][i] = fmaf(part, c1 * e.x, acc[mt][i]);
+            }
+        }
+    };
+    // exact int8 wrap of (q - z) and of the product, nibble by nibble
+    auto step_wrap = [&](int u, int ksc, const v4i& ql, const v4i& qh, int z, int sc4, float bs) __attribute__((always_inline)) {
+        auto deq4 = [&](int q4) {
+            unsigned o = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int q = (q4 >> (8 * b)) & 0xf;
+                const int d = (int)(int8_t)(q - z);
+                o |= ((unsigned)((d * sc4) & 0xff)) << (8 * b);
+            }
+            return (int)o;
+        };
+        v4i bl, bh;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { bl[i] = deq4(ql[i]); bh[i] = deq4(qh[i]); }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const v8i a = afrag[u][mt];
+            v4i pr = {0, 0, 0, 0};
+            pr = mfma_i8_16x16x64((v4i){a[0], a[1], a[2], a[3]}, bl, pr);
+            pr = mfma_i8_16x16x64((v4i){a[4], a[5], a[6], a[7]}, bh, pr);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float2 e = row_entry(u, mt, i, ksc);
+                acc[mt][i] = fmaf((float)pr[i], bs * e.x, acc[mt][i]);
+            }
+        }
+    };
+    auto mul_tile = [&](const TileRegs& t, int buf) __attribute__((always_inline)) {
+        const uint8_t* row = tbuf + buf * TB + half * ROWSTRIDE;
+        bool ok[U], all_ok = true;
+        float bs[U];
+        int ksc[U], zu[U], su[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            ksc[u] = min(ks0 + u, steps - 1);
+            const int z = (int)(t.z << (24 - 8 * u)) >> 24, sc4 = (int)(t.s << (24 - 8 * u)) >> 24;
+            zu[u] = z;
+            su[u] = sc4;
+            // (q - z) * s for q = 0 and q = 15 bound every product of the group (24-bit multiplies are exact here)
+            const int p0 = -__mul24(z, sc4), p15 = p0 + 15 * sc4;
+            ok[u] = z >= -112 && min(p0, p15) >= -128 && max(p0, p15) <= 127;
+            all_ok = all_ok && ok[u];
+            const unsigned raw = (unsigned)__builtin_amdgcn_readlane((int)t.bs, u);
+            if constexpr (SDT == LLMK_F32) bs[u] = __uint_as_float(raw);
+            else bs[u] = ScaleIO<SDT>::cvt((unsigned short)raw);
+            if (!step_ok(u)) bs[u] = 0.f;
+        }
+        if (__builtin_amdgcn_ballot_w64(!all_ok) == 0) {
+            // one straight-line block for the whole tile: the LDS reads of a step overlap the arithmetic of the one before
+            v4i ql[2], qh[2];
+            load_q(row, ksc[0], ql[0], qh[0]);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (u + 1 < U) load_q(row, ksc[u + 1], ql[(u + 1) & 1], qh[(u + 1) & 1]);
+                step_fast(u, ksc[u], ql[u & 1], qh[u & 1], zu[u], su[u], bs[u]);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                v4i ql, qh;
+                load_q(row, ksc[u], ql, qh);
+                if (__builtin_amdgcn_ballot_w64(!ok[u]) == 0) step_fast(u, ksc[u], ql, qh, zu[u], su[u], bs[u]);
+                else step_wrap(u, ksc[u], ql, qh, zu[u], su[u], bs[u]);
+            }
+        }
+    };
+    // cross-wave reduction and store of the finished tile; the same barrier publishes the next tile's bytes
+    auto finish = [&](int tl, const TileRegs& next, int next_buf) __attribute__((always_inline)) {
+        float* rbuf = red + parity * NW * MT * 256;
+        parity ^= 1;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) *(v4f*)(rbuf + ((wave * MT + mt) * 64 + lane) * 4) = acc[mt];
+        stage_tile(next, next_buf);
+        __syncthreads();
+        const int n0 = tl * 16;
+        for (int o = tid; o < MT * 256; o += NW * 64) {
+            const int mt = o >> 8, row16 = (o & 255) >> 4, col = o & 15;
+            const int src = (mt * 64 + (row16 >> 2) * 16 + col) * 4 + (row16 & 3);
+            const int m = m0 + 16 * mt + row16, n = n0 + col;
+            if (m >= M || n >= N) continue;
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += rbuf[w * MT * 256 + src];
+            st_out(p.c, (int64_t)m * N + n, sum, p.c_dtype);
+        }
+        clear_acc();
+    };
+    int lbuf = 0;
+    auto one = [&](const TileRegs& cur, const TileRegs& nxt, TileRegs& fill) __attribute__((always_inline)) {
+        issue_tile(fill, tile + (D - 1) * stride);
+        mul_tile(cur, lbuf);
+        finish(tile, nxt, lbuf ^ 1);
+        lbuf ^= 1;
+        tile += stride;
+    };
+    while (tile < ntiles) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            one(tr[j], tr[(j + 1) % D], tr[(j + D - 1) % D]);
+            if (tile >= ntiles) break;
+        }
+    }
+}
+
+template <int MT, int SDT>
+int launch_w4a8_stream(const W4A8Args& p, hipStream_t st) {
+    const int steps = p.K >> 7, rounds = p.K * 4 > 8192 ? 2 : 1;
+    const int ntiles = (p.N + 15) >> 4, mtiles = (p.M + 16 * MT - 1) / (16 * MT);
+    const size_t smem = (size_t)2 * 8 * MT * 256 * 4 + (size_t)MT * 16 * steps * 8 + (size_t)2 * 2 * (rounds * 8192 + 64);
+    auto k1 = w4a8_stream_kernel<MT, SDT, 1>;
+    auto k2 = w4a8_stream_kernel<MT, SDT, 2>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot reserve LDS: %s", hipGetErrorString(e));
+        configured = true;
+    }
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot query the device");
+    }
+    const int gx = min(ntiles, max(1, cus / min(mtiles, cus)));        // one workgroup per CU (LDS bound)
+    dim3 grid((unsigned)gx, (unsigned)mtiles);
+    if (rounds == 1) k1<<<grid, 512, smem, st>>>(p);
+    else k2<<<grid, 512, smem, st>>>(p);
+    LLMK_CHECK_LAUNCH("gemm_w4a8(stream)");
+    return LLMK_OK;
+}
+
 }  // namespace
 
 extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, const void* b_s, int s_dtype,
@@ -42,6 +342,26 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
     if (group_int4 < 4 || group_int4 % 4 || K % group_int4) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a8: group_int4=%d must divide K and be a multiple of 4", group_int4);
     if (M == 0 || N == 0) return LLMK_OK;
     if (!a || !a_s || !b_packed || !b_s || !b_s4 || !b_z4 || !c) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a8: null pointer");
+    // Measured on MI355X with x = N * K / 4096^2: the fused kernel takes about 5 + 3.4 x microseconds per 32 rows
+    // of M; expanding to int8 and running the int8 GEMM about 26 + 3.6 x for x <= 4 and more beyond.
+    const double x = (double)N * (double)K / (4096.0 * 4096.0);
+    const int64_t row_blocks = (M + 31) / 32;
+    const bool fused_wins = row_blocks <= 2 || (row_blocks == 3 && x <= 3.0) || (row_blocks == 4 && x <= 2.0);
+    if (fused_wins && K <= 4096 && group_int4 == 128 && !(((uintptr_t)a | (uintptr_t)b_packed) & 15)) {
+        W4A8Args p{a, a_s, b_packed, b_s, b_s4, b_z4, c, c_dtype, (int)M, (int)N, (int)K};
+        if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: c_dtype %d", c_dtype);
+        hipStream_t st = (hipStream_t)stream;
+#define LLMK_W4A8_MT(SDT)                                                    \
+        do {                                                                 \
+            if (M <= 16) return launch_w4a8_stream<1, SDT>(p, st);           \
+            return launch_w4a8_stream<2, SDT>(p, st);                        \
+        } while (0)
+        if (s_dtype == LLMK_F16) LLMK_W4A8_MT(LLMK_F16);
+        if (s_dtype == LLMK_BF16) LLMK_W4A8_MT(LLMK_BF16);
+        if (s_dtype == LLMK_F32) LLMK_W4A8_MT(LLMK_F32);
+#undef LLMK_W4A8_MT
+        LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: s_dtype %d", s_dtype);
+    }
     if (!workspace || workspace_bytes < N * K) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a8: workspace of N*K=%lld bytes required", (long long)(N * K));
     if (K > 0) {
         dim3 grid((unsigned)cdiv64((N / 8) * (K / 4), 256)), blk(256);

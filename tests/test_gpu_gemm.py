@@ -120,7 +120,9 @@ def test_int8_per_token_int32_bit_exact(dev, M, N, K):
 
 
 # ------------------------------------------------------------------------------------------- w4a8
-@pytest.mark.parametrize("M,N,K", [(1, 128, 128), (16, 256, 512), (37, 136, 256), (16, 4096, 4096), (128, 1024, 7168)])
+@pytest.mark.parametrize("M,N,K", [(1, 128, 128), (16, 256, 512), (37, 136, 256), (16, 4096, 4096), (128, 1024, 7168),
+                                   (5, 8, 128), (33, 264, 2048), (64, 4096, 4096), (17, 1032, 2176), (16, 14336, 4096),
+                                   (16, 512, 4224)])
 def test_w4a8_gemm(dev, M, N, K):
     announce("w4a8_gemm", M, N, K)
     torch.manual_seed(N + K)
@@ -147,6 +149,29 @@ def test_w4a8_exact_and_wrap(dev):
     a = torch.randint(-7, 8, (M, K), dtype=torch.int8)
     ones_a = torch.ones(M, K // 128, dtype=torch.float16)
     ones_b = torch.ones(1, K // 128, dtype=torch.float16)
+    packed, _ = bp.pack_rows(wq.numpy(), 4, 32)
+    with default_dtype(torch.float32):
+        c = w4a8_kernel.w4a8_gemm(a.to(dev), ones_a.to(dev), torch.from_numpy(packed).to(dev), ones_b.to(dev),
+                                  s4.to(dev), z4.to(dev))
+    b8 = q.w4a8_dequant_int8(wq, s4, z4)
+    assert torch.equal(c.cpu().long(), a.long() @ b8.long().T)
+
+
+@pytest.mark.parametrize("M,N,K,sdt", [(16, 5000, 1024, torch.float16), (40, 8192, 4096, torch.float32),
+                                       (3, 312, 384, torch.bfloat16)])
+def test_w4a8_decode_exact_mixed_wrap(dev, M, N, K, sdt):
+    """Decode-size shapes over many column tiles with a sprinkle of out-of-contract (s4, z4): exact integers."""
+    announce("w4a8 decode exact", M, N, K, sdt)
+    torch.manual_seed(M + N)
+    wq = torch.randint(0, 16, (N, K), dtype=torch.uint8)
+    s4 = torch.randint(1, 9, (N, K // 128), dtype=torch.int8)
+    z4 = torch.randint(0, 16, (N, K // 128), dtype=torch.int8)
+    wild = torch.rand(N, K // 128) < 0.02
+    s4[wild] = torch.randint(-128, 128, (int(wild.sum()),), dtype=torch.int8)
+    z4[wild] = torch.randint(-128, 128, (int(wild.sum()),), dtype=torch.int8)
+    a = torch.randint(-3, 4, (M, K), dtype=torch.int8)
+    ones_a = torch.ones(M, K // 128, dtype=sdt)
+    ones_b = torch.ones((N + 127) // 128, K // 128, dtype=sdt)
     packed, _ = bp.pack_rows(wq.numpy(), 4, 32)
     with default_dtype(torch.float32):
         c = w4a8_kernel.w4a8_gemm(a.to(dev), ones_a.to(dev), torch.from_numpy(packed).to(dev), ones_b.to(dev),
