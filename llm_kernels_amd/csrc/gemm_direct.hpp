@@ -96,7 +96,8 @@ struct DirectArgs {
 
 // SDT: dtype code of the block scales, fixed at compile time so that a scale load is a plain typed load with
 // no branch (and hence no wait for memory) between it and the loads around it.
-template <int KIND, int MT, int NW, bool GROUPED, bool RESIDENT, int SDT>
+// VEC: the weight scales of a batch are one vector load (needs four steps per batch and steps % 4 == 0).
+template <int KIND, int MT, int NW, bool GROUPED, bool RESIDENT, int SDT, bool VEC = false>
 __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     typedef typename ScaleIO<SDT>::Raw SRaw;
     constexpr bool HALF = (KIND == K_F16 || KIND == K_BF16);
@@ -157,7 +158,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     };
     const int ntiles = (N + 15) / 16;
     auto ks_of = [&](int ks0, int u, bool& valid) {
-        const int ks = ks0 + u * NW;
+        // ks0 = first step of the batch + wave; VEC: each wave takes U consecutive steps, else waves interleave
+        const int ks = VEC ? (ks0 - wave) + wave * U + u : ks0 + u * NW;
         valid = ks < steps;
         return valid ? ks : steps - 1;
     };
@@ -176,8 +178,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
             }
         }
         if constexpr (BLOCKSCALE) {
+            if constexpr (VEC) {
+                static_assert(U == 4, "one vector of four scales per batch");
+                struct __attribute__((packed)) Quad { SRaw v[4]; };
+                const Quad q = *(const Quad*)((const SRaw*)p.b_s + bs_row + min((ks0 - wave) + wave * U, steps - U));
 #pragma unroll
-            for (int u = 0; u < U; ++u) { bool valid; t.bs[u] = ((const SRaw*)p.b_s)[bs_row + ks_of(ks0, u, valid)]; }
+                for (int u = 0; u < U; ++u) t.bs[u] = q.v[u];
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) { bool valid; t.bs[u] = ((const SRaw*)p.b_s)[bs_row + ks_of(ks0, u, valid)]; }
+            }
         }
     };
     auto load_a = [&](ABatch& t, int ks0) {
@@ -333,7 +343,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         int ks0 = wave;
         auto one = [&](ABatch& ca, BBatch& cb, ABatch& fa, BBatch& fb) __attribute__((always_inline)) {
             const int nk = ks0 + NW * U;
-            const bool more = nk < steps;
+            const bool more = (VEC ? (nk - wave) + wave * U : nk) < steps;   // this wave's first step of the next batch
             const int nt = more ? tile : tile + stride;
             const bool any = nt < ntiles;
             const int fk = more ? nk : wave;
@@ -366,6 +376,10 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
     // Column tiles are processed persistently by as many workgroups as are resident at once (so that every
     // workgroup streams tile after tile with its next tiles already requested), split over the m-tile rows.
     const bool resident = steps <= NW * U;
+    constexpr bool CAN_VEC = SCALED && U == 4;
+    // long K: consecutive steps per wave, one load for the four weight scales of a batch (measured faster at
+    // K = 14336, slower at K = 4096 where the interleaved order spreads the first requests over more channels)
+    const bool vec = CAN_VEC && !resident && steps % 4 == 0;
     static int slots[2] = {0, 0};             // resident workgroups on the whole device, per kernel variant
     if (slots[resident] == 0) {
         int dev = 0, cus = 0, per_cu = 0;
@@ -379,6 +393,13 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
     }
     const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
     dim3 grid((unsigned)gx, (unsigned)mtiles), block(NW * 64);
+    if constexpr (CAN_VEC) {
+        if (vec) {
+            gemm_direct_kernel<KIND, MT, NW, GROUPED, false, SDT, true><<<grid, block, smem, stream>>>(p);
+            LLMK_CHECK_LAUNCH(name);
+            return LLMK_OK;
+        }
+    }
     if (resident) gemm_direct_kernel<KIND, MT, NW, GROUPED, true, SDT><<<grid, block, smem, stream>>>(p);
     else gemm_direct_kernel<KIND, MT, NW, GROUPED, false, SDT><<<grid, block, smem, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
