@@ -18,9 +18,12 @@ int check_common(const char* name, const void* a, const void* b, int64_t M, int6
 }  // namespace
 
 extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    (void)N;
-    // large-M kernels stream fp32 activation scales; 16-bit scales are widened into the workspace first
-    return (M > 64 && K > 0) ? M * (K / 128) * 4 : 0;
+    // large-M kernels stream fp32 activation scales; 16-bit scales are widened into the workspace first;
+    // mid-size M with few tiles adds the fp32 split-K partials behind them
+    if (M <= 64 || K <= 0) return 0;
+    const int64_t scales = (M * (K / 128) * 4 + 255) & ~(int64_t)255;
+    const int z = splitk_factor(M, N, K);
+    return scales + (z > 1 ? (int64_t)z * M * N * 4 : 0);
 }
 
 extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* b, const float* b_s, void* c,

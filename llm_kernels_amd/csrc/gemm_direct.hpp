@@ -92,6 +92,8 @@ struct DirectArgs {
     const int64_t* weight_indices;  // grouped only
     int c_dtype, s_dtype;
     int M, N, K, E;
+    float* partial;        // split-K (dense tile kernel only): fp32 [ksplit][M][N] partial sums
+    int ksplit;            // 0 / 1 = no split
 };
 
 // SDT: dtype code of the block scales, fixed at compile time so that a scale load is a plain typed load with

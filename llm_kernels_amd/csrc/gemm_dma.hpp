@@ -92,7 +92,14 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     constexpr int ESZ = SCALED ? 1 : 2;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
-    const int KT = K >> 7;
+    const int KT_all = K >> 7;
+    // split-K: workgroup z multiplies K steps [kt0, kt0 + KT) and writes fp32 partial sums
+    int kt0 = 0, KT = KT_all;
+    if (!GROUPED && p.ksplit > 1) {
+        const int per = (KT_all + p.ksplit - 1) / p.ksplit;
+        kt0 = (int)blockIdx.z * per;
+        KT = max(0, min(per, KT_all - kt0));
+    }
     const int n0 = blockIdx.x * D_BN;
 
     int m_start, m_end;
@@ -112,14 +119,14 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         if (!found) return;
         const int64_t widx = p.weight_indices ? p.weight_indices[e] : e;
         bbase += widx * (int64_t)N * K;
-        bs_off = widx * (int64_t)((N + 127) / 128) * KT;
+        bs_off = widx * (int64_t)((N + 127) / 128) * KT_all;
     } else {
         m_start = blockIdx.y * BM;
         m_end = min(p.M, m_start + BM);
     }
 
     float* bsl = (float*)(lds + D_NSTAGE * D_STAGE);
-    const int64_t bs_row = bs_off + (int64_t)blockIdx.x * KT;
+    const int64_t bs_row = bs_off + (int64_t)blockIdx.x * KT_all + kt0;
 
     // ---- per-thread source offsets (bytes, 32 bit) of the 7 loads of a stage.
     // Load i of a wave fills LDS rows 8q .. 8q+7 with q = wave*4+i (A) or wave*2+i (B), q & 1 == i & 1.
@@ -141,13 +148,13 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const int col = (R & 64) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
-    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT * 4u;
+    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
 
     auto issue = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
-        const uint8_t* ga = p.a + (int64_t)kt * 128;
-        const uint8_t* gb = bbase + (int64_t)kt * 128;
-        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
+        const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
+        const uint8_t* gb = bbase + (int64_t)(kt0 + kt) * 128;
+        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
 #pragma unroll
         for (int i = 0; i < MI; ++i) dma16(st + (uint32_t)(wave * MI + i) * 1024u, aoff[i], ga);
 #pragma unroll
@@ -340,8 +347,11 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     }
 
     // ---- epilogue: every lane writes 16 consecutive outputs of each of its four rows
-    const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
-    const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
+    const bool split = !GROUPED && p.ksplit > 1;
+    void* cout = split ? (void*)(p.partial + (int64_t)blockIdx.z * p.M * N) : p.c;
+    const int cdt = split ? LLMK_F32 : p.c_dtype;
+    const int esz = cdt == LLMK_F32 ? 4 : 2;
+    const bool vec_ok = ((((uintptr_t)cout) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
     const int nb = n0 + wn * 64 + 16 * g;
     const int n_valid = N - nb;
 #pragma unroll
@@ -349,9 +359,28 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const int m = m_start + wm * WR + 16 * i + r;
         if (m >= m_end || n_valid <= 0) continue;
         const int64_t off = (int64_t)m * N + nb;
-        if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
-        else if (p.c_dtype == LLMK_F16) store_row16<LLMK_F16>(p.c, off, acc[i], n_valid, vec_ok);
-        else store_row16<LLMK_F32>(p.c, off, acc[i], n_valid, vec_ok);
+        if (cdt == LLMK_BF16) store_row16<LLMK_BF16>(cout, off, acc[i], n_valid, vec_ok);
+        else if (cdt == LLMK_F16) store_row16<LLMK_F16>(cout, off, acc[i], n_valid, vec_ok);
+        else store_row16<LLMK_F32>(cout, off, acc[i], n_valid, vec_ok);
+    }
+}
+
+// sum of the split-K partials -> output dtype
+template <int ODT>
+__global__ void splitk_sum_kernel(const float* __restrict__ partial, void* __restrict__ c, int64_t mn, int z) {
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= mn) return;
+    if (i + 4 <= mn && mn % 4 == 0) {
+        v4f s = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < z; ++k) s += *(const v4f*)(partial + (int64_t)k * mn + i);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) FloatIO<ODT>::st(c, i + q, s[q]);
+    } else {
+        for (int64_t j = i; j < min(i + 4, mn); ++j) {
+            float s = 0.f;
+            for (int k = 0; k < z; ++k) s += partial[(int64_t)k * mn + j];
+            FloatIO<ODT>::st(c, j, s);
+        }
     }
 }
 
@@ -381,10 +410,19 @@ int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     }
     constexpr int BM = 64 * MI;
     const int tiles_m = (p.M + BM - 1) / BM + (GROUPED ? p.E : 0);
-    dim3 grid((unsigned)((p.N + D_BN - 1) / D_BN), (unsigned)tiles_m);
+    const bool split = !GROUPED && p.ksplit > 1 && p.partial;
+    dim3 grid((unsigned)((p.N + D_BN - 1) / D_BN), (unsigned)tiles_m, split ? (unsigned)p.ksplit : 1u);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
     kern<<<grid, D_THREADS, D_LDS, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
+    if (split) {
+        const int64_t mn = (int64_t)p.M * p.N;
+        const unsigned blocks = (unsigned)cdiv64(cdiv64(mn, 4), 256);
+        if (p.c_dtype == LLMK_BF16) splitk_sum_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
+        else if (p.c_dtype == LLMK_F16) splitk_sum_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
+        else splitk_sum_kernel<LLMK_F32><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
+        LLMK_CHECK_LAUNCH(name);
+    }
     return LLMK_OK;
 }
 

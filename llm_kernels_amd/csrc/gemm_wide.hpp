@@ -248,6 +248,17 @@ int launch_wide(const DirectArgs& p, hipStream_t stream, const char* name) {
     return LLMK_OK;
 }
 
+// K split of the 64-row-tile kernel: as many slices as bring the grid to about one workgroup per CU, each
+// slice at least eight K steps long; 1 = no split.  (Also sizes the scratch, so it depends on the shape only.)
+inline int splitk_factor(int64_t M, int64_t N, int64_t K) {
+    if (M <= 64 || M > 512) return 1;
+    const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
+    if (tiles >= 128) return 1;          // measured: no gain from two slices at 128 tiles (the summing pass costs as much)
+    int64_t z = 256 / tiles;
+    z = z < (K >> 10) ? z : (K >> 10);
+    return (int)(z > 8 ? 8 : (z < 1 ? 1 : z));
+}
+
 // Tile shape by occupancy: the largest tile (least operand re-reading) that still gives every CU a
 // workgroup.  Segments of a grouped GEMM are judged by their average length.
 template <int KIND, bool GROUPED>
@@ -255,6 +266,7 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
     auto wgs = [&](int bm, int bn) { return ((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm); };
+    if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
     if (wgs(256, 256) >= 240) return launch_wide<KIND, GROUPED>(p, stream, name);
     if (wgs(256, 128) >= 256 || rows > 1024) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
     if (wgs(128, 128) >= 256 || rows > 512) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
@@ -266,6 +278,7 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
 template <int KIND, bool GROUPED>
 int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream_t stream, const char* name) {
     if (!dma_eligible(p)) return launch_tiled<KIND, GROUPED>(p, stream, name);
+    int64_t used = 0;
     if (p.s_dtype != LLMK_F32) {
         const int64_t n = (int64_t)p.M * (p.K >> 7);
         if (!workspace || workspace_bytes < n * 4) return launch_tiled<KIND, GROUPED>(p, stream, name);
@@ -274,6 +287,17 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
         else scales_to_f32_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
         LLMK_CHECK_LAUNCH(name);
         p.a_s = workspace;
+        used = (n * 4 + 255) & ~(int64_t)255;
+    }
+    // Few 64-row tiles (mid-size M, moderate N): split K over workgroups so that every CU streams weights,
+    // fp32 partials in the workspace, one summing pass.
+    if constexpr (!GROUPED) {
+        const int z = splitk_factor(p.M, p.N, p.K);
+        const int64_t need = (int64_t)z * p.M * p.N * 4;
+        if (z > 1 && workspace && workspace_bytes - used >= need && !(((uintptr_t)workspace + used) & 15)) {
+            p.partial = (float*)((uint8_t*)workspace + used);
+            p.ksplit = z;
+        }
     }
     return launch_dma<KIND, GROUPED>(p, stream, name);
 }

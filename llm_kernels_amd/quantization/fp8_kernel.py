@@ -60,5 +60,5 @@ def fp8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Ten
     assert a_s.dtype == torch.float32 and b_s.dtype == torch.float32, 'fp8 scales must be float32'
     c = a.new_empty(*a.size()[:-1], N, dtype=torch.get_default_dtype())
     _lib.call("llmk_gemm_fp8_block", _lib.ptr(a), _lib.ptr(a_s), _lib.ptr(b), _lib.ptr(b_s), _lib.ptr(c),
-              _lib.dt(c.dtype), M, N, K, None, 0, _lib.stream(a), exc=AssertionError)
+              _lib.dt(c.dtype), M, N, K, *_lib.gemm_workspace(a.device, M, N, K), _lib.stream(a), exc=AssertionError)
     return c

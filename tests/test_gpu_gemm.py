@@ -181,6 +181,28 @@ def test_w4a8_decode_exact_mixed_wrap(dev, M, N, K, sdt):
 
 
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
+@pytest.mark.parametrize("M,N,K,out", [(128, 1024, 4096, torch.bfloat16), (200, 520, 3200, torch.float32),
+                                       (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16)])
+def test_mid_m_split_k_shapes(dev, kind, M, N, K, out):
+    """Mid-size M with few column tiles: the K range is split over workgroups (uneven slices included)."""
+    announce("split-K", kind, M, N, K, out)
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    with default_dtype(out):
+        if kind == "fp8":
+            a, a_s = q.act_quant_fp8(x)
+            b, b_s = q.weight_quant_fp8(w)
+            c = fp8_kernel.fp8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+        else:
+            a, a_s = q.act_quant_int8(x)
+            b, b_s = q.weight_quant_int8(w)
+            c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert c.dtype == out
+    assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="split-K " + kind)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("M,N,K", [(65, 128, 128), (130, 200, 256), (300, 384, 512), (520, 256, 384), (1100, 130, 256)])
 def test_tiled_kernels_ragged_shapes(dev, kind, M, N, K):
     """Shapes that exercise every tile height of the large-M kernel, with ragged M and N."""
