@@ -158,12 +158,25 @@ __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
     }
 }
 
+// four outputs per thread (MN is a multiple of 64): all Z partial vectors are requested before the first add
 __global__ void splitk_reduce_f16_kernel(const float* __restrict__ ws, _Float16* __restrict__ C, int64_t MN, int Z) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= MN) return;
-    float s = 0.f;
-    for (int z = 0; z < Z; ++z) s += ws[(int64_t)z * MN + i];
-    C[i] = (_Float16)s;
+    v4f s = {0.f, 0.f, 0.f, 0.f};
+    int z = 0;
+    for (; z + 8 <= Z; z += 8) {
+        v4f t[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = *(const v4f*)(ws + (int64_t)(z + j) * MN + i);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += t[j];
+    }
+    for (; z < Z; ++z) s += *(const v4f*)(ws + (int64_t)z * MN + i);
+    const v2h lo = {(_Float16)s[0], (_Float16)s[1]}, hi = {(_Float16)s[2], (_Float16)s[3]};
+    unsigned u0, u1;
+    __builtin_memcpy(&u0, &lo, 4);
+    __builtin_memcpy(&u1, &hi, 4);
+    *(uint2*)(C + i) = make_uint2(u0, u1);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -553,7 +566,7 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
         }
     }
     MarlinPlan pl = marlin_plan(M, N, K);
-    if (pl.z > 1 && (!workspace || workspace_bytes < (int64_t)pl.z * M * N * 4)) {
+    if (pl.z > 1 && (!workspace || workspace_bytes < (int64_t)pl.z * M * N * 4 || (((uintptr_t)workspace) & 15) || (((uintptr_t)c) & 7))) {
         pl.z = 1;                                   // no scratch: every workgroup walks all of K
         pl.steps_per_z = (int)((K / 16 + 1) / 2);
     }
@@ -575,7 +588,7 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
 #undef LLMK_MARLIN_LAUNCH
     LLMK_CHECK_LAUNCH("gemm_w4a16_marlin");
     if (pl.z > 1) {
-        splitk_reduce_f16_kernel<<<(unsigned)cdiv64(M * N, 256), 256, 0, st>>>((const float*)workspace, C, M * N, pl.z);
+        splitk_reduce_f16_kernel<<<(unsigned)cdiv64(M * N, 4 * 256), 256, 0, st>>>((const float*)workspace, C, M * N, pl.z);
         LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(reduce)");
     }
     return LLMK_OK;
