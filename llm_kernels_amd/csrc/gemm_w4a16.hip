@@ -304,7 +304,7 @@ __global__ void nk_dequant_kernel(const int32_t* __restrict__ B, const _Float16*
 // two tiles requested ahead.  When a wave's K share fits one batch (RESIDENT) its activation fragments are
 // loaded and permuted once and stay in registers for every tile.  The group scale multiplies the fp32
 // partial of the step (one FMA per output) instead of the eight fp16 weights.
-template <int MT, int NT, bool RESIDENT>
+template <int MT, int NT, bool RESIDENT, bool VS = false>
 __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     const _Float16* __restrict__ A, const int32_t* __restrict__ B, const _Float16* __restrict__ S,
     _Float16* __restrict__ C, int M, int N, int K, int groupsize) {
@@ -329,6 +329,9 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     struct ABatch {
         v4i a[U][MT][4];
     };
+    // step u of the batch that starts at ks0 (= first step of the batch + wave).  VS: every wave takes U
+    // consecutive steps and, with 128-wide groups, fetches their four scales with one load.
+    auto step_of = [&](int ks0, int u) { return VS ? (ks0 - wave) + wave * U + u : ks0 + u * NW; };
     auto clamp_step = [&](int ks) { return min(ks, steps - 1); };
     auto load_b = [&](BBatch& t, int tile, int ks0) __attribute__((always_inline)) {
 #pragma unroll
@@ -336,14 +339,21 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
             const int nrow = min((tile * NT + nt) * 16 + r, N - 1);
             const int32_t* brow = B + (int64_t)nrow * kwords + 4 * g;
 #pragma unroll
-            for (int u = 0; u < U; ++u) t.w[nt][u] = *(const v4i*)(brow + clamp_step(ks0 + u * NW) * 16);
+            for (int u = 0; u < U; ++u) t.w[nt][u] = *(const v4i*)(brow + clamp_step(step_of(ks0, u)) * 16);
         }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const int nrow = min((tile * NT + nt) * 16 + r, N - 1);
             const unsigned short* srow = (const unsigned short*)S + (int64_t)nrow * ngroups;
+            if constexpr (VS) {
+                static_assert(U == 4, "four scales per load");
+                const uint2 q = *(const uint2*)(srow + min(step_of(ks0, 0), steps - U));
+                t.s[nt][0] = (unsigned short)q.x; t.s[nt][1] = (unsigned short)(q.x >> 16);
+                t.s[nt][2] = (unsigned short)q.y; t.s[nt][3] = (unsigned short)(q.y >> 16);
+            } else {
 #pragma unroll
-            for (int u = 0; u < U; ++u) t.s[nt][u] = srow[(clamp_step(ks0 + u * NW) * 128) / groupsize];
+                for (int u = 0; u < U; ++u) t.s[nt][u] = srow[(clamp_step(step_of(ks0, u)) * 128) / groupsize];
+            }
         }
     };
     auto load_a = [&](ABatch& t, int ks0) __attribute__((always_inline)) {
@@ -352,7 +362,7 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) t.a[u][mt][j] = *(const v4i*)(arow[mt] + clamp_step(ks0 + u * NW) * 128 + 8 * j);
+                for (int j = 0; j < 4; ++j) t.a[u][mt][j] = *(const v4i*)(arow[mt] + clamp_step(step_of(ks0, u)) * 128 + 8 * j);
     };
     // k order of a dequantised word is [0,4,1,5,2,6,3,7]: bring the activation fragment into the same order
     auto perm_a = [&](ABatch& t) __attribute__((always_inline)) {
@@ -374,7 +384,7 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     auto mul = [&](const ABatch& ta, const BBatch& tb, int ks0, v4f (&acc)[NT][MT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const bool valid = ks0 + u * NW < steps;
+            const bool valid = step_of(ks0, u) < steps;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const float sc = valid ? f16_to_f32(tb.s[nt][u]) : 0.f;
@@ -461,7 +471,7 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
         int ks0 = wave;
         auto one = [&](ABatch& ca, BBatch& cb, ABatch& fa, BBatch& fb) __attribute__((always_inline)) {
             const int nk = ks0 + NW * U;
-            const bool more = nk < steps;
+            const bool more = step_of(nk, 0) < steps;
             const int nt = more ? tile : tile + stride;
             const bool any = nt < ntiles;
             const int fk = more ? nk : wave;
@@ -500,6 +510,15 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
     }
     const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
     dim3 grid((unsigned)gx, (unsigned)mtiles);
+    if constexpr (U == 4) {
+        // consecutive steps per wave and one load for their four scales
+        if (groupsize == 128 && steps % 4 == 0 && !(((uintptr_t)S) & 7)) {
+            if (resident) w4a16_nk_stream_kernel<MT, NT, true, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
+            else w4a16_nk_stream_kernel<MT, NT, false, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
+            LLMK_CHECK_LAUNCH("gemm_w4a16_nk(stream)");
+            return LLMK_OK;
+        }
+    }
     if (resident) w4a16_nk_stream_kernel<MT, NT, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
     else w4a16_nk_stream_kernel<MT, NT, false><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
     LLMK_CHECK_LAUNCH("gemm_w4a16_nk(stream)");
