@@ -156,19 +156,25 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     // the next stage and for its own LDS reads, and meets the others at the barrier.  Behind the barrier
     // the next stage is complete and nobody reads the current one any more, so the loads of step kt + 2
     // (ISSUE) may overwrite it, and the fragments of step kt + 1 are fetched while row 7 is multiplied.
-    auto step = [&](int kt, auto sync_c, auto issue_c) {
+    // NR = tile rows (of 16) this wave multiplies.  Dense GEMM: always 8.  Grouped GEMM: the last m-tile of
+    // a segment is ragged, and a wave whose rows lie (partly) behind the segment end runs a variant of the
+    // loop that neither fetches nor multiplies the tile rows from NR on (their accumulators are never
+    // stored); the loop is instantiated for NR = 8, 4 and 0 so that it stays free of branches (a two-row variant
+    // measured no faster: short tails are bound by the per-step barrier, not by the matrix pipe).
+    auto step = [&](int kt, auto sync_c, auto issue_c, auto nr_c) {
         constexpr bool SYNC = decltype(sync_c)::value, ISSUE = decltype(issue_c)::value;
+        constexpr int NR = decltype(nr_c)::value;
         const uint8_t* As = stage_a(kt);
         float sa[8];
-        if constexpr (SCALED) {
+        if constexpr (SCALED && NR > 0) {
             const float* Ss = (const float*)(lds + (kt & 1) * W_STAGE + W_A + W_B) + wm * 128 + r;
             const float bs = bsl[(wn >> 1) * D_MAX_KT + kt];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) sa[i] = Ss[i * 16] * bs;
+            for (int i = 0; i < NR; ++i) sa[i] = Ss[i * 16] * bs;
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            if (i < 7) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+            if (i + 1 < NR) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
             if (i == 7 && SYNC) {
                 __builtin_amdgcn_sched_barrier(0);
                 __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
@@ -178,16 +184,18 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if constexpr (SCALED) {
-                    t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
-                    if (i > 0) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
-                    else acc[7][j] += t[1][j] * sprev;
+                    if (i < NR) t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
+                    if (i > 0 && i <= NR) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
+                    else if (i == 0 && NR == 8) acc[7][j] += t[1][j] * sprev;
                 } else {
-                    acc[i][j] = mma16(bf[j], af[i & 1], acc[i][j]);
+                    if (i < NR) acc[i][j] = mma16(bf[j], af[i & 1], acc[i][j]);
                 }
                 if (i == 7 && SYNC) {
                     if (j == 0 && ISSUE) issue(kt + 2);
-                    bf[j] = ldfrag(stage_b(kt + 1) + j * 2048);
-                    if (j == 3) af[0] = ldfrag(stage_a(kt + 1));
+                    if (NR > 0) {
+                        bf[j] = ldfrag(stage_b(kt + 1) + j * 2048);
+                        if (j == 3) af[0] = ldfrag(stage_a(kt + 1));
+                    }
                 }
                 // Nothing moves across a tile boundary: the FMAs retire a product finished four MFMAs
                 // ago, never the one just issued, and each activation fragment is requested a whole
@@ -195,7 +203,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if constexpr (SCALED) sprev = sa[7];
+        if constexpr (SCALED && NR == 8) sprev = sa[7];
     };
 
     if (KT > 1) issue(1);
@@ -206,13 +214,23 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     }
     const std::true_type yes;
     const std::false_type no;
-    int kt = 0;
-    for (; kt + 2 < KT; ++kt) step(kt, yes, yes);
-    if (kt + 1 < KT) { step(kt, yes, no); ++kt; }
-    if (kt < KT) step(kt, no, no);
-    if constexpr (SCALED) {
+    auto run = [&](auto nr_c) {
+        int kt = 0;
+        for (; kt + 2 < KT; ++kt) step(kt, yes, yes, nr_c);
+        if (kt + 1 < KT) { step(kt, yes, no, nr_c); ++kt; }
+        if (kt < KT) step(kt, no, no, nr_c);
+        if constexpr (SCALED && decltype(nr_c)::value == 8) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[7][j] += t[1][j] * sprev;
+            for (int j = 0; j < 4; ++j) acc[7][j] += t[1][j] * sprev;
+        }
+    };
+    if constexpr (GROUPED) {
+        const int live = m_end - m_start - wm * 128;       // rows of this wave inside the segment (wave-uniform)
+        if (live > 64) run(std::integral_constant<int, 8>{});
+        else if (live > 0) run(std::integral_constant<int, 4>{});
+        else run(std::integral_constant<int, 0>{});
+    } else {
+        run(std::integral_constant<int, 8>{});
     }
 
     // ---- epilogue: every lane writes 16 consecutive outputs of each of its eight rows
