@@ -55,6 +55,8 @@ template <int DT> __device__ __forceinline__ float rnd(float v) {
 
 // gated activation of one element with the reference's rounding points (activation in fp32, rounded to the
 // tensor dtype, product in the tensor dtype, optional per-expert scale in the tensor dtype)
+constexpr int AMQ_UNROLL = 4;      // groups per thread of the fused activation + quantisation kernel
+
 template <int IDT>
 __device__ __forceinline__ float gated_act(float gv, float up, int act, bool has_scale, float scale) {
     if (act == 0) {
@@ -97,28 +99,40 @@ __global__ void act_mul_quant_kernel(const void* __restrict__ gateup, void* __re
                                      const void* __restrict__ reorder_topk_ids, int ids_bytes,
                                      const float* __restrict__ scales, int start_e, int end_e, int64_t M, int64_t two_i,
                                      int act, int mode) {
+    // a workgroup owns AMQ_UNROLL x 16 consecutive groups; a thread requests the operands of all its groups
+    // before it converts the first one
     const int64_t I = two_i / 2, gpr = I / 128;
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t grp = tid >> 4;
-    const bool live = grp < M * gpr;
-    const int64_t gs = live ? grp : 0;
-    const int64_t row = gs / gpr, col = (gs - row * gpr) * 128 + (tid & 15) * EPL;
-    const int64_t e = ld_id(reorder_topk_ids, row, ids_bytes);
-    const bool local = e >= start_e && e <= end_e;
-    const bool has_scale = scales != nullptr && local;
-    const float scale = has_scale ? rnd<IDT>(1.0f / scales[e - start_e]) : 1.0f;
-    float gv[EPL], up[EPL], r[EPL];
-    load8<IDT>(gateup, row * two_i + col, gv);
-    load8<IDT>(gateup, row * two_i + I + col, up);
-    float m = 0.f;
+    const int sub = threadIdx.x & 15;
+    int64_t grp[AMQ_UNROLL], row[AMQ_UNROLL], col[AMQ_UNROLL];
+    bool live[AMQ_UNROLL];
+    float gv[AMQ_UNROLL][EPL], up[AMQ_UNROLL][EPL];
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) {
-        r[j] = gated_act<IDT>(gv[j], up[j], act, has_scale, scale);
-        m = fmaxf(m, fabsf(r[j]));
+    for (int k = 0; k < AMQ_UNROLL; ++k) {
+        grp[k] = ((int64_t)blockIdx.x * AMQ_UNROLL + k) * (blockDim.x >> 4) + (threadIdx.x >> 4);
+        live[k] = grp[k] < M * gpr;
+        const int64_t gs = live[k] ? grp[k] : 0;
+        row[k] = gs / gpr;
+        col[k] = (gs - row[k] * gpr) * 128 + sub * EPL;
+        load8<IDT>(gateup, row[k] * two_i + col[k], gv[k]);
+        load8<IDT>(gateup, row[k] * two_i + I + col[k], up[k]);
     }
-    m = group_max<16>(m);
-    if (!live || !local) return;
-    quant_store8<FP8>(r, m, q_out, row * I + col, s_out, grp, (tid & 15) == 0, mode);
+#pragma unroll
+    for (int k = 0; k < AMQ_UNROLL; ++k) {
+        const int64_t e = ld_id(reorder_topk_ids, row[k], ids_bytes);
+        const bool local = e >= start_e && e <= end_e;
+        const bool has_scale = scales != nullptr && local;
+        const float scale = has_scale ? rnd<IDT>(1.0f / scales[e - start_e]) : 1.0f;
+        float r[EPL];
+        float m = 0.f;
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) {
+            r[j] = gated_act<IDT>(gv[k][j], up[k][j], act, has_scale, scale);
+            m = fmaxf(m, fabsf(r[j]));
+        }
+        m = group_max<16>(m);
+        if (!live[k] || !local) continue;
+        quant_store8<FP8>(r, m, q_out, row[k] * I + col[k], s_out, grp[k], sub == 0, mode);
+    }
 }
 
 // Token permutation and 1 x 128 activation quantisation in one pass: a token's row is read once, quantised
@@ -236,7 +250,7 @@ extern "C" int llmk_moe_act_and_mul_quant(const void* gateup, int in_dtype, void
     if (!gateup || !q_out || !s_out || !reorder_topk_ids) LLMK_FAIL(LLMK_ERR_ARG, "moe_act_and_mul_quant: null pointer");
     if (((uintptr_t)gateup | (uintptr_t)q_out) & 15) LLMK_FAIL(LLMK_ERR_ARG, "moe_act_and_mul_quant: buffers must be 16-byte aligned");
     const int64_t threads = M * (two_i / 256) * 16;
-    const unsigned grid = (unsigned)cdiv64(threads, 256);
+    const unsigned grid = (unsigned)cdiv64(threads, 256 * AMQ_UNROLL);
     LLMK_DISPATCH_FLOAT(in_dtype, IDT, {
         if (kind == LLMK_KIND_FP8) act_mul_quant_kernel<IDT, true><<<grid, 256, 0, (hipStream_t)stream>>>(gateup, q_out, s_out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, M, two_i, act, round_mode);
         else act_mul_quant_kernel<IDT, false><<<grid, 256, 0, (hipStream_t)stream>>>(gateup, q_out, s_out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, M, two_i, act, round_mode);
