@@ -20,7 +20,7 @@ int check_common(const char* name, const void* a, const void* b, int64_t M, int6
 extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     // large-M kernels stream fp32 activation scales; 16-bit scales are widened into the workspace first;
     // mid-size M with few tiles adds the fp32 split-K partials behind them
-    if (M <= 64 || K <= 0) return 0;
+    if (K <= 0 || (M <= 64 && !mid_m_prefers_tiles(M, N, K))) return 0;
     const int64_t scales = (M * (K / 128) * 4 + 255) & ~(int64_t)255;
     const int z = splitk_factor(M, N, K);
     return scales + (z > 1 ? (int64_t)z * M * N * 4 : 0);
@@ -36,7 +36,8 @@ extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* 
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
-    if (M > 64) return launch_big<K_FP8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_fp8_block(tiled)");
+    if (M > 64 || (mid_m_prefers_tiles(M, N, K) && workspace && workspace_bytes >= llmk_gemm_workspace_bytes(M, N, K)))
+        return launch_big<K_FP8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_fp8_block(tiled)");
     return launch_direct<K_FP8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_fp8_block");
 }
 
@@ -51,7 +52,8 @@ extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
-    if (M > 64) return launch_big<K_I8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_i8_block(tiled)");
+    if (M > 64 || (mid_m_prefers_tiles(M, N, K) && workspace && workspace_bytes >= llmk_gemm_workspace_bytes(M, N, K)))
+        return launch_big<K_I8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_i8_block(tiled)");
     return launch_direct<K_I8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_block");
 }
 

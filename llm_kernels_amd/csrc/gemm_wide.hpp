@@ -268,13 +268,21 @@ int launch_wide(const DirectArgs& p, hipStream_t stream, const char* name) {
 
 // K split of the 64-row-tile kernel: as many slices as bring the grid to about one workgroup per CU, each
 // slice at least eight K steps long; 1 = no split.  (Also sizes the scratch, so it depends on the shape only.)
+// With 128 or more tiles the summing pass costs what two slices save unless K is long.
 inline int splitk_factor(int64_t M, int64_t N, int64_t K) {
-    if (M <= 64 || M > 512) return 1;
+    if (M <= 16 || M > 512) return 1;
     const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
-    if (tiles >= 128) return 1;          // measured: no gain from two slices at 128 tiles (the summing pass costs as much)
-    int64_t z = 256 / tiles;
+    if (tiles >= 256 || (tiles >= 128 && K < 8192)) return 1;
+    int64_t z = (255 + tiles) / tiles;
     z = z < (K >> 10) ? z : (K >> 10);
     return (int)(z > 8 ? 8 : (z < 1 ? 1 : z));
+}
+
+// 16 < M <= 64: the weight-streaming kernel re-reads the activations for every 16 columns, which costs more
+// than the 64-row tile kernel (with split-K when its tiles are few) once the weight matrix is large (measured
+// crossover between 17 M and 25 M elements).
+inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
+    return M > 16 && M <= 64 && N * K >= (int64_t)20 << 20;
 }
 
 // Tile shape by occupancy: the largest tile (least operand re-reading) that still gives every CU a

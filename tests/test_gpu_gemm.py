@@ -182,7 +182,9 @@ def test_w4a8_decode_exact_mixed_wrap(dev, M, N, K, sdt):
 
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("M,N,K,out", [(128, 1024, 4096, torch.bfloat16), (200, 520, 3200, torch.float32),
-                                       (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16)])
+                                       (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16),
+                                       (48, 2560, 16384, torch.bfloat16), (64, 14336, 4096, torch.float16),
+                                       (256, 4096, 14336, torch.bfloat16)])
 def test_mid_m_split_k_shapes(dev, kind, M, N, K, out):
     """Mid-size M with few column tiles: the K range is split over workgroups (uneven slices included)."""
     announce("split-K", kind, M, N, K, out)
