@@ -426,8 +426,11 @@ int launch_direct_mt(const DirectArgs& p, hipStream_t stream, const char* name) 
 
 template <int KIND, bool GROUPED>
 int launch_direct(const DirectArgs& p, int max_rows_per_segment_hint, hipStream_t stream, const char* name) {
-    // m-tiles per workgroup: 1 for decode-sized M, up to 4 otherwise
-    if (max_rows_per_segment_hint <= 16) return launch_direct_mt<KIND, 1, GROUPED>(p, stream, name);
+    // m-tiles per workgroup: 1 for decode-sized M, up to 4 otherwise.  When a wave's K share fits one batch at
+    // one m-tile per workgroup (activations resident in registers), 16-row workgroups side by side beat taller
+    // ones that have to re-read their activations for every column tile.
+    constexpr int KSTEP = (KIND == K_F16 || KIND == K_BF16) ? 64 : 128;
+    if (max_rows_per_segment_hint <= 16 || p.K / KSTEP <= 32) return launch_direct_mt<KIND, 1, GROUPED>(p, stream, name);
     if (max_rows_per_segment_hint <= 32) return launch_direct_mt<KIND, 2, GROUPED>(p, stream, name);
     return launch_direct_mt<KIND, 4, GROUPED>(p, stream, name);
 }

@@ -532,8 +532,8 @@ struct MarlinPlan {
 
 MarlinPlan marlin_plan(int64_t M, int64_t N, int64_t K) {
     MarlinPlan pl{};
-    pl.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-    pl.nw = pl.mt == 1 ? 8 : (pl.mt == 2 ? 4 : 2);          // nw * mt * 8 KiB of reduction LDS <= 64 KiB
+    pl.mt = 1;                                              // 16-row workgroups side by side (measured faster than taller ones)
+    pl.nw = 8;                                              // nw * mt * 8 KiB of reduction LDS <= 64 KiB
     pl.mblocks = (int)cdiv64(M, 16 * pl.mt);
     pl.col_groups = (int)((N / 64 + 1) / 2);
     const int total_steps = (int)((K / 16 + 1) / 2);
@@ -601,9 +601,7 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
         if (pl.z > 1) w4a16_marlin_kernel<MT, NW, true><<<grid, blk, smem, st>>>(A, B, S, C, ws, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
         else w4a16_marlin_kernel<MT, NW, false><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
     } while (0)
-    if (pl.mt == 1) LLMK_MARLIN_LAUNCH(1, 8);
-    else if (pl.mt == 2) LLMK_MARLIN_LAUNCH(2, 4);
-    else LLMK_MARLIN_LAUNCH(4, 2);
+    LLMK_MARLIN_LAUNCH(1, 8);
 #undef LLMK_MARLIN_LAUNCH
     LLMK_CHECK_LAUNCH("gemm_w4a16_marlin");
     if (pl.z > 1) {
@@ -642,8 +640,10 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
         }
     }
     if (groupsize % 128 == 0 && M <= 64) {
-        // one 16-column block per tile: two blocks per tile (NT = 2) measured slower at every shape tried
-        if (M <= 16) return launch_nk_stream<1, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
+        // one 16-column block per tile: two blocks per tile (NT = 2) measured slower at every shape tried.
+        // While the activations of a 16-row workgroup stay resident (K <= 4096), such workgroups side by side
+        // beat taller ones by up to 2x.
+        if (M <= 16 || K <= 4096) return launch_nk_stream<1, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
         if (M <= 32) return launch_nk_stream<2, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
         return launch_nk_stream<4, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
     }

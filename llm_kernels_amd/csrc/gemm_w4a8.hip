@@ -353,7 +353,8 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
         hipStream_t st = (hipStream_t)stream;
 #define LLMK_W4A8_MT(SDT)                                                    \
         do {                                                                 \
-            if (M <= 16) return launch_w4a8_stream<1, SDT>(p, st);           \
+            /* 16-row workgroups side by side win while the weights are small, 32-row ones beyond */ \
+            if (M <= 16 || N * K <= ((int64_t)20 << 20)) return launch_w4a8_stream<1, SDT>(p, st); \
             return launch_w4a8_stream<2, SDT>(p, st);                        \
         } while (0)
         if (s_dtype == LLMK_F16) LLMK_W4A8_MT(LLMK_F16);
