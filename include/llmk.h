@@ -117,8 +117,9 @@ int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, cons
  * ref: quantization/w4a8_kernel.py:317-448 */
 /* workspace: at least N*K bytes (the expanded int8 weights); with round16(N*K) +
  * llmk_gemm_workspace_bytes(M,N,K) bytes large M runs on the fast tile kernels.
- * Decode-size calls (small M, K <= 4096, group_int4 == 128, 16-byte aligned a and b_packed)
- * run one fused kernel that reads the packed words once and does not touch the workspace. */
+ * Decode-size calls (small M, group_int4 == 128, 16-byte aligned a and b_packed) run one fused
+ * kernel that reads the packed words once; it touches the workspace only for K > 4096 (fp32
+ * partial sums of the K ranges, ceil(K / 4096) * M * N * 4 bytes). */
 int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, const void* b_s,
                    int s_dtype, const int8_t* b_s4, const int8_t* b_z4, void* c, int c_dtype,
                    int64_t M, int64_t N, int64_t K, int group_int4,

@@ -34,7 +34,7 @@ __global__ void w4a8_expand_kernel(const int32_t* __restrict__ packed, const int
 
 
 // ------------------------------------------------------------------------------------------------------------
-// Fused decode-size kernel (M <= 64, K <= 4096, 128-wide second-level groups).  The packed words are streamed
+// Fused decode-size kernel (small M, 128-wide second-level groups, K in ranges of at most 4096 per workgroup).  The packed words are streamed
 // HBM -> registers -> LDS fully coalesced; each lane then picks the nibble of its column out of the words it
 // needs, and the dequantisation (q - z4) * s4 is moved out of the inner product:
 //     sum_k a_k (q_k - z) s = s (sum_k a_k q_k - z sum_k a_k)      per 128-K group,
@@ -48,6 +48,8 @@ __global__ void w4a8_expand_kernel(const int32_t* __restrict__ packed, const int
 struct W4A8Args {
     const int8_t* a; const void* a_s; const int32_t* packed; const void* b_s; const int8_t* s4; const int8_t* z4;
     void* c; int c_dtype; int M, N, K;
+    int Kc;             // K range of one workgroup (multiple of 128, at most 4096); gridDim.z ranges cover K
+    float* partial;     // more than one range: fp32 partial sums [gridDim.z][M][N], summed by a second kernel
 };
 
 template <int MT, int SDT, int ROUNDS>
@@ -60,7 +62,10 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4, col8 = r & 7, half = r >> 3;
-    const int M = p.M, N = p.N, K = p.K, steps = K >> 7;
+    // this workgroup's K range: elements [k0, k0 + K) of rows that are Kfull long
+    const int M = p.M, N = p.N, Kfull = p.K, sfull = Kfull >> 7;
+    const int k0 = (int)blockIdx.z * p.Kc, sk0 = k0 >> 7;
+    const int K = min(p.Kc, Kfull - k0), steps = K >> 7;
     const int m0 = blockIdx.y * 16 * MT;
     const int ntiles = (N + 15) >> 4, np = N >> 3;
     // wave w multiplies the `cs` consecutive 128-K steps from w * cs: its zero points and second-level scales
@@ -80,7 +85,7 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
             const int prow = live ? min(tile * 2 + hh, np - 1) : 0;
-            const uint8_t* rowp = (const uint8_t*)p.packed + (int64_t)prow * K * 4;
+            const uint8_t* rowp = (const uint8_t*)p.packed + ((int64_t)prow * Kfull + k0) * 4;
 #pragma unroll
             for (int rd = 0; rd < ROUNDS; ++rd) {
                 const uint32_t off = (uint32_t)(rd * 8192 + wave * 1024 + lane * 16);
@@ -88,8 +93,8 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
             }
         }
         const int n = live ? min(tile * 16 + r, N - 1) : 0;
-        // dword at byte n * steps + ks0 of each table, pulled back inside the table at its very end
-        const int64_t want = (int64_t)n * steps + ks0, last = (int64_t)N * steps - 4;
+        // dword at byte n * (K / 128) + first step of this wave, pulled back inside the table at its very end
+        const int64_t want = (int64_t)n * sfull + sk0 + ks0, last = (int64_t)N * sfull - 4;
         const int64_t at = min(want, last);
         const int sh = (int)(want - at) * 8;
         unsigned zw, sw;
@@ -97,7 +102,7 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
         __builtin_memcpy(&sw, p.s4 + at, 4);
         t.z = sh < 32 ? zw >> sh : 0u;
         t.s = sh < 32 ? sw >> sh : 0u;
-        const int64_t bsrow = (int64_t)((min(tile, ntiles - 1) * 16) >> 7) * steps;
+        const int64_t bsrow = (int64_t)((min(tile, ntiles - 1) * 16) >> 7) * sfull + sk0;
         const int kb = min(ks0 + (lane & 3), steps - 1);
         if constexpr (SDT == LLMK_F32) t.bs = __float_as_uint(((const float*)p.b_s)[bsrow + kb]);
         else t.bs = ((const unsigned short*)p.b_s)[bsrow + kb];
@@ -120,8 +125,8 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
         for (int mt = 0; mt < MT; ++mt) {
             const int ks = min(ks0 + u, steps - 1);
             const int arow = min(m0 + 16 * mt + r, M - 1);
-            afrag[u][mt] = ld_split((const uint8_t*)p.a + (int64_t)arow * K + 16 * g + (int64_t)ks * 128);
-            ascale[u][mt] = ScaleIO<SDT>::cvt(((const typename ScaleIO<SDT>::Raw*)p.a_s)[(int64_t)arow * steps + ks]);
+            afrag[u][mt] = ld_split((const uint8_t*)p.a + (int64_t)arow * Kfull + k0 + 16 * g + (int64_t)ks * 128);
+            ascale[u][mt] = ScaleIO<SDT>::cvt(((const typename ScaleIO<SDT>::Raw*)p.a_s)[(int64_t)arow * sfull + sk0 + ks]);
         }
 
     int tile = blockIdx.x;
@@ -283,7 +288,8 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
             float sum = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) sum += rbuf[w * MT * 256 + src];
-            st_out(p.c, (int64_t)m * N + n, sum, p.c_dtype);
+            if (p.partial) p.partial[((int64_t)blockIdx.z * M + m) * N + n] = sum;
+            else st_out(p.c, (int64_t)m * N + n, sum, p.c_dtype);
         }
         clear_acc();
     };
@@ -305,8 +311,17 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
 }
 
 template <int MT, int SDT>
-int launch_w4a8_stream(const W4A8Args& p, hipStream_t st) {
-    const int steps = p.K >> 7, rounds = p.K * 4 > 8192 ? 2 : 1;
+int launch_w4a8_stream(W4A8Args p, void* workspace, int64_t workspace_bytes, hipStream_t st) {
+    // K ranges of at most 4096 elements, equally long up to one step
+    const int steps_all = p.K >> 7, nz = (steps_all + 31) / 32;
+    p.Kc = ((steps_all + nz - 1) / nz) * 128;
+    p.partial = nullptr;
+    if (nz > 1) {
+        if (!workspace || workspace_bytes < (int64_t)nz * p.M * p.N * 4 || (((uintptr_t)workspace) & 15))
+            LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a8: K > 4096 needs %lld bytes of 16-byte aligned workspace", (long long)nz * p.M * p.N * 4);
+        p.partial = (float*)workspace;
+    }
+    const int steps = p.Kc >> 7, rounds = p.Kc * 4 > 8192 ? 2 : 1;
     const int ntiles = (p.N + 15) >> 4, mtiles = (p.M + 16 * MT - 1) / (16 * MT);
     const size_t smem = (size_t)2 * 8 * MT * 256 * 4 + (size_t)MT * 16 * steps * 8 + (size_t)2 * 2 * (rounds * 8192 + 64);
     auto k1 = w4a8_stream_kernel<MT, SDT, 1>;
@@ -324,11 +339,20 @@ int launch_w4a8_stream(const W4A8Args& p, hipStream_t st) {
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot query the device");
     }
-    const int gx = min(ntiles, max(1, cus / min(mtiles, cus)));        // one workgroup per CU (LDS bound)
-    dim3 grid((unsigned)gx, (unsigned)mtiles);
+    const int rows = mtiles * nz;                                      // workgroup rows that share the column tiles
+    const int gx = min(ntiles, max(1, cus / min(rows, cus)));          // one workgroup per CU (LDS bound)
+    dim3 grid((unsigned)gx, (unsigned)mtiles, (unsigned)nz);
     if (rounds == 1) k1<<<grid, 512, smem, st>>>(p);
     else k2<<<grid, 512, smem, st>>>(p);
     LLMK_CHECK_LAUNCH("gemm_w4a8(stream)");
+    if (nz > 1) {
+        const int64_t mn = (int64_t)p.M * p.N;
+        const unsigned blocks = (unsigned)cdiv64(cdiv64(mn, 4), 256);
+        if (p.c_dtype == LLMK_BF16) splitk_sum_kernel<LLMK_BF16><<<blocks, 256, 0, st>>>(p.partial, p.c, mn, nz);
+        else if (p.c_dtype == LLMK_F16) splitk_sum_kernel<LLMK_F16><<<blocks, 256, 0, st>>>(p.partial, p.c, mn, nz);
+        else splitk_sum_kernel<LLMK_F32><<<blocks, 256, 0, st>>>(p.partial, p.c, mn, nz);
+        LLMK_CHECK_LAUNCH("gemm_w4a8(sum)");
+    }
     return LLMK_OK;
 }
 
@@ -347,15 +371,18 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
     const double x = (double)N * (double)K / (4096.0 * 4096.0);
     const int64_t row_blocks = (M + 31) / 32;
     const bool fused_wins = row_blocks <= 2 || (row_blocks == 3 && x <= 3.0) || (row_blocks == 4 && x <= 2.0);
-    if (fused_wins && K <= 4096 && group_int4 == 128 && !(((uintptr_t)a | (uintptr_t)b_packed) & 15)) {
-        W4A8Args p{a, a_s, b_packed, b_s, b_s4, b_z4, c, c_dtype, (int)M, (int)N, (int)K};
+    // K > 4096 runs as ranges of at most 4096 with fp32 partial sums in the workspace (up to 64 rows)
+    const int64_t nz = (K / 128 + 31) / 32;
+    const bool long_k_ok = nz == 1 || (row_blocks <= 2 && workspace && workspace_bytes >= nz * M * N * 4 && !(((uintptr_t)workspace) & 15));
+    if (fused_wins && long_k_ok && group_int4 == 128 && !(((uintptr_t)a | (uintptr_t)b_packed) & 15)) {
+        W4A8Args p{a, a_s, b_packed, b_s, b_s4, b_z4, c, c_dtype, (int)M, (int)N, (int)K, 0, nullptr};
         if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: c_dtype %d", c_dtype);
         hipStream_t st = (hipStream_t)stream;
 #define LLMK_W4A8_MT(SDT)                                                    \
         do {                                                                 \
             /* 16-row workgroups side by side win while the weights are small, 32-row ones beyond */ \
-            if (M <= 16 || N * K <= ((int64_t)20 << 20)) return launch_w4a8_stream<1, SDT>(p, st); \
-            return launch_w4a8_stream<2, SDT>(p, st);                        \
+            if (M <= 16 || N * K <= ((int64_t)20 << 20)) return launch_w4a8_stream<1, SDT>(p, workspace, workspace_bytes, st); \
+            return launch_w4a8_stream<2, SDT>(p, workspace, workspace_bytes, st); \
         } while (0)
         if (s_dtype == LLMK_F16) LLMK_W4A8_MT(LLMK_F16);
         if (s_dtype == LLMK_BF16) LLMK_W4A8_MT(LLMK_BF16);

@@ -122,7 +122,7 @@ def test_int8_per_token_int32_bit_exact(dev, M, N, K):
 # ------------------------------------------------------------------------------------------- w4a8
 @pytest.mark.parametrize("M,N,K", [(1, 128, 128), (16, 256, 512), (37, 136, 256), (16, 4096, 4096), (128, 1024, 7168),
                                    (5, 8, 128), (33, 264, 2048), (64, 4096, 4096), (17, 1032, 2176), (16, 14336, 4096),
-                                   (16, 512, 4224)])
+                                   (16, 512, 4224), (16, 4096, 14336), (64, 520, 12416)])
 def test_w4a8_gemm(dev, M, N, K):
     announce("w4a8_gemm", M, N, K)
     torch.manual_seed(N + K)
@@ -158,7 +158,8 @@ def test_w4a8_exact_and_wrap(dev):
 
 
 @pytest.mark.parametrize("M,N,K,sdt", [(16, 5000, 1024, torch.float16), (40, 8192, 4096, torch.float32),
-                                       (3, 312, 384, torch.bfloat16)])
+                                       (3, 312, 384, torch.bfloat16), (16, 1032, 8320, torch.float16),
+                                       (50, 264, 14336, torch.float32)])
 def test_w4a8_decode_exact_mixed_wrap(dev, M, N, K, sdt):
     """Decode-size shapes over many column tiles with a sprinkle of out-of-contract (s4, z4): exact integers."""
     announce("w4a8 decode exact", M, N, K, sdt)
