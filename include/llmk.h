@@ -140,7 +140,8 @@ int llmk_gemm_w4a16_marlin(const void* a_f16, const int32_t* b, void* c_f16, con
                            void* workspace, int64_t workspace_bytes, void* stream);
 /* Same product for W stored [N, K/8] int32 by pack_weights_over_cols (nibble i of a word = k*8+i)
  * with s fp16 [N, K/g]; a/c fp16 or bf16 (dtype code).  fp16 only at present.  workspace is optional:
- * with N*K*2 bytes (16-byte aligned) M > 64 runs as dequantise + tiled MFMA GEMM. */
+ * with N*K*2 bytes (16-byte aligned) M > 64 runs as dequantise + tiled MFMA GEMM; with
+ * ceil(K/4096)*M*N*4 bytes M <= 64, K > 4096 runs as K ranges with fp32 partial sums. */
 int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s_f16,
                        int ac_dtype, int64_t M, int64_t N, int64_t K, int groupsize,
                        void* workspace, int64_t workspace_bytes, void* stream);

@@ -307,20 +307,23 @@ __global__ void nk_dequant_kernel(const int32_t* __restrict__ B, const _Float16*
 template <int MT, int NT, bool RESIDENT, bool VS = false>
 __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     const _Float16* __restrict__ A, const int32_t* __restrict__ B, const _Float16* __restrict__ S,
-    _Float16* __restrict__ C, int M, int N, int K, int groupsize) {
+    _Float16* __restrict__ C, int M, int N, int Kfull, int groupsize, int Kc, float* __restrict__ partial) {
     constexpr int NW = 8;
     constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
     extern __shared__ float red[];                       // [2][NW][NT][MT][64][4]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, g = lane >> 4;
-    const int steps = K >> 7, ngroups = K / groupsize, kwords = K >> 3;
+    // K range [k0, k0 + K) of this workgroup (gridDim.z ranges of Kc cover rows that are Kfull long; with more
+    // than one range the outputs are fp32 partial sums for a summing pass)
+    const int k0 = (int)blockIdx.z * Kc, K = min(Kc, Kfull - k0);
+    const int steps = K >> 7, ngroups = Kfull / groupsize, kwords = Kfull >> 3;
     const int m0 = blockIdx.y * 16 * MT;
     const int ntiles = (N + 16 * NT - 1) / (16 * NT);    // a tile is NT adjacent 16-column blocks
 
     const _Float16* arow[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (int64_t)min(m0 + 16 * mt + r, M - 1) * K + 32 * g;
+    for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (int64_t)min(m0 + 16 * mt + r, M - 1) * Kfull + k0 + 32 * g;
 
     struct BBatch {
         v4i w[NT][U];
@@ -337,7 +340,7 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const int nrow = min((tile * NT + nt) * 16 + r, N - 1);
-            const int32_t* brow = B + (int64_t)nrow * kwords + 4 * g;
+            const int32_t* brow = B + (int64_t)nrow * kwords + (k0 >> 3) + 4 * g;
 #pragma unroll
             for (int u = 0; u < U; ++u) t.w[nt][u] = *(const v4i*)(brow + clamp_step(step_of(ks0, u)) * 16);
         }
@@ -347,12 +350,12 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
             const unsigned short* srow = (const unsigned short*)S + (int64_t)nrow * ngroups;
             if constexpr (VS) {
                 static_assert(U == 4, "four scales per load");
-                const uint2 q = *(const uint2*)(srow + min(step_of(ks0, 0), steps - U));
+                const uint2 q = *(const uint2*)(srow + (k0 >> 7) + min(step_of(ks0, 0), steps - U));
                 t.s[nt][0] = (unsigned short)q.x; t.s[nt][1] = (unsigned short)(q.x >> 16);
                 t.s[nt][2] = (unsigned short)q.y; t.s[nt][3] = (unsigned short)(q.y >> 16);
             } else {
 #pragma unroll
-                for (int u = 0; u < U; ++u) t.s[nt][u] = srow[(clamp_step(step_of(ks0, u)) * 128) / groupsize];
+                for (int u = 0; u < U; ++u) t.s[nt][u] = srow[(k0 + clamp_step(step_of(ks0, u)) * 128) / groupsize];
             }
         }
     };
@@ -445,7 +448,8 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
             float v = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) v += rbuf[w * NB * 256 + src];
-            C[(int64_t)m * N + n] = (_Float16)v;
+            if (partial) partial[((int64_t)blockIdx.z * M + m) * N + n] = v;
+            else C[(int64_t)m * N + n] = (_Float16)v;
         }
         clear_acc();
     };
@@ -492,9 +496,11 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
 
 template <int MT, int NT>
 int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Float16* C, int M, int N, int K, int groupsize,
-                     hipStream_t st) {
+                     int nz, float* partial, hipStream_t st) {
     constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
-    const int steps = K >> 7, ntiles = (N + 16 * NT - 1) / (16 * NT), mtiles = (M + 16 * MT - 1) / (16 * MT);
+    // nz K ranges, equally long up to one step
+    const int steps_all = K >> 7, steps = (steps_all + nz - 1) / nz, Kc = steps * 128;
+    const int ntiles = (N + 16 * NT - 1) / (16 * NT), mtiles = (M + 16 * MT - 1) / (16 * MT);
     const bool resident = steps <= 8 * U;
     const size_t smem = (size_t)2 * 8 * NT * MT * 256 * sizeof(float);
     static int slots[2] = {0, 0};
@@ -508,20 +514,28 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a16_nk: occupancy query failed: %s", hipGetErrorString(e));
         slots[resident] = max(1, cus * max(1, per_cu));
     }
-    const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
-    dim3 grid((unsigned)gx, (unsigned)mtiles);
+    const int rows = mtiles * nz;
+    const int gx = min(ntiles, max(1, slots[resident] / min(rows, slots[resident])));
+    dim3 grid((unsigned)gx, (unsigned)mtiles, (unsigned)nz);
+    float* part = nz > 1 ? partial : nullptr;
+    bool launched = false;
     if constexpr (U == 4) {
         // consecutive steps per wave and one load for their four scales
-        if (groupsize == 128 && steps % 4 == 0 && !(((uintptr_t)S) & 7)) {
-            if (resident) w4a16_nk_stream_kernel<MT, NT, true, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
-            else w4a16_nk_stream_kernel<MT, NT, false, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
-            LLMK_CHECK_LAUNCH("gemm_w4a16_nk(stream)");
-            return LLMK_OK;
+        if (groupsize == 128 && steps_all % 4 == 0 && steps % 4 == 0 && !(((uintptr_t)S) & 7)) {
+            if (resident) w4a16_nk_stream_kernel<MT, NT, true, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize, Kc, part);
+            else w4a16_nk_stream_kernel<MT, NT, false, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize, Kc, part);
+            launched = true;
         }
     }
-    if (resident) w4a16_nk_stream_kernel<MT, NT, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
-    else w4a16_nk_stream_kernel<MT, NT, false><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize);
+    if (!launched) {
+        if (resident) w4a16_nk_stream_kernel<MT, NT, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize, Kc, part);
+        else w4a16_nk_stream_kernel<MT, NT, false><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize, Kc, part);
+    }
     LLMK_CHECK_LAUNCH("gemm_w4a16_nk(stream)");
+    if (nz > 1) {
+        splitk_reduce_f16_kernel<<<(unsigned)cdiv64((int64_t)M * N, 4 * 256), 256, 0, st>>>(partial, C, (int64_t)M * N, nz);
+        LLMK_CHECK_LAUNCH("gemm_w4a16_nk(reduce)");
+    }
     return LLMK_OK;
 }
 
@@ -643,9 +657,15 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
         // one 16-column block per tile: two blocks per tile (NT = 2) measured slower at every shape tried.
         // While the activations of a 16-row workgroup stay resident (K <= 4096), such workgroups side by side
         // beat taller ones by up to 2x.
-        if (M <= 16 || K <= 4096) return launch_nk_stream<1, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
-        if (M <= 32) return launch_nk_stream<2, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
-        return launch_nk_stream<4, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, st);
+        // K > 4096: ranges of at most 4096 (each with resident activations) and fp32 partial sums, when the
+        // workspace holds them
+        const int nz = (int)((K / 128 + 31) / 32);
+        const bool ranges = nz > 1 && (M * N) % 4 == 0 && K % groupsize == 0 && ((K / 128 + nz - 1) / nz * 128) % groupsize == 0 &&
+                            workspace && workspace_bytes >= (int64_t)nz * M * N * 4 && !((uintptr_t)workspace & 15) && !((uintptr_t)c & 7);
+        if (ranges) return launch_nk_stream<1, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, nz, (float*)workspace, st);
+        if (M <= 16 || K <= 4096) return launch_nk_stream<1, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, 1, nullptr, st);
+        if (M <= 32) return launch_nk_stream<2, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, 1, nullptr, st);
+        return launch_nk_stream<4, 1>(A, b_packed, S, C, (int)M, (int)N, (int)K, groupsize, 1, nullptr, st);
     }
     const unsigned gx = (unsigned)cdiv64(N, 16);
     if (M <= 16) {

@@ -32,7 +32,12 @@ def w4a16_gemm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, gr
     N = w_packed.size(0)
     assert w_packed.size(1) * 8 == K, 'packed weight must be [N, K/8]'
     y = x.new_empty(*x.size()[:-1], N)
-    ws = _lib.workspace(x.device, N * K * 2) if M > 64 else None      # fp16 copy of W for the compute-bound path
+    if M > 64:
+        ws = _lib.workspace(x.device, N * K * 2)          # fp16 copy of W for the compute-bound path
+    elif K > 4096:
+        ws = _lib.workspace(x.device, -(-K // 4096) * M * N * 4)   # fp32 partial sums of the K ranges
+    else:
+        ws = None
     _lib.call("llmk_gemm_w4a16_nk", _lib.ptr(x), _lib.ptr(w_packed), _lib.ptr(y), _lib.ptr(scales),
               _lib.dt(x.dtype), M, N, K, group_size, _lib.ptr(ws), ws.numel() if ws is not None else 0,
               _lib.stream(x), exc=AssertionError)

@@ -91,7 +91,8 @@ def test_mul_error_behaviour(dev):
 @pytest.mark.parametrize("M,N,K,gs", [(16, 4096, 4096, 128), (1, 64, 128, 128), (7, 100, 256, 64), (16, 256, 512, 32),
                                       (40, 512, 1024, 128), (16, 128, 384, -1), (16, 28672, 4096, 128), (16, 1000, 14336, 128),
                                       (3, 8200, 4096, 256), (32, 4100, 2048, 128), (64, 520, 8192, 128), (33, 4096, 512, 512),
-                                      (300, 1000, 512, 64), (4096, 4096, 256, 128)])
+                                      (300, 1000, 512, 64), (4096, 4096, 256, 128), (48, 1000, 12416, 128), (1, 4096, 14336, 128),
+                                      (64, 264, 8448, 256), (20, 129, 4224, 128), (16, 264, 8320, 128)])
 def test_w4a16_nk(dev, M, N, K, gs):
     announce("w4a16 nk", M, N, K, gs)
     torch.manual_seed(0)
