@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from oracle import gemm_ref as g, quant_ref as q, bitpack_ref as bp
+from llm_kernels_amd import _lib
 from llm_kernels_amd.quantization import fp8_kernel, int8_kernel, w4a8_kernel
 from helpers import announce, assert_close_scaled, default_dtype
 
@@ -203,6 +204,24 @@ def test_mid_m_split_k_shapes(dev, kind, M, N, K, out):
             c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
     assert c.dtype == out
     assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="split-K " + kind)
+
+
+def test_fp8_gemm_without_scratch_takes_the_streaming_kernel(dev):
+    """The scratch is optional: the same call without it runs another kernel and agrees with the oracle too."""
+    announce("fp8 no scratch")
+    torch.manual_seed(5)
+    M, N, K = 48, 2560, 8192
+    a, a_s = q.act_quant_fp8(torch.randn(M, K).bfloat16())
+    b, b_s = q.weight_quant_fp8(torch.randn(N, K) * 0.02)
+    ad, asd, bd, bsd = a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev)
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    _lib.call("llmk_gemm_fp8_block", _lib.ptr(ad), _lib.ptr(asd), _lib.ptr(bd), _lib.ptr(bsd), _lib.ptr(c),
+              _lib.dt(c.dtype), M, N, K, None, 0, _lib.stream(ad))
+    ref = g.gemm_blockwise(a, a_s, b, b_s)
+    assert_close_scaled(c, ref, what="fp8 without scratch")
+    with default_dtype(torch.bfloat16):
+        c2 = fp8_kernel.fp8_gemm(ad, asd, bd, bsd)
+    assert_close_scaled(c2, ref, what="fp8 with scratch")
 
 
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
