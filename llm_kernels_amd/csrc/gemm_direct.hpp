@@ -215,18 +215,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     int tile = blockIdx.x;
     ABatch acur, anxt;
     BBatch bcur, bnxt, bnx2;
-    if (steps > 0 && tile < ntiles) {
-        load_b(bcur, tile, wave);
-        load_a(acur, wave);
-    }
+    // Request order: activation scales, activations (both mostly L2 hits), then the first weight batch (HBM).
+    // Loads return in order, so the scale table is written and published while the weights are still on
+    // their way.
+    SRaw stage_as[4];
     if constexpr (BLOCKSCALE) {
-        SRaw stage_as[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int idx = (int)threadIdx.x + q * NW * 64;
             stage_as[q] = 0;
             if (idx < n_as) stage_as[q] = ((const SRaw*)p.a_s)[as_base + min(idx, n_as_valid - 1)];
         }
+    }
+    if (steps > 0 && tile < ntiles) {
+        load_a(acur, wave);
+        load_b(bcur, tile, wave);
+    }
+    if constexpr (BLOCKSCALE) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int idx = (int)threadIdx.x + q * NW * 64;

@@ -416,8 +416,9 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     ABatch acur, anxt;
     BBatch bcur, bnxt, bnx2;
     if (tile < ntiles) {
-        load_b(bcur, tile, wave);
+        // activations first (mostly L2 hits): they are permuted while the weights are still on their way
         load_a(acur, wave);
+        load_b(bcur, tile, wave);
         if (RESIDENT && tile + stride < ntiles) load_b(bnxt, tile + stride, wave);
         __builtin_amdgcn_sched_barrier(0);
         if (RESIDENT) perm_a(acur);
