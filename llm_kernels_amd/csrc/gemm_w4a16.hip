@@ -565,7 +565,11 @@ MarlinPlan marlin_plan(int64_t M, int64_t N, int64_t K) {
 
 extern "C" int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    if (M > 64) return K % 64 == 0 ? N * K * 2 : 0;      // dequantised fp16 copy of W for the tiled GEMM
+    if (M > 64) {                                        // dequantised fp16 copy of W for the tiled GEMM (+ split-K partials)
+        if (K % 64) return 0;
+        const int z = llmk::splitk_factor_half(M, N, K);
+        return ((N * K * 2 + 255) & ~(int64_t)255) + (z > 1 ? (int64_t)z * M * N * 4 : 0);
+    }
     const MarlinPlan pl = marlin_plan(M, N, K);
     return pl.z > 1 ? (int64_t)pl.z * M * N * 4 : 0;
 }
@@ -596,7 +600,9 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
             dim3 dgrid((unsigned)(N / 64), (unsigned)cdiv64(K, 128));
             marlin_dequant_kernel<<<dgrid, 256, 0, st>>>((const v4i*)b, (const _Float16*)s, (_Float16*)workspace, (int)N, (int)K, groupsize);
             LLMK_CHECK_LAUNCH("gemm_w4a16_marlin(dequant)");
-            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_marlin(tiled)");
+            const int64_t used = (N * K * 2 + 255) & ~(int64_t)255;
+            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_marlin(tiled)", (uint8_t*)workspace + used,
+                                                             workspace_bytes > used ? workspace_bytes - used : 0);
         }
     }
     MarlinPlan pl = marlin_plan(M, N, K);
@@ -651,7 +657,9 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
         if (llmk::dma_eligible(p, 2)) {
             nk_dequant_kernel<<<(unsigned)cdiv64(N * (K / 8), 256), 256, 0, st>>>(b_packed, S, (_Float16*)workspace, N, K, groupsize);
             LLMK_CHECK_LAUNCH("gemm_w4a16_nk(dequant)");
-            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_nk(tiled)");
+            const int64_t used = (N * K * 2 + 255) & ~(int64_t)255;
+            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_nk(tiled)", (uint8_t*)workspace + used,
+                                                             workspace_bytes > used ? workspace_bytes - used : 0);
         }
     }
     if (groupsize % 128 == 0 && M <= 64) {

@@ -328,10 +328,20 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
     return launch_dma<KIND, GROUPED>(p, stream, name);
 }
 
-// fp16 / bf16 operands, no scales (K % 64 == 0)
+// K slices for the half-precision tile kernel (a K step is 64 elements there): same rule as splitk_factor
+inline int splitk_factor_half(int64_t M, int64_t N, int64_t K) { return splitk_factor(M, N, 2 * K); }
+
+// fp16 / bf16 operands, no scales (K % 64 == 0); `workspace` (optional) holds the fp32 split-K partials
 template <int KIND, bool GROUPED>
-int launch_big_half(const DirectArgs& p, hipStream_t stream, const char* name) {
+int launch_big_half(DirectArgs p, hipStream_t stream, const char* name, void* workspace = nullptr, int64_t workspace_bytes = 0) {
     if (!dma_eligible(p, 2)) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: shape not supported by the tiled half-precision kernel", name);
+    if constexpr (!GROUPED) {
+        const int z = splitk_factor_half(p.M, p.N, p.K);
+        if (z > 1 && workspace && workspace_bytes >= (int64_t)z * p.M * p.N * 4 && !(((uintptr_t)workspace) & 15)) {
+            p.partial = (float*)workspace;
+            p.ksplit = z;
+        }
+    }
     return launch_dma<KIND, GROUPED>(p, stream, name);
 }
 

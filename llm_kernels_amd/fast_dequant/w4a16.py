@@ -33,7 +33,8 @@ def w4a16_gemm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, gr
     assert w_packed.size(1) * 8 == K, 'packed weight must be [N, K/8]'
     y = x.new_empty(*x.size()[:-1], N)
     if M > 64:
-        ws = _lib.workspace(x.device, N * K * 2)          # fp16 copy of W for the compute-bound path
+        # fp16 copy of W for the compute-bound path, split-K partials behind it for mid-size M
+        ws = _lib.workspace(x.device, ((N * K * 2 + 255) // 256) * 256 + (8 * M * N * 4 if M <= 512 else 0))
     elif K > 4096:
         ws = _lib.workspace(x.device, -(-K // 4096) * M * N * 4)   # fp32 partial sums of the K ranges
     else:
