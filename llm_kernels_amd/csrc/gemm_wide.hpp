@@ -285,22 +285,20 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
     return M > 16 && M <= 64 && N * K >= (int64_t)20 << 20;
 }
 
-// More than this many 256 x 256 tiles: the 256 x 256 kernel.  Up to 128 such tiles the 256 x 128 kernel covers
-// the problem in one round of twice as many workgroups; beyond that it needs two rounds (about 2 x 40 us at
-// K = 4096) where the large tile needs one (about 64 us).
-constexpr int WIDE_MIN_TILES = 128;
-
-// Tile shape by occupancy: the largest tile (least operand re-reading) that still gives every CU a
-// workgroup.  Segments of a grouped GEMM are judged by their average length.
+// Tile shape by estimated time: rounds of 256 workgroups times the measured cost of one round of each tile
+// shape (microseconds at K = 4096 for fp8; the ratios hold for the other kinds and K).  Ties go to the larger
+// tile (less operand re-reading).  Segments of a grouped GEMM are judged by their average length.
 template <int KIND, bool GROUPED>
 int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
+    if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
-    auto wgs = [&](int bm, int bn) { return ((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm); };
-    if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
-    if (wgs(256, 256) > WIDE_MIN_TILES) return launch_wide<KIND, GROUPED>(p, stream, name);
-    if (wgs(256, 128) >= 256 || rows > 1024) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
-    if (wgs(128, 128) >= 256 || rows > 512) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
+    auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm) + 255) / 256; };
+    const double t_wide = 64.0 * rounds(256, 256), t4 = 43.0 * rounds(256, 128), t2 = 26.0 * rounds(128, 128),
+                 t1 = 16.0 * rounds(64, 128);
+    if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) return launch_wide<KIND, GROUPED>(p, stream, name);
+    if (t4 <= t2 && t4 <= t1) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
+    if (t2 <= t1) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
     return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
 }
 
