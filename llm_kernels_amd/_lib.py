@@ -128,20 +128,6 @@ def gemm_workspace(device, M, N, K):
     return ptr(buf), buf.numel()
 
 
-_zws = {}
-
-
-def zeroed_workspace(device, nbytes, tag):
-    """Per (device, stream, tag) scratch that starts zeroed and belongs to one kernel family only
-    (it carries self-resetting split-K ticket counters)."""
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream, tag)
-    buf = _zws.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.zeros(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
-        _zws[key] = buf
-    return buf
-
-
 _ws = {}
 
 
