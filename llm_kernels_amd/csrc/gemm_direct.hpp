@@ -398,7 +398,10 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
         slots[resident] = max(1, cus * max(1, per_cu));
     }
-    const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
+    // Grouped: most of the over-provisioned row tiles are empty and their workgroups leave at once, so every row
+    // tile gets a full set of column workgroups instead of a share.
+    const int gx = GROUPED ? min(ntiles, slots[resident])
+                           : min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
     dim3 grid((unsigned)gx, (unsigned)mtiles), block(NW * 64);
     if constexpr (CAN_VEC) {
         if (vec) {
