@@ -96,6 +96,13 @@ struct DirectArgs {
     int ksplit;            // 0 / 1 = no split
 };
 
+// Upper bound of the row tiles of a grouped GEMM (segment ends are only known on the device): every segment
+// adds at most one ragged tile, and no segment has more tiles than rows.
+inline int grouped_row_tiles(int M, int E, int tile_rows) {
+    const int64_t bound = ((int64_t)M + tile_rows - 1) / tile_rows + E;
+    return (int)(bound < M ? bound : M);
+}
+
 // SDT: dtype code of the block scales, fixed at compile time so that a scale load is a plain typed load with
 // no branch (and hence no wait for memory) between it and the loads around it.
 // VEC: the weight scales of a batch are one vector load (needs four steps per batch and steps % 4 == 0).
@@ -376,7 +383,7 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
     const int steps = p.K / (HALF ? 64 : 128);
     const int ntiles = (p.N + 15) / 16;
-    const int mtiles = (p.M + 16 * MT - 1) / (16 * MT) + (GROUPED ? p.E : 0);
+    const int mtiles = GROUPED ? grouped_row_tiles(p.M, p.E, 16 * MT) : (p.M + 16 * MT - 1) / (16 * MT);
     if (ntiles == 0 || mtiles == 0) return LLMK_OK;
     const size_t smem = (size_t)(MT == 4 ? 1 : 2) * NW * MT * 256 * sizeof(float) + (SCALED ? (size_t)MT * 16 * steps * sizeof(float) : 0);
     if (smem > 64 * 1024) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: K=%d too large for the weight-streaming kernel's scale table", name, p.K);
@@ -398,10 +405,7 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
         slots[resident] = max(1, cus * max(1, per_cu));
     }
-    // Grouped: most of the over-provisioned row tiles are empty and their workgroups leave at once, so every row
-    // tile gets a full set of column workgroups instead of a share.
-    const int gx = GROUPED ? min(ntiles, slots[resident])
-                           : min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
+    const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
     dim3 grid((unsigned)gx, (unsigned)mtiles), block(NW * 64);
     if constexpr (CAN_VEC) {
         if (vec) {

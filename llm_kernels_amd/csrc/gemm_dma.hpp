@@ -409,7 +409,7 @@ int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
         configured = true;
     }
     constexpr int BM = 64 * MI;
-    const int tiles_m = (p.M + BM - 1) / BM + (GROUPED ? p.E : 0);
+    const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, BM) : (p.M + BM - 1) / BM;
     const bool split = !GROUPED && p.ksplit > 1 && p.partial;
     dim3 grid((unsigned)((p.N + D_BN - 1) / D_BN), (unsigned)tiles_m, split ? (unsigned)p.ksplit : 1u);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;

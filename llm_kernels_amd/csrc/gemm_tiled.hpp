@@ -149,7 +149,7 @@ int launch_tiled_sdt(const DirectArgs& p, hipStream_t stream, const char* name) 
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, T_LDS, hipGetErrorString(e));
         configured = true;
     }
-    const int tiles_m = (p.M + T_BM - 1) / T_BM + (GROUPED ? p.E : 0);
+    const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, T_BM) : (p.M + T_BM - 1) / T_BM;
     dim3 grid((unsigned)((p.N + T_BN - 1) / T_BN), (unsigned)tiles_m);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
     kern<<<grid, T_THREADS, T_LDS, stream>>>(p);

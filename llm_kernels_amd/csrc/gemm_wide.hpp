@@ -258,7 +258,7 @@ int launch_wide(const DirectArgs& p, hipStream_t stream, const char* name) {
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, W_LDS, hipGetErrorString(e));
         configured = true;
     }
-    const int tiles_m = (p.M + W_BM - 1) / W_BM + (GROUPED ? p.E : 0);
+    const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, W_BM) : (p.M + W_BM - 1) / W_BM;
     dim3 grid((unsigned)((p.N + W_BN - 1) / W_BN), (unsigned)tiles_m);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
     kern<<<grid, W_THREADS, W_LDS, stream>>>(p);

@@ -317,7 +317,10 @@ extern "C" int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind
     // Tile kernels when the average segment is longer than 64 rows, and from two rows per expert up when the
     // expert weights are large (measured on 8 experts of 4096 x 14336, whole forward, tile vs weight-streaming
     // kernel: 256 vs 158 us at 1 token, 295 vs 289 us at 8, 344 vs 374 us at 16, 362 vs 481 us at 64).
-    const bool big = M > 64 * (int64_t)E || (M > 2 * (int64_t)E && N * K >= ((int64_t)20 << 20));
+    // Also with several short segments: the weight-streaming kernel spreads its workgroups over the row tiles and
+    // leaves each of them a fraction of the column workgroups (measured: tile kernels faster from six row tiles).
+    const bool big = M > 64 * (int64_t)E || (M > 2 * (int64_t)E && N * K >= ((int64_t)20 << 20)) ||
+                     grouped_row_tiles((int)M, E, 16) >= 6;
     if (big && kind == LLMK_KIND_I8) return launch_big<K_I8_BLOCK, true>(p, workspace, workspace_bytes, st, "grouped_gemm(i8, tiled)");
     if (big && kind == LLMK_KIND_FP8) return launch_big<K_FP8_BLOCK, true>(p, workspace, workspace_bytes, st, "grouped_gemm(fp8, tiled)");
     if (big && kind == LLMK_KIND_F16 && dma_eligible(p, 2)) return launch_big_half<K_F16, true>(p, st, "grouped_gemm(f16, tiled)");
