@@ -235,6 +235,8 @@ class Case:
 
 
 WORKLOADS = {}
+for _op in ("fp8", "w4a16_nk"):                 # Llama-3 lm_head at decode size
+    WORKLOADS["%s_m16_n128256_k4096" % _op] = (_op, 16, 128256, 4096)
 for _op in ("fp8", "int8", "w4a8", "w4a16", "w4a16_nk"):
     for _M in (1, 16, 128, 256, 1024, 4096):
         for _N, _K in ((4096, 4096), (6144, 4096), (14336, 4096), (28672, 4096), (4096, 14336)):
@@ -243,6 +245,7 @@ for _op in ("fp8", "int8", "w4a8", "w4a16", "w4a16_nk"):
 MOE_WORKLOADS = {"moe_mixtral_fp8_t4096": "fp8", "moe_mixtral_int8_t4096": "int8"}
 DEFAULT_WORKLOAD = "fp8_m4096_n4096_k4096"
 HEADLINE_SET = ["w4a16_m16_n4096_k4096", "w4a16_nk_m16_n4096_k4096", "w4a16_nk_m16_n28672_k4096", "fp8_m16_n4096_k4096", "fp8_m16_n28672_k4096", "fp8_m16_n4096_k14336",
+                "fp8_m16_n128256_k4096", "w4a16_nk_m16_n128256_k4096",
                 "w4a16_m4096_n4096_k4096", "w4a16_nk_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "w4a8_m16_n4096_k4096", "moe_mixtral_fp8_t4096"]
 
 
