@@ -59,7 +59,9 @@ __device__ __forceinline__ void reduce_waves(float (&acc)[NACC], float* buf, int
 // chunk half h = r >> 3; g = l >> 4 plays the role of the mma k-pair q.  One MFMA 16x16x32
 // step consumes two 16-K strips; MFMA (j, b) produces columns {64(2cp+h) + 16j + 8b + c}.
 // A fragment order per lane: k in {2g, 2g+1, 2g+8, 2g+9} of strip 0, then of strip 1.
-template <int MT, int NW, bool TO_WS>
+// A_LDS: the activations of the workgroup's K range are staged once in LDS, already in fragment order (one
+// 16-byte read per lane and step), instead of four 4-byte global loads per lane and step.
+template <int MT, int NW, bool TO_WS, bool A_LDS = false>
 __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
     const _Float16* __restrict__ A, const v4i* __restrict__ B, const _Float16* __restrict__ S,
     _Float16* __restrict__ C, float* __restrict__ ws, int M, int N, int K, int groupsize, int steps_per_z) {
@@ -84,6 +86,25 @@ __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
 #pragma unroll
     for (int i = 0; i < MT * 32; ++i) acc[i] = 0.f;
 
+    // LDS image of A for steps [ks_begin, ks_end): row-major over the tile rows, per step 64 bytes = four lane
+    // groups x {strip 0: k 2g, 2g+1 | 2g+8, 2g+9; strip 1: the same}; rows padded by 16 bytes (bank spread).
+    const int nst = max(ks_end - ks_begin, 0);
+    const int rstride = nst * 64 + 16;
+    uint8_t* alds = (uint8_t*)red;
+    if constexpr (A_LDS) {
+        const int chunks = 16 * MT * nst * 4;                // 16-byte pieces: (row, step, strip parity, k half)
+        for (int idx = threadIdx.x; idx < chunks; idx += NW * 64) {
+            const int row = idx / (nst * 4), rem = idx - row * (nst * 4), ks = rem >> 2, ch = rem & 3;
+            const int strip = 2 * (ks_begin + ks) + (ch >> 1);
+            v4i v = {0, 0, 0, 0};
+            if (strip < strips) v = *(const v4i*)(A + (int64_t)min(m0 + row, M - 1) * K + strip * 16 + (ch & 1) * 8);
+            uint8_t* dst = alds + row * rstride + ks * 64 + ch * 4;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *(int*)(dst + q * 16) = v[q];
+        }
+        __syncthreads();
+    }
+
     // Batches of U steps: every load of a batch (weights, scales, activations) is issued before the first
     // one is used, with clamped indices and no branch in between, so that a batch costs one memory round
     // trip.  Steps past the end of the range multiply by a zero activation fragment.
@@ -105,8 +126,12 @@ __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
             const int o1 = 2 * ks + 1 < strips ? 8 : 0;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                const unsigned* ap = (const unsigned*)(arow[mt] + 32 * ks);
-                x[u][mt] = (v4i){(int)ap[0], (int)ap[4], (int)ap[o1], (int)ap[o1 + 4]};
+                if constexpr (A_LDS) {
+                    x[u][mt] = *(const v4i*)(alds + (16 * mt + r) * rstride + (ks - ks_begin) * 64 + g * 16);
+                } else {
+                    const unsigned* ap = (const unsigned*)(arow[mt] + 32 * ks);
+                    x[u][mt] = (v4i){(int)ap[0], (int)ap[4], (int)ap[o1], (int)ap[o1 + 4]};
+                }
             }
         }
         __builtin_amdgcn_sched_barrier(0);       // keep every load above ahead of the first use below
@@ -141,6 +166,7 @@ __global__ __launch_bounds__(NW * 64) void w4a16_marlin_kernel(
 
     // one-barrier reduction over the waves: slot e of lane l of wave w sits at red[(w * NE + e) * 64 + l]
     constexpr int NE = MT * 32;
+    if constexpr (A_LDS) __syncthreads();                    // the reduction buffer reuses the activation image
 #pragma unroll
     for (int e = 0; e < NE; ++e) red[(wave * NE + e) * 64 + lane] = acc[e];
     __syncthreads();
@@ -616,10 +642,26 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
     _Float16* C = (_Float16*)c;
     float* ws = (float*)workspace;
     dim3 grid(pl.col_groups, pl.mblocks, pl.z), blk(pl.nw * 64);
-    const size_t smem = (size_t)pl.nw * pl.mt * 32 * 64 * sizeof(float);
+    const size_t red_bytes = (size_t)pl.nw * pl.mt * 32 * 64 * sizeof(float);
+    const size_t a_bytes = (size_t)16 * pl.mt * ((size_t)pl.steps_per_z * 64 + 16);     // activation image of one K range
+    // staged while every workgroup fits on the chip at once; with several rounds of workgroups the unoverlapped
+    // staging of each costs more than the global fragment loads (measured at N = 128256: 88 vs 84 us)
+    const bool a_lds = a_bytes <= 144 * 1024 && (int64_t)pl.col_groups * pl.mblocks * pl.z <= 512;
+    const size_t smem = a_lds && a_bytes > red_bytes ? a_bytes : red_bytes;
+    if (smem > 64 * 1024) {
+        static bool configured = false;
+        if (!configured) {
+            hipError_t e = hipFuncSetAttribute((const void*)w4a16_marlin_kernel<1, 8, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e == hipSuccess) e = hipFuncSetAttribute((const void*)w4a16_marlin_kernel<1, 8, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a16_marlin: cannot reserve LDS: %s", hipGetErrorString(e));
+            configured = true;
+        }
+    }
 #define LLMK_MARLIN_LAUNCH(MT, NW)                                                                              \
     do {                                                                                                        \
-        if (pl.z > 1) w4a16_marlin_kernel<MT, NW, true><<<grid, blk, smem, st>>>(A, B, S, C, ws, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
+        if (pl.z > 1 && a_lds) w4a16_marlin_kernel<MT, NW, true, true><<<grid, blk, smem, st>>>(A, B, S, C, ws, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
+        else if (pl.z > 1) w4a16_marlin_kernel<MT, NW, true><<<grid, blk, smem, st>>>(A, B, S, C, ws, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
+        else if (a_lds) w4a16_marlin_kernel<MT, NW, false, true><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
         else w4a16_marlin_kernel<MT, NW, false><<<grid, blk, smem, st>>>(A, B, S, C, nullptr, (int)M, (int)N, (int)K, groupsize, pl.steps_per_z); \
     } while (0)
     LLMK_MARLIN_LAUNCH(1, 8);
