@@ -36,6 +36,10 @@ def _bytes_i8(M, N, K):
     return M * K + N * K + 2 * M * kb + 2 * nb * kb + 2 * M * N
 
 
+def _bytes_i8_pt(M, N, K):
+    return M * K + N * K + 4 * M + 4 * N + 2 * M * N
+
+
 def _bytes_w4a16(M, N, K, g=128):
     return 2 * M * K + N * K // 2 + 2 * N * K // g + 2 * M * N
 
@@ -141,13 +145,13 @@ class Case:
     def __init__(self, name, op, M, N, K):
         self.name, self.op, self.M, self.N, self.K = name, op, M, N, K
         self.flops = 2.0 * M * N * K
-        self.bytes = {"fp8": _bytes_fp8, "int8": _bytes_i8, "w4a8": _bytes_w4a8}.get(op, None)
+        self.bytes = {"fp8": _bytes_fp8, "int8": _bytes_i8, "int8_pt": _bytes_i8_pt, "w4a8": _bytes_w4a8}.get(op, None)
         self.bytes = self.bytes(M, N, K) if self.bytes else _bytes_w4a16(M, N, K)
-        self.mfma_dtype = {"fp8": "fp8", "int8": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
+        self.mfma_dtype = {"fp8": "fp8", "int8": "int8", "int8_pt": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
         intensity = self.flops / self.bytes
         ridge = PEAK_TFLOPS[self.mfma_dtype] * 1e12 / (PEAK_HBM_GBS * 1e9)
         self.bound = "hbm" if intensity < ridge else "mfma"
-        self.dtype = {"fp8": "fp8_e4m3", "int8": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
+        self.dtype = {"fp8": "fp8_e4m3", "int8": "int8", "int8_pt": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
 
     # ---- device side
     def setup(self, dev):
@@ -157,7 +161,7 @@ class Case:
         from llm_kernels_amd.fast_dequant import w4a16
         M, N, K, op = self.M, self.N, self.K, self.op
         torch.manual_seed(0)
-        wbytes = {"fp8": N * K, "int8": N * K}.get(op, N * K // 2)
+        wbytes = {"fp8": N * K, "int8": N * K, "int8_pt": N * K}.get(op, N * K // 2)
         nbuf = 1 if self.bound == "mfma" else max(2, min(64, -(-CACHE_DEFEAT_BYTES // wbytes)))
         self.nbuf = nbuf
         x = torch.randn(M, K, device=dev)
@@ -173,6 +177,11 @@ class Case:
             b, b_s = int8_kernel.weight_quant(w)
             bs = [b.clone() for _ in range(nbuf)]
             self.launch = lambda i: int8_kernel.int8_gemm(a, a_s, bs[i % nbuf], b_s)
+        elif op == "int8_pt":               # per-token x per-channel scales, one int32 accumulation over K
+            a, a_s = int8_kernel.act_quant_per_token(x.bfloat16())
+            b, b_s = int8_kernel.weight_quant_per_channel(w)
+            bs = [b.clone() for _ in range(nbuf)]
+            self.launch = lambda i: int8_kernel.int8_gemm_per_token(a, a_s, bs[i % nbuf], b_s)
         elif op == "w4a8":
             a, a_s = w4a8_kernel.act_quant(x.bfloat16())
             b, b_s, s4, z4 = w4a8_kernel.weight_quant(w.half())
@@ -209,6 +218,13 @@ class Case:
                 ad = a.float() * a_s.repeat_interleave(128, 1)
                 bd = quant_ref.weight_dequant_block(b, b_s)
                 return ad @ bd.T
+        elif op == "int8_pt":
+            xf, wf = x.bfloat16().float(), w.float()
+            sa, sb = xf.abs().amax(1) / 127.0, wf.abs().amax(1) / 127.0
+            a, b = torch.round(xf / sa[:, None]).to(torch.int8), torch.round(wf / sb[:, None]).to(torch.int8)
+
+            def run():
+                return (a.float() * sa[:, None]) @ (b.float() * sb[:, None]).T
         elif op in ("int8", "w4a8"):
             a, a_s = quant_ref.act_quant_int8(x.bfloat16(), rounding="away" if op == "int8" else "up")
             if op == "int8":
@@ -237,7 +253,7 @@ class Case:
 WORKLOADS = {}
 for _op in ("fp8", "w4a16_nk"):                 # Llama-3 lm_head at decode size
     WORKLOADS["%s_m16_n128256_k4096" % _op] = (_op, 16, 128256, 4096)
-for _op in ("fp8", "int8", "w4a8", "w4a16", "w4a16_nk"):
+for _op in ("fp8", "int8", "int8_pt", "w4a8", "w4a16", "w4a16_nk"):
     for _M in (1, 16, 128, 256, 1024, 4096):
         for _N, _K in ((4096, 4096), (6144, 4096), (14336, 4096), (28672, 4096), (4096, 14336)):
             WORKLOADS["%s_m%d_n%d_k%d" % (_op, _M, _N, _K)] = (_op, _M, _N, _K)
@@ -348,7 +364,7 @@ def main():
     else:
         if args.workload not in WORKLOADS:
             # any other shape of a known operator, spelt like the registered names: <op>_m<M>_n<N>_k<K>
-            m = re.fullmatch(r"(fp8|int8|w4a8|w4a16|w4a16_nk)_m(\d+)_n(\d+)_k(\d+)", args.workload)
+            m = re.fullmatch(r"(fp8|int8|int8_pt|w4a8|w4a16|w4a16_nk)_m(\d+)_n(\d+)_k(\d+)", args.workload)
             if not m:
                 raise SystemExit("unknown workload %r" % args.workload)
             WORKLOADS[args.workload] = (m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4)))

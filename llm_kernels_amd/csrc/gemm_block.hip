@@ -15,12 +15,44 @@ int check_common(const char* name, const void* a, const void* b, int64_t M, int6
     return LLMK_OK;
 }
 
+// Decode-sized M with K beyond one resident batch per wave (32 steps): the weight-streaming kernel runs on
+// K ranges of at most 32 steps side by side (gridDim.z) and a second kernel adds their fp32 partial sums.
+inline int stream_k_ranges(int64_t M, int64_t N, int64_t K) {
+    if (M > 64 || K <= 4096 || mid_m_prefers_tiles(M, N, K)) return 1;
+    return (int)((K / 128 + 31) / 32);
+}
+
+template <int KIND>
+int launch_stream(DirectArgs& p, void* workspace, int64_t workspace_bytes, hipStream_t stream, const char* name) {
+    const int nz = stream_k_ranges(p.M, p.N, p.K);
+    const int64_t mn = (int64_t)p.M * p.N;
+    if (nz > 1 && workspace && workspace_bytes >= nz * mn * 4) {
+        const int steps = p.K / 128;
+        p.kc_steps = ((steps + nz - 1) / nz + 3) & ~3;         // even ranges, whole 4-step groups
+        p.partial = (float*)workspace;
+        p.ksplit = (steps + p.kc_steps - 1) / p.kc_steps;
+        int rc = launch_direct<KIND, false>(p, p.M, stream, name);
+        if (rc) return rc;
+        const unsigned blocks = (unsigned)((mn + 1023) / 1024);
+        if (p.c_dtype == LLMK_BF16) splitk_sum_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
+        else if (p.c_dtype == LLMK_F16) splitk_sum_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
+        else splitk_sum_kernel<LLMK_F32><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
+        LLMK_CHECK_LAUNCH(name);
+        return LLMK_OK;
+    }
+    return launch_direct<KIND, false>(p, p.M, stream, name);
+}
+
 }  // namespace
 
 extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     // large-M kernels stream fp32 activation scales; 16-bit scales are widened into the workspace first;
     // mid-size M with few tiles adds the fp32 split-K partials behind them
-    if (K <= 0 || (M <= 64 && !mid_m_prefers_tiles(M, N, K))) return 0;
+    if (K <= 0) return 0;
+    if (M <= 64 && !mid_m_prefers_tiles(M, N, K)) {
+        const int nz = stream_k_ranges(M, N, K);
+        return nz > 1 ? (int64_t)nz * M * N * 4 : 0;
+    }
     const int64_t scales = (M * (K / 128) * 4 + 255) & ~(int64_t)255;
     const int z = splitk_factor(M, N, K);
     return scales + (z > 1 ? (int64_t)z * M * N * 4 : 0);
@@ -38,7 +70,7 @@ extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* 
     p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
     if (M > 64 || (mid_m_prefers_tiles(M, N, K) && workspace && workspace_bytes >= llmk_gemm_workspace_bytes(M, N, K)))
         return launch_big<K_FP8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_fp8_block(tiled)");
-    return launch_direct<K_FP8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_fp8_block");
+    return launch_stream<K_FP8_BLOCK>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_fp8_block");
 }
 
 extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const void* b_s, int s_dtype,
@@ -54,7 +86,7 @@ extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t
     p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
     if (M > 64 || (mid_m_prefers_tiles(M, N, K) && workspace && workspace_bytes >= llmk_gemm_workspace_bytes(M, N, K)))
         return launch_big<K_I8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_i8_block(tiled)");
-    return launch_direct<K_I8_BLOCK, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_block");
+    return launch_stream<K_I8_BLOCK>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_i8_block");
 }
 
 extern "C" int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, const float* b_s, void* c,
@@ -67,5 +99,7 @@ extern "C" int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.c_i32 = c_i32; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+    // large M: the tile kernels accumulate int32 over the whole K range inside the MFMA and scale in the epilogue
+    if (M > 64 && dma_eligible(p)) return launch_dma<K_I8_ROWCOL, false>(p, (hipStream_t)stream, "gemm_i8_rowcol(tiled)");
     return launch_direct<K_I8_ROWCOL, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_rowcol");
 }

@@ -92,8 +92,9 @@ struct DirectArgs {
     const int64_t* weight_indices;  // grouped only
     int c_dtype, s_dtype;
     int M, N, K, E;
-    float* partial;        // split-K (dense tile kernel only): fp32 [ksplit][M][N] partial sums
+    float* partial;        // split-K: fp32 [ksplit][M][N] partial sums
     int ksplit;            // 0 / 1 = no split
+    int kc_steps;          // weight-streaming kernel with K ranges: 128-byte steps per range (gridDim.z ranges)
 };
 
 // Upper bound of the row tiles of a grouped GEMM (segment ends are only known on the device): every segment
@@ -106,8 +107,11 @@ inline int grouped_row_tiles(int M, int E, int tile_rows) {
 // SDT: dtype code of the block scales, fixed at compile time so that a scale load is a plain typed load with
 // no branch (and hence no wait for memory) between it and the loads around it.
 // VEC: the weight scales of a batch are one vector load (needs four steps per batch and steps % 4 == 0).
-template <int KIND, int MT, int NW, bool GROUPED, bool RESIDENT, int SDT, bool VEC = false>
+// KR: blockIdx.z selects a K range of p.kc_steps steps (short enough for RESIDENT); the workgroup writes its
+// fp32 sums to p.partial[blockIdx.z] and a second kernel adds the ranges.
+template <int KIND, int MT, int NW, bool GROUPED, bool RESIDENT, int SDT, bool VEC = false, bool KR = false>
 __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
+    static_assert(!KR || (RESIDENT && !GROUPED && !VEC), "K ranges: dense, resident activations");
     typedef typename ScaleIO<SDT>::Raw SRaw;
     constexpr bool HALF = (KIND == K_F16 || KIND == K_BF16);
     constexpr int ESZ = HALF ? 2 : 1;
@@ -119,7 +123,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: K-step indices stay scalar
     const int r = lane & 15, g = lane >> 4;
     const int K = p.K, N = p.N;
-    const int steps = K / KSTEP;
+    const int steps_all = K / KSTEP;                         // row length of the scale tables
+    const int kz0 = KR ? (int)blockIdx.z * p.kc_steps : 0;   // first step of this workgroup's K range
+    const int steps = KR ? min(p.kc_steps, steps_all - kz0) : steps_all;
 
     int m_start, m_end;
     const uint8_t* bbase = p.b;
@@ -149,8 +155,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int arow = min(m_start + 16 * mt + r, m_end - 1);
-        ap[mt] = p.a + ((int64_t)arow * K) * ESZ + 16 * g;
+        ap[mt] = p.a + ((int64_t)arow * K) * ESZ + 16 * g + (int64_t)kz0 * 128;
     }
+    if constexpr (KR) bbase += (int64_t)kz0 * 128;
 
     // A batch is U K-steps of this wave; all its loads are issued before any of them is consumed.  Steps
     // past the end are clamped to the last step and nullified.  When the whole K range of a wave fits in
@@ -175,7 +182,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
     auto load_b = [&](BBatch& t, int tile, int ks0) {
         const int nrow = min(tile * 16 + r, N - 1);
         const uint8_t* bp = bbase + ((int64_t)nrow * K) * ESZ + 16 * g;
-        const int64_t bs_row = bs_off + (int64_t)(tile * 16 / 128) * steps;
+        const int64_t bs_row = bs_off + (int64_t)(tile * 16 / 128) * steps_all + kz0;
         // all data loads first, then the scales as raw bits: nothing in here waits for memory
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -231,7 +238,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         for (int q = 0; q < 4; ++q) {
             const int idx = (int)threadIdx.x + q * NW * 64;
             stage_as[q] = 0;
-            if (idx < n_as) stage_as[q] = ((const SRaw*)p.a_s)[as_base + min(idx, n_as_valid - 1)];
+            if constexpr (KR) {       // the rows of a K range are not contiguous in a_s
+                const int row = idx / steps, k = idx - row * steps;
+                if (idx < n_as) stage_as[q] = ((const SRaw*)p.a_s)[(int64_t)min(m_start + row, m_end - 1) * steps_all + kz0 + k];
+            } else {
+                if (idx < n_as) stage_as[q] = ((const SRaw*)p.a_s)[as_base + min(idx, n_as_valid - 1)];
+            }
         }
     }
     if (steps > 0 && tile < ntiles) {
@@ -324,7 +336,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
                 float sum = 0.f;
 #pragma unroll
                 for (int w = 0; w < NW; ++w) sum += rbuf[w * MT * 256 + src];
-                st_out(p.c, (int64_t)m * N + n, sum, p.c_dtype);
+                if constexpr (KR) p.partial[((int64_t)blockIdx.z * p.M + m) * N + n] = sum;
+                else st_out(p.c, (int64_t)m * N + n, sum, p.c_dtype);
             }
         }
         if constexpr (RB == 1) __syncthreads();
@@ -385,6 +398,30 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
     const int ntiles = (p.N + 15) / 16;
     const int mtiles = GROUPED ? grouped_row_tiles(p.M, p.E, 16 * MT) : (p.M + 16 * MT - 1) / (16 * MT);
     if (ntiles == 0 || mtiles == 0) return LLMK_OK;
+    if constexpr (SCALED && !GROUPED && MT == 1) {
+        if (p.kc_steps > 0) {
+            // K ranges: every range fits one resident batch per wave; the caller adds the fp32 partial sums
+            if (p.kc_steps > NW * U || !p.partial) LLMK_FAIL(LLMK_ERR_ARG, "%s: bad K range setup", name);
+            const int nz = (steps + p.kc_steps - 1) / p.kc_steps;
+            const size_t smem_r = (size_t)2 * NW * 256 * sizeof(float) + (size_t)16 * p.kc_steps * sizeof(float);
+            static int slots_r = 0;
+            if (slots_r == 0) {
+                int dev = 0, cus = 0, per_cu = 0;
+                hipError_t e = hipGetDevice(&dev);
+                if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+                if (e == hipSuccess)
+                    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, 1, NW, false, true, SDT, false, true>, NW * 64, smem_r);
+                if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
+                slots_r = max(1, cus * max(1, per_cu));
+            }
+            const int rows = mtiles * nz;
+            const int gx = min(ntiles, max(1, slots_r / min(rows, slots_r)));
+            gemm_direct_kernel<KIND, 1, NW, false, true, SDT, false, true>
+                <<<dim3((unsigned)gx, (unsigned)mtiles, (unsigned)nz), dim3(NW * 64), smem_r, stream>>>(p);
+            LLMK_CHECK_LAUNCH(name);
+            return LLMK_OK;
+        }
+    }
     const size_t smem = (size_t)(MT == 4 ? 1 : 2) * NW * MT * 256 * sizeof(float) + (SCALED ? (size_t)MT * 16 * steps * sizeof(float) : 0);
     if (smem > 64 * 1024) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: K=%d too large for the weight-streaming kernel's scale table", name, p.K);
     // Column tiles are processed persistently by as many workgroups as are resident at once (so that every
@@ -442,7 +479,7 @@ int launch_direct(const DirectArgs& p, int max_rows_per_segment_hint, hipStream_
     // one m-tile per workgroup (activations resident in registers), 16-row workgroups side by side beat taller
     // ones that have to re-read their activations for every column tile.
     constexpr int KSTEP = (KIND == K_F16 || KIND == K_BF16) ? 64 : 128;
-    if (max_rows_per_segment_hint <= 16 || p.K / KSTEP <= 32) return launch_direct_mt<KIND, 1, GROUPED>(p, stream, name);
+    if (max_rows_per_segment_hint <= 16 || p.K / KSTEP <= 32 || p.kc_steps > 0) return launch_direct_mt<KIND, 1, GROUPED>(p, stream, name);
     if (max_rows_per_segment_hint <= 32) return launch_direct_mt<KIND, 2, GROUPED>(p, stream, name);
     return launch_direct_mt<KIND, 4, GROUPED>(p, stream, name);
 }

@@ -74,6 +74,68 @@ __device__ __forceinline__ void store_row16(void* c, int64_t off, const v4f (&v)
     }
 }
 
+// 16 consecutive int32 accumulators of one row -> memory
+__device__ __forceinline__ void store_row16_i32(int32_t* c, int64_t off, const v4f (&v)[4], int n_valid, bool vec_ok) {
+    if (vec_ok && n_valid >= 16) {
+        v4f* dst = (v4f*)(c + off);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[j] = v[j];          // raw bits
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (4 * j + q < n_valid) c[off + 4 * j + q] = __float_as_int(v[j][q]);
+    }
+}
+
+// Unscaled kinds accumulate inside the MFMA over the whole K range: two 16x16x32 half-precision MFMAs, or two
+// 16x16x64 int8 MFMAs whose int32 accumulators travel as raw bits in the fp32 accumulator registers.
+template <int KIND>
+__device__ __forceinline__ v4f mma_plain(const v8i& x, const v8i& y, v4f c) {
+    if constexpr (KIND == K_I8_ROWCOL) {
+        v4i ci;
+        __builtin_memcpy(&ci, &c, 16);
+        const v4i x0 = {x[0], x[1], x[2], x[3]}, x1 = {x[4], x[5], x[6], x[7]};
+        const v4i y0 = {y[0], y[1], y[2], y[3]}, y1 = {y[4], y[5], y[6], y[7]};
+        ci = mfma_i8_16x16x64(x0, y0, ci);
+        ci = mfma_i8_16x16x64(x1, y1, ci);
+        __builtin_memcpy(&c, &ci, 16);
+        return c;
+    } else if constexpr (KIND == K_F16) {
+        v8h x0, x1, y0, y1;
+        __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
+        __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
+        c = mfma_f16_16x16x32(x0, y0, c);
+        return mfma_f16_16x16x32(x1, y1, c);
+    } else {
+        v8bf x0, x1, y0, y1;
+        __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
+        __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
+        c = mfma_bf16_16x16x32(x0, y0, c);
+        return mfma_bf16_16x16x32(x1, y1, c);
+    }
+}
+
+// Per-token x per-channel int8: the epilogue of a lane's 16 consecutive outputs of row m.  Stores the raw
+// accumulators when asked for and turns them into float(acc) * a_s[m] * b_s[n] (in that order, like the
+// weight-streaming kernel) in place.
+__device__ __forceinline__ void rowcol_epilogue(const DirectArgs& p, v4f (&v)[4], int m, int64_t off, int nb, int n_valid) {
+    if (p.c_i32) {
+        const bool vec_i = ((((uintptr_t)p.c_i32) & 15) == 0) && (p.N % 4 == 0);
+        store_row16_i32(p.c_i32, off, v, n_valid, vec_i);
+    }
+    if (!p.c) return;
+    const float as = ((const float*)p.a_s)[m];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float bs = ((const float*)p.b_s)[nb + min(4 * j + q, n_valid - 1)];
+            v[j][q] = (float)__float_as_int(v[j][q]) * as * bs;
+        }
+}
+
 // MI = 16-row tiles per wave along M (4, 2 or 1): the workgroup tile is 64*MI rows x 128 columns.
 template <int KIND, bool GROUPED, int MI>
 __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
@@ -85,11 +147,11 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
-    // SCALED: 8-bit operands with per-128-K block scales.  Otherwise fp16 / bf16 operands, no scales: a K
-    // step is still one 128-byte row segment (64 elements, two 16x16x32 MFMAs per tile) and the MFMAs
-    // accumulate directly.  Kb = bytes per operand row.
+    // SCALED: 8-bit operands with per-128-K block scales.  Otherwise no scales inside the K loop (fp16 / bf16
+    // operands, or int8 with per-token and per-channel scales applied in the epilogue): a K step is still
+    // one 128-byte row segment (two MFMAs per tile) and the MFMAs accumulate directly.
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
-    constexpr int ESZ = SCALED ? 1 : 2;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
     const int KT_all = K >> 7;
@@ -229,21 +291,6 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             for (int i = 0; i < MI; ++i) sa[i] = Ss[i * 16] * bs;
         }
     };
-    auto mma16 = [&](const v8i& x, const v8i& y, v4f c) {      // two 16x16x32 half-precision MFMAs
-        if constexpr (KIND == K_F16) {
-            v8h x0, x1, y0, y1;
-            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
-            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
-            c = mfma_f16_16x16x32(x0, y0, c);
-            return mfma_f16_16x16x32(x1, y1, c);
-        } else {
-            v8bf x0, x1, y0, y1;
-            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
-            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
-            c = mfma_bf16_16x16x32(x0, y0, c);
-            return mfma_bf16_16x16x32(x1, y1, c);
-        }
-    };
     // The weight fragment is the MFMA row operand and the activation fragment the column operand, i.e.
     // the tile is produced transposed: a lane owns output row r and four consecutive columns per MFMA.
     // Branch-free so that the whole body is a single scheduling region.
@@ -252,7 +299,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = mma16(bf[j], af[i], acc[i][j]);
+                for (int j = 0; j < 4; ++j) acc[i][j] = mma_plain<KIND>(bf[j], af[i], acc[i][j]);
         } else if constexpr (MI == 1) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -359,6 +406,10 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const int m = m_start + wm * WR + 16 * i + r;
         if (m >= m_end || n_valid <= 0) continue;
         const int64_t off = (int64_t)m * N + nb;
+        if constexpr (KIND == K_I8_ROWCOL) {
+            rowcol_epilogue(p, acc[i], m, off, nb, n_valid);
+            if (!p.c) continue;
+        }
         if (cdt == LLMK_BF16) store_row16<LLMK_BF16>(cout, off, acc[i], n_valid, vec_ok);
         else if (cdt == LLMK_F16) store_row16<LLMK_F16>(cout, off, acc[i], n_valid, vec_ok);
         else store_row16<LLMK_F32>(cout, off, acc[i], n_valid, vec_ok);

@@ -32,7 +32,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     const int r = lane & 15, g = lane >> 4;
     const int wm = wave >> 2, wn = wave & 3;
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
-    constexpr int ESZ = SCALED ? 1 : 2;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
     const int KT = K >> 7;
@@ -122,22 +122,6 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const v4i x = *(const v4i*)(base + lo), y = *(const v4i*)(base + hi);
         return (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
     };
-    auto mma16 = [&](const v8i& x, const v8i& y, v4f c) {      // two 16x16x32 half-precision MFMAs
-        if constexpr (KIND == K_F16) {
-            v8h x0, x1, y0, y1;
-            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
-            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
-            c = mfma_f16_16x16x32(x0, y0, c);
-            return mfma_f16_16x16x32(x1, y1, c);
-        } else {
-            v8bf x0, x1, y0, y1;
-            __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
-            __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
-            c = mfma_bf16_16x16x32(x0, y0, c);
-            return mfma_bf16_16x16x32(x1, y1, c);
-        }
-    };
-
     // Partial products of a tile row live in one of two register sets: while the MFMAs of row i fill
     // set i & 1, the FMAs scale and accumulate row i - 1 from the other set, four MFMAs after it was
     // produced.  Row 7 of a step is retired by row 0 of the next one, with the scale of its own step.
@@ -188,7 +172,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                     if (i > 0 && i <= NR) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
                     else if (i == 0 && NR == 8) acc[7][j] += t[1][j] * sprev;
                 } else {
-                    if (i < NR) acc[i][j] = mma16(bf[j], af[i & 1], acc[i][j]);
+                    if (i < NR) acc[i][j] = mma_plain<KIND>(bf[j], af[i & 1], acc[i][j]);
                 }
                 if (i == 7 && SYNC) {
                     if (j == 0 && ISSUE) issue(kt + 2);
@@ -243,6 +227,10 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const int m = m_start + wm * 128 + 16 * i + r;
         if (m >= m_end || n_valid <= 0) continue;
         const int64_t off = (int64_t)m * N + nb;
+        if constexpr (KIND == K_I8_ROWCOL) {
+            rowcol_epilogue(p, acc[i], m, off, nb, n_valid);
+            if (!p.c) continue;
+        }
         if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
         else if (p.c_dtype == LLMK_F16) store_row16<LLMK_F16>(p.c, off, acc[i], n_valid, vec_ok);
         else store_row16<LLMK_F32>(p.c, off, acc[i], n_valid, vec_ok);

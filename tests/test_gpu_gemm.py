@@ -106,7 +106,9 @@ def test_int8_block_accumulators_bit_exact(dev, M, N, K):
     assert torch.equal(c1.cpu().long(), a1.long() @ b1.long().T)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (16, 4096, 4096), (130, 200, 1024), (128, 4096, 14336)])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (16, 4096, 4096), (130, 200, 1024), (128, 4096, 14336),
+                                   (65, 136, 128), (300, 264, 640), (1000, 521, 1152), (2048, 4096, 2048),
+                                   (4096, 4096, 1024), (3850, 4110, 640)])
 def test_int8_per_token_int32_bit_exact(dev, M, N, K):
     announce("int8 rowcol", M, N, K)
     torch.manual_seed(M + K)
@@ -116,6 +118,11 @@ def test_int8_per_token_int32_bit_exact(dev, M, N, K):
         c, acc = int8_kernel.int8_gemm_per_token(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev), return_int32=True)
     assert acc.dtype == torch.int32 and torch.equal(acc.cpu(), g.int8_gemm_int32(a, b))
     assert_close_scaled(c, g.int8_gemm_rowcol(a, a_s, b, b_s), what="int8 rowcol")
+    with default_dtype(torch.float32):     # scaled output alone (no accumulator buffer), full-range operands
+        a2 = torch.randint(-128, 128, (M, K), dtype=torch.int8)
+        b2 = torch.randint(-128, 128, (N, K), dtype=torch.int8)
+        c2 = int8_kernel.int8_gemm_per_token(a2.to(dev), a_s.to(dev), b2.to(dev), b_s.to(dev))
+    assert_close_scaled(c2, g.int8_gemm_rowcol(a2, a_s, b2, b_s), what="int8 rowcol full range")
     ag, asg = int8_kernel.act_quant_per_token(torch.randn(M, K, device=dev))
     assert ag.dtype == torch.int8 and asg.shape == (M,)
 
@@ -204,6 +211,44 @@ def test_mid_m_split_k_shapes(dev, kind, M, N, K, out):
             c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
     assert c.dtype == out
     assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="split-K " + kind)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
+@pytest.mark.parametrize("M,N,K,out", [(16, 4096, 14336, torch.bfloat16), (1, 1000, 8192, torch.float32),
+                                       (13, 264, 4224, torch.float16), (50, 520, 12416, torch.bfloat16),
+                                       (16, 28672, 4224, torch.bfloat16), (33, 136, 16384, torch.float32)])
+def test_decode_k_ranges(dev, kind, M, N, K, out):
+    """Decode-sized M with K > 4096: the weight-streaming kernel runs on K ranges side by side and a second
+    kernel adds the fp32 partial sums (ragged last range, ragged rows and columns included)."""
+    announce("K ranges", kind, M, N, K, out)
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    with default_dtype(out):
+        if kind == "fp8":
+            a, a_s = q.act_quant_fp8(x)
+            b, b_s = q.weight_quant_fp8(w)
+            c = fp8_kernel.fp8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+        else:
+            a, a_s = q.act_quant_int8(x)
+            b, b_s = q.weight_quant_int8(w)
+            c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert c.dtype == out
+    assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="K ranges " + kind)
+
+
+def test_int8_decode_k_ranges_exact(dev):
+    """Unit scales, small integers: the sum over K ranges is the exact integer product."""
+    announce("K ranges exact")
+    torch.manual_seed(9)
+    M, N, K = 16, 1032, 12416
+    a = torch.randint(-15, 16, (M, K), dtype=torch.int8)
+    b = torch.randint(-15, 16, (N, K), dtype=torch.int8)
+    a_s = torch.ones(M, K // 128, dtype=torch.float32)
+    b_s = torch.ones((N + 127) // 128, K // 128, dtype=torch.float32)
+    with default_dtype(torch.float32):
+        c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert torch.equal(c.cpu().long(), a.long() @ b.long().T)
 
 
 def test_fp8_gemm_without_scratch_takes_the_streaming_kernel(dev):
