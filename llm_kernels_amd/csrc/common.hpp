@@ -42,11 +42,29 @@ __device__ __forceinline__ float bf16_to_f32(unsigned short h) {
     return __uint_as_float(((unsigned)h) << 16);
 }
 // round-to-nearest-even fp32 -> bf16 (NaN kept quiet)
+// round-to-nearest-even conversions on the hardware converters of gfx950 (v_cvt_pk_bf16_f32, v_cvt_pk_f16_f32)
 __device__ __forceinline__ unsigned short f32_to_bf16(float f) {
-    unsigned u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (unsigned short)(u >> 16);
+    const __bf16 v = (__bf16)f;
+    unsigned short h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+}
+// two floats -> one dword of two 16-bit values (a in the low half)
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const bf2 v = __builtin_convertvector((f2){a, b}, bf2);
+    unsigned u;
+    __builtin_memcpy(&u, &v, 4);
+    return u;
+}
+__device__ __forceinline__ unsigned pack_f16x2(float a, float b) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const h2 v = __builtin_convertvector((f2){a, b}, h2);
+    unsigned u;
+    __builtin_memcpy(&u, &v, 4);
+    return u;
 }
 __device__ __forceinline__ float f16_to_f32(unsigned short h) {
     _Float16 v;

@@ -51,14 +51,12 @@ __device__ __forceinline__ void store_row16(void* c, int64_t off, const v4f (&v)
             v4i lo, hi;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                unsigned short h[8];
+                v4i w;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    h[q] = ODT == LLMK_F16 ? f32_to_f16(v[2 * j][q]) : f32_to_bf16(v[2 * j][q]);
-                    h[4 + q] = ODT == LLMK_F16 ? f32_to_f16(v[2 * j + 1][q]) : f32_to_bf16(v[2 * j + 1][q]);
+                    const float x = v[2 * j + (q >> 1)][2 * (q & 1)], y = v[2 * j + (q >> 1)][2 * (q & 1) + 1];
+                    w[q] = (int)(ODT == LLMK_F16 ? pack_f16x2(x, y) : pack_bf16x2(x, y));
                 }
-                v4i w = {(int)(h[0] | ((unsigned)h[1] << 16)), (int)(h[2] | ((unsigned)h[3] << 16)),
-                         (int)(h[4] | ((unsigned)h[5] << 16)), (int)(h[6] | ((unsigned)h[7] << 16))};
                 if (j == 0) lo = w; else hi = w;
             }
             v4i* dst = (v4i*)((unsigned short*)c + off);
@@ -117,15 +115,9 @@ __device__ __forceinline__ v4f mma_plain(const v8i& x, const v8i& y, v4f c) {
     }
 }
 
-// Per-token x per-channel int8: the epilogue of a lane's 16 consecutive outputs of row m.  Stores the raw
-// accumulators when asked for and turns them into float(acc) * a_s[m] * b_s[n] (in that order, like the
-// weight-streaming kernel) in place.
-__device__ __forceinline__ void rowcol_epilogue(const DirectArgs& p, v4f (&v)[4], int m, int64_t off, int nb, int n_valid) {
-    if (p.c_i32) {
-        const bool vec_i = ((((uintptr_t)p.c_i32) & 15) == 0) && (p.N % 4 == 0);
-        store_row16_i32(p.c_i32, off, v, n_valid, vec_i);
-    }
-    if (!p.c) return;
+// Per-token x per-channel int8, a lane's 16 consecutive outputs of row m: raw accumulators (as bits) ->
+// float(acc) * a_s[m] * b_s[n], in that order, like the weight-streaming kernel.
+__device__ __forceinline__ void rowcol_scale(const DirectArgs& p, v4f (&v)[4], int m, int nb, int n_valid) {
     const float as = ((const float*)p.a_s)[m];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -134,6 +126,15 @@ __device__ __forceinline__ void rowcol_epilogue(const DirectArgs& p, v4f (&v)[4]
             const float bs = ((const float*)p.b_s)[nb + min(4 * j + q, n_valid - 1)];
             v[j][q] = (float)__float_as_int(v[j][q]) * as * bs;
         }
+}
+
+// the same with the optional store of the raw accumulators in front
+__device__ __forceinline__ void rowcol_epilogue(const DirectArgs& p, v4f (&v)[4], int m, int64_t off, int nb, int n_valid) {
+    if (p.c_i32) {
+        const bool vec_i = ((((uintptr_t)p.c_i32) & 15) == 0) && (p.N % 4 == 0);
+        store_row16_i32(p.c_i32, off, v, n_valid, vec_i);
+    }
+    if (p.c) rowcol_scale(p, v, m, nb, n_valid);
 }
 
 // MI = 16-row tiles per wave along M (4, 2 or 1): the workgroup tile is 64*MI rows x 128 columns.
