@@ -415,7 +415,8 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
                 slots_r = max(1, cus * max(1, per_cu));
             }
             const int rows = mtiles * nz;
-            const int gx = min(ntiles, max(1, slots_r / min(rows, slots_r)));
+            int gx = min(ntiles, max(1, slots_r / min(rows, slots_r)));
+            { const int per_wg = (ntiles + gx - 1) / gx; gx = (ntiles + per_wg - 1) / per_wg; }
             gemm_direct_kernel<KIND, 1, NW, false, true, SDT, false, true>
                 <<<dim3((unsigned)gx, (unsigned)mtiles, (unsigned)nz), dim3(NW * 64), smem_r, stream>>>(p);
             LLMK_CHECK_LAUNCH(name);
@@ -442,7 +443,10 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
         slots[resident] = max(1, cus * max(1, per_cu));
     }
-    const int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
+    int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
+    // every workgroup the same number of column tiles (the slowest one sets the time): fewer workgroups
+    // rather than a last round that only some of them take part in
+    { const int per_wg = (ntiles + gx - 1) / gx; gx = (ntiles + per_wg - 1) / per_wg; }
     dim3 grid((unsigned)gx, (unsigned)mtiles), block(NW * 64);
     if constexpr (CAN_VEC) {
         if (vec) {

@@ -542,7 +542,8 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
         slots[resident] = max(1, cus * max(1, per_cu));
     }
     const int rows = mtiles * nz;
-    const int gx = min(ntiles, max(1, slots[resident] / min(rows, slots[resident])));
+    int gx = min(ntiles, max(1, slots[resident] / min(rows, slots[resident])));
+    { const int per_wg = (ntiles + gx - 1) / gx; gx = (ntiles + per_wg - 1) / per_wg; }   // equal tile counts
     dim3 grid((unsigned)gx, (unsigned)mtiles, (unsigned)nz);
     float* part = nz > 1 ? partial : nullptr;
     bool launched = false;

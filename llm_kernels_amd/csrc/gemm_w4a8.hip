@@ -340,7 +340,8 @@ int launch_w4a8_stream(W4A8Args p, void* workspace, int64_t workspace_bytes, hip
             LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot query the device");
     }
     const int rows = mtiles * nz;                                      // workgroup rows that share the column tiles
-    const int gx = min(ntiles, max(1, cus / min(rows, cus)));          // one workgroup per CU (LDS bound)
+    int gx = min(ntiles, max(1, cus / min(rows, cus)));                // one workgroup per CU (LDS bound)
+    { const int per_wg = (ntiles + gx - 1) / gx; gx = (ntiles + per_wg - 1) / per_wg; }   // equal tile counts
     dim3 grid((unsigned)gx, (unsigned)mtiles, (unsigned)nz);
     if (rounds == 1) k1<<<grid, 512, smem, st>>>(p);
     else k2<<<grid, 512, smem, st>>>(p);
