@@ -423,8 +423,18 @@ __global__ void splitk_sum_kernel(const float* __restrict__ partial, void* __res
     const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= mn) return;
     if (i + 4 <= mn && mn % 4 == 0) {
+        // four independent loads at a time (the partials come from other CUs' writes: every load is a long
+        // round trip), added in slice order
         v4f s = {0.f, 0.f, 0.f, 0.f};
-        for (int k = 0; k < z; ++k) s += *(const v4f*)(partial + (int64_t)k * mn + i);
+        int k = 0;
+        for (; k + 4 <= z; k += 4) {
+            v4f t[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) t[j] = *(const v4f*)(partial + (int64_t)(k + j) * mn + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s += t[j];
+        }
+        for (; k < z; ++k) s += *(const v4f*)(partial + (int64_t)k * mn + i);
 #pragma unroll
         for (int q = 0; q < 4; ++q) FloatIO<ODT>::st(c, i + q, s[q]);
     } else {
