@@ -99,7 +99,8 @@ int llmk_weight_dequant_w4a8(const int32_t* packed, const void* s_f16, const int
 /* ------------------------------------------------------------------ dense quantized GEMMs
  * C[M,N] = sum_kb dot_kb(A, B) * a_s[m, kb] * b_s[n / 128, kb], K % 128 == 0, any M, N >= 1.
  * A [M,K], B [N,K] both K-contiguous.  c_dtype selects the epilogue (torch default dtype).
- * workspace/workspace_bytes: optional split-K scratch (may be NULL/0 -> no split-K).
+ * workspace/workspace_bytes: optional scratch of llmk_gemm_workspace_bytes(M, N, K) bytes (fp32 activation
+ * scales for large M, fp32 partial sums of the split-K / K-range variants); NULL/0 -> single-pass variants.
  * ref: quantization/fp8_kernel.py:113-191 (a_s, b_s fp32)                                   */
 int llmk_gemm_fp8_block(const void* a_e4m3, const float* a_s, const void* b_e4m3, const float* b_s,
                         void* c, int c_dtype, int64_t M, int64_t N, int64_t K,
@@ -109,7 +110,9 @@ int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const 
                        int s_dtype, void* c, int c_dtype, int64_t M, int64_t N, int64_t K,
                        void* workspace, int64_t workspace_bytes, void* stream);
 /* per-token x per-channel W8A8 with one full-K int32 accumulation (a scheme with
- * no counterpart function in the reference).  c may be NULL; c_i32 (raw accumulators) may be NULL. */
+ * no counterpart function in the reference).  c may be NULL; c_i32 (raw accumulators) may be NULL.
+ * M <= 64 streams the weights once; larger M runs on the MFMA tile kernels (int32 accumulation inside
+ * the MFMA, c = float(acc) * a_s[m] * b_s[n] in the epilogue of either path). */
 int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, const float* b_s,
                         void* c, int c_dtype, int32_t* c_i32, int64_t M, int64_t N, int64_t K,
                         void* stream);
