@@ -4,7 +4,7 @@
 // Workgroup: 512 threads = 8 waves (4 along M x 2 along N), output tile 256 x 128, K step 128
 // (one scale block).  Wave tile 64 x 64 = 4 x 4 MFMA tiles, two waves per SIMD.
 //
-// LDS stage (50176 B): A 256 rows x 128 B, B 128 rows x 128 B, and the fp32 activation-scale column
+// LDS stage (50176 B for 256 rows): A rows x 128 B, B 128 rows x 128 B, and the fp32 activation-scale column
 // of this K step.  A direct-to-LDS load writes lane l's 16 bytes at base + 16 l, so rows cannot be
 // padded; instead the 16-byte chunk index is XOR-swizzled with ((row >> 1) & 7) on the global side:
 // LDS slot s of row R holds global chunk s ^ ((R >> 1) & 7).  Two 128-byte rows span the 64 banks, so
@@ -20,11 +20,14 @@
 
 namespace llmk {
 
-constexpr int D_BM = 256, D_BN = 128, D_THREADS = 512, D_NSTAGE = 3;
-constexpr int D_A = D_BM * 128, D_B = D_BN * 128, D_S = D_BM * 4;
-constexpr int D_STAGE = D_A + D_B + D_S;                 // 50176
+constexpr int D_BN = 128, D_THREADS = 512, D_NSTAGE = 3;
+constexpr int D_B = D_BN * 128, D_S = 256 * 4;
 constexpr int D_MAX_KT = 256;                            // weight-scale table entries (K <= 32768)
-constexpr int D_LDS = D_NSTAGE * D_STAGE + D_MAX_KT * 4; // 151552 bytes of the 160 KB
+// stage bytes and LDS per tile height (MI 16-row tiles per wave, 64 * MI rows): 50176 / 33792 / 25600 per
+// stage, 151552 / 102400 / 77824 bytes in all, so that two workgroups of the 64-row tile share a CU
+constexpr int d_a(int mi) { return 64 * mi * 128; }
+constexpr int d_stage(int mi) { return d_a(mi) + D_B + D_S; }
+constexpr int d_lds(int mi) { return D_NSTAGE * d_stage(mi) + D_MAX_KT * 4; }
 
 __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
@@ -100,7 +103,7 @@ __device__ __forceinline__ v4f mma_plain(const v8i& x, const v8i& y, v4f c) {
         ci = mfma_i8_16x16x64(x1, y1, ci);
         __builtin_memcpy(&c, &ci, 16);
         return c;
-    } else if constexpr (KIND == K_F16) {
+    } else if constexpr (KIND == K_F16 || KIND == K_W4NK) {
         v8h x0, x1, y0, y1;
         __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
         __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
@@ -137,11 +140,48 @@ __device__ __forceinline__ void rowcol_epilogue(const DirectArgs& p, v4f (&v)[4]
     if (p.c) rowcol_scale(p, v, m, nb, n_valid);
 }
 
+// ---- 4-bit weights inside the tile kernel (K_W4NK) ----
+// nibble -> fp16 without integer->float converts: (q | 0x6400) is the fp16 number 1024 + q,
+// ((q << 4) | 0x6400) is 1024 + 16 q; one packed subtract / fma gives q - 8 exactly.
+__device__ __forceinline__ v2h w4_as_h2(unsigned u) { v2h r; __builtin_memcpy(&r, &u, 4); return r; }
+__device__ __forceinline__ unsigned w4_as_u32(v2h h) { unsigned r; __builtin_memcpy(&r, &h, 4); return r; }
+// one packed word (nibble j = element 8*word + j of the row) -> eight fp16 (q - 8) * scale in K order
+__device__ __forceinline__ v4i w4_word_to_f16x8(unsigned w, v2h sc) {
+    const v2h k1032 = {(_Float16)1032.f, (_Float16)1032.f};
+    const v2h k16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const v2h k72 = {(_Float16)72.f, (_Float16)72.f};
+    const unsigned w8 = w >> 8;
+    const unsigned p04 = w4_as_u32((w4_as_h2((w & 0x000f000fu) | 0x64006400u) - k1032) * sc);
+    const unsigned p15 = w4_as_u32((w4_as_h2((w & 0x00f000f0u) | 0x64006400u) * k16 - k72) * sc);
+    const unsigned p26 = w4_as_u32((w4_as_h2((w8 & 0x000f000fu) | 0x64006400u) - k1032) * sc);
+    const unsigned p37 = w4_as_u32((w4_as_h2((w8 & 0x00f000f0u) | 0x64006400u) * k16 - k72) * sc);
+    v4i o;
+    o[0] = (int)__builtin_amdgcn_perm(p15, p04, 0x05040100u);
+    o[1] = (int)__builtin_amdgcn_perm(p37, p26, 0x05040100u);
+    o[2] = (int)__builtin_amdgcn_perm(p15, p04, 0x07060302u);
+    o[3] = (int)__builtin_amdgcn_perm(p37, p26, 0x07060302u);
+    return o;
+}
+// Register loads issued from inline asm like the direct-to-LDS loads, so that they take part in the same
+// hand-counted vmcnt scheme (a compiler-tracked load would make the compiler wait for every load in flight).
+// The destination is only read behind an explicit s_waitcnt.
+__device__ __forceinline__ uint64_t asm_load_b64(uint32_t voff, const void* sbase) {
+    uint64_t v;
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+__device__ __forceinline__ unsigned asm_load_u16(uint32_t voff, const void* sbase) {
+    unsigned v;
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+
 // MI = 16-row tiles per wave along M (4, 2 or 1): the workgroup tile is 64*MI rows x 128 columns.
 template <int KIND, bool GROUPED, int MI>
 __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     constexpr int BM = 64 * MI;              // tile rows
     constexpr int WR = 16 * MI;              // rows per wave
+    constexpr int D_A = d_a(MI), D_STAGE = d_stage(MI);
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -151,8 +191,12 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // SCALED: 8-bit operands with per-128-K block scales.  Otherwise no scales inside the K loop (fp16 / bf16
     // operands, or int8 with per-token and per-channel scales applied in the epilogue): a K step is still
     // one 128-byte row segment (two MFMAs per tile) and the MFMAs accumulate directly.
+    // K_W4NK: fp16 activations by direct-to-LDS loads as for K_F16; the weight rows of a stage are expanded
+    // from the packed words by the threads themselves (one 8-byte load, 16 weights, two 16-byte LDS writes per
+    // thread and K step), one K step behind the loads and one ahead of the multiplication.
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    constexpr bool W4 = (KIND == K_W4NK);
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
     const int KT_all = K >> 7;
@@ -212,6 +256,16 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
     const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
+    // K_W4NK: thread t expands quarter (t & 3) of LDS row t >> 2 (16 weights of a 64-element K step)
+    uint32_t w4_off = 0, w4_soff = 0, w4_lds = 0;
+    if constexpr (W4) {
+        const int R = tid >> 2, q = tid & 3, rho = R & 63;
+        const int col = (R & 64) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
+        const uint32_t n = (uint32_t)min(n0 + col, N - 1);
+        w4_off = n * (uint32_t)(p.K >> 1) + (uint32_t)q * 8u;                  // bytes into the packed matrix
+        w4_soff = n * (uint32_t)(p.K / p.group) * 2u;                          // bytes into the scale matrix
+        w4_lds = (uint32_t)R * 128u + (uint32_t)((2 * q) ^ ((R >> 1) & 7)) * 16u;   // chunk 2q; chunk 2q+1 is at ^16
+    }
 
     auto issue = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
@@ -220,11 +274,35 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
 #pragma unroll
         for (int i = 0; i < MI; ++i) dma16(st + (uint32_t)(wave * MI + i) * 1024u, aoff[i], ga);
+        if constexpr (!W4) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) dma16(st + D_A + (uint32_t)(wave * 2 + i) * 1024u, boff[i], gb);
+            for (int i = 0; i < 2; ++i) dma16(st + D_A + (uint32_t)(wave * 2 + i) * 1024u, boff[i], gb);
+        }
         if constexpr (SCALED) dma4(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, soff, gs);
     };
-    // loads per stage per thread: MI (A) + 2 (B) + 1 (scale column); imm = vmcnt | no expcnt/lgkmcnt wait
+    // K_W4NK: packed words and group scale of K step kt -> registers (requested before the activation loads
+    // of the same step, so that waiting for them leaves exactly those MI loads in flight) ...
+    uint64_t w4_words = 0;
+    unsigned w4_scale = 0;
+    auto w4_request = [&](int kt) {
+        if constexpr (W4) {
+            w4_words = asm_load_b64(w4_off, (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 32);
+            w4_scale = asm_load_u16(w4_soff, (const uint8_t*)p.b_s + (int64_t)(((kt0 + kt) * 64) / p.group) * 2);
+        }
+    };
+    // ... and from there, expanded, into the weight rows of stage kt
+    auto w4_expand = [&](int kt) {
+        if constexpr (W4) {
+            __builtin_amdgcn_s_waitcnt(0x0F70 | MI);       // everything but the MI youngest (activation) loads
+            __builtin_amdgcn_sched_barrier(0);
+            const v2h sc = w4_as_h2(w4_scale | (w4_scale << 16));
+            uint8_t* dst = lds + (kt % D_NSTAGE) * D_STAGE + D_A + w4_lds;
+            *(v4i*)dst = w4_word_to_f16x8((unsigned)w4_words, sc);
+            *(v4i*)(dst + ((w4_lds & 16u) ? -16 : 16)) = w4_word_to_f16x8((unsigned)(w4_words >> 32), sc);
+        }
+    };
+    // loads per stage per thread: MI (A) + 2 (B, or words + scale for K_W4NK) + 1 (scale column);
+    // imm = vmcnt | no expcnt/lgkmcnt wait
     constexpr int WAIT_ONE_STAGE = 0x0F70 | (MI + 2 + (SCALED ? 1 : 0));
 
     // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 64 x 64 tile
@@ -234,8 +312,8 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-    if (KT > 0) issue(0);
-    if (KT > 1) issue(1);
+    if (KT > 0) { w4_request(0); issue(0); w4_expand(0); }
+    if (KT > 1) { w4_request(1); issue(1); }
     // weight scales of this tile for every K step -> LDS.  These are the only compiler-tracked vector
     // loads; they sit behind the first two stages in the memory queue, so waiting for them also waits
     // for stage 0 and 1 (an acceptable one-off: the pipeline is being filled anyway).
@@ -342,6 +420,8 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     int kt = 0;
     if (wave < 4) {
         for (; kt + 2 < KT; ++kt) {
+            w4_expand(kt + 1);
+            w4_request(kt + 2);
             issue(kt + 2);
             load_frags(kt);
             compute();
@@ -349,6 +429,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             __syncthreads();
         }
         if (kt + 1 < KT) {
+            w4_expand(kt + 1);
             load_frags(kt);
             compute();
             __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
@@ -361,6 +442,8 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         }
     } else {
         for (; kt + 2 < KT; ++kt) {
+            w4_expand(kt + 1);
+            w4_request(kt + 2);
             issue(kt + 2);
             compute();
             __builtin_amdgcn_sched_barrier(0);
@@ -369,6 +452,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             __syncthreads();
         }
         if (kt + 1 < KT) {
+            w4_expand(kt + 1);
             compute();
             __builtin_amdgcn_sched_barrier(0);
             load_frags(kt);
@@ -466,8 +550,8 @@ int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     static bool configured = false;
     auto kern = gemm_dma_kernel<KIND, GROUPED, MI>;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, D_LDS);
-        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, D_LDS, hipGetErrorString(e));
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, d_lds(MI));
+        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, d_lds(MI), hipGetErrorString(e));
         configured = true;
     }
     constexpr int BM = 64 * MI;
@@ -475,7 +559,7 @@ int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     const bool split = !GROUPED && p.ksplit > 1 && p.partial;
     dim3 grid((unsigned)((p.N + D_BN - 1) / D_BN), (unsigned)tiles_m, split ? (unsigned)p.ksplit : 1u);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
-    kern<<<grid, D_THREADS, D_LDS, stream>>>(p);
+    kern<<<grid, D_THREADS, d_lds(MI), stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     if (split) {
         const int64_t mn = (int64_t)p.M * p.N;

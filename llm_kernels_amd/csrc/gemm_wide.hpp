@@ -279,12 +279,15 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
 template <int KIND, bool GROUPED>
 int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
+    constexpr bool HAS_WIDE = KIND != K_W4NK;             // the 4-bit expansion exists in the 128-column kernels only
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
     auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm) + 255) / 256; };
     const double t_wide = 64.0 * rounds(256, 256), t4 = 43.0 * rounds(256, 128), t2 = 26.0 * rounds(128, 128),
                  t1 = 16.0 * rounds(64, 128);
-    if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) return launch_wide<KIND, GROUPED>(p, stream, name);
+    if constexpr (HAS_WIDE) {
+        if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) return launch_wide<KIND, GROUPED>(p, stream, name);
+    }
     if (t4 <= t2 && t4 <= t1) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
     if (t2 <= t1) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
     return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);

@@ -159,6 +159,24 @@ def test_mul_large_tile_shapes(dev, M, N, K, gs):
     assert_close_scaled(C, g.w4a16_gemm(A, q4, s, gs), what="marlin large tiles")
 
 
+@pytest.mark.parametrize("M,N,K,gs", [(65, 136, 128, 64), (128, 4096, 4096, 128), (200, 1000, 1152, 128), (256, 520, 8192, 256),
+                                      (512, 264, 2048, 64), (100, 129, 14336, -1), (130, 4100, 4224, 128), (96, 28672, 1024, 128)])
+def test_w4a16_nk_mid_m_fused_tiles(dev, M, N, K, gs):
+    """64 < M <= 512: the tile kernels expand the packed words themselves (one or several K slices, ragged rows
+    and columns, group sizes from 64 to the whole row)."""
+    announce("w4a16 nk fused tiles", M, N, K, gs)
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).half()
+    w = torch.randn(N, K) * 0.02
+    grp = K if gs == -1 else gs
+    qn, s = q.w4a16_quant_nk(w, grp)
+    packed, _ = bp.pack_cols(qn.numpy(), 4, 32)
+    y = w4a16.w4a16_gemm(x.to(dev), torch.from_numpy(packed).to(dev), s.to(dev), gs)
+    assert y.dtype == torch.half and y.shape == (M, N)
+    ref = g.w4a16_gemm(x, qn.t().int().contiguous(), s.t().contiguous(), grp)
+    assert_close_scaled(y, ref, what="w4a16 nk fused tiles")
+
+
 @pytest.mark.parametrize("M,N,K,gs", [(4096, 4096, 256, 128), (3990, 4100, 384, 64), (4096, 3848, 128, 32)])
 def test_w4a16_nk_large_tile_shapes(dev, M, N, K, gs):
     announce("w4a16 nk large tiles", M, N, K, gs)
