@@ -14,7 +14,8 @@
 namespace llmk {
 
 enum : int { K_FP8_BLOCK = 0, K_I8_BLOCK = 1, K_I8_ROWCOL = 2, K_F16 = 3, K_BF16 = 4,
-             K_W4NK = 5 };   // fp16 activations x 4-bit weights packed [N, K/8] (tile kernels only)
+             K_W4NK = 5,      // fp16 activations x 4-bit weights packed [N, K/8] (tile kernels only)
+             K_W4MARLIN = 6 };// the same with weights and scales in the Marlin layout
 
 __device__ __forceinline__ float ld_scale(const void* p, int64_t i, int dt) {
     if (dt == LLMK_F32) return ((const float*)p)[i];
@@ -96,7 +97,7 @@ struct DirectArgs {
     float* partial;        // split-K: fp32 [ksplit][M][N] partial sums
     int ksplit;            // 0 / 1 = no split
     int kc_steps;          // weight-streaming kernel with K ranges: 128-byte steps per range (gridDim.z ranges)
-    int group;             // K_W4NK: K elements per fp16 group scale (b_s is [N, K / group])
+    int group;             // K_W4NK / K_W4MARLIN: K elements per fp16 group scale
 };
 
 // Upper bound of the row tiles of a grouped GEMM (segment ends are only known on the device): every segment

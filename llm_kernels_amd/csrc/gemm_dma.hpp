@@ -103,7 +103,7 @@ __device__ __forceinline__ v4f mma_plain(const v8i& x, const v8i& y, v4f c) {
         ci = mfma_i8_16x16x64(x1, y1, ci);
         __builtin_memcpy(&c, &ci, 16);
         return c;
-    } else if constexpr (KIND == K_F16 || KIND == K_W4NK) {
+    } else if constexpr (KIND == K_F16 || KIND == K_W4NK || KIND == K_W4MARLIN) {
         v8h x0, x1, y0, y1;
         __builtin_memcpy(&x0, &x, 16); __builtin_memcpy(&x1, ((const char*)&x) + 16, 16);
         __builtin_memcpy(&y0, &y, 16); __builtin_memcpy(&y1, ((const char*)&y) + 16, 16);
@@ -195,7 +195,9 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // from the packed words by the threads themselves (one 8-byte load, 16 weights, two 16-byte LDS writes per
     // thread and K step), one K step behind the loads and one ahead of the multiplication.
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
-    constexpr bool W4 = (KIND == K_W4NK);
+    // K_W4MARLIN: the same for the Marlin layout (16-byte units of 32 values: 4 k x 8 columns): a thread takes
+    // half a unit and scatters its eight fp16 pairs over the weight rows.
+    constexpr bool W4NK = (KIND == K_W4NK), W4M = (KIND == K_W4MARLIN), W4 = W4NK || W4M;
     constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
@@ -258,7 +260,20 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
     // K_W4NK: thread t expands quarter (t & 3) of LDS row t >> 2 (16 weights of a 64-element K step)
     uint32_t w4_off = 0, w4_soff = 0, w4_lds = 0;
-    if constexpr (W4) {
+    if constexpr (W4M) {
+        // A K step of 64 is four strips of 16 k; the tile's 128 columns are two 64-column chunks: 256 units.
+        // Thread t: unit (strip sl, chunk ch, lane ml = 8 columns c x 4 k-pairs q), words 2h and 2h + 1.
+        // Word j, byte pair b of a unit: column 16 j + 8 b + c of the chunk, k = 2 q, 2 q + 1 (low nibbles of
+        // the two halfwords) and 2 q + 8, 2 q + 9 (high nibbles) of the strip.
+        const int h = tid & 1, ml = (tid >> 1) & 31, ch = (tid >> 6) & 1, sl = tid >> 7, c = ml >> 2, q = ml & 3;
+        const int nchunks = N >> 6;
+        const int chunk = min((n0 >> 6) + ch, nchunks - 1);
+        w4_off = (uint32_t)((sl * nchunks + chunk) * 32 + ml) * 16u + (uint32_t)h * 8u;      // + 4 strips per K step
+        w4_soff = (uint32_t)(64 * chunk + 8 * c + 4 * h) * 2u;                              // + scale row per K step
+        // first of the eight pairs (j = 2h, b = 0, low nibbles): LDS row of column 16 j + c, K chunk 2 sl
+        w4_lds = (uint32_t)(ch * 8 + h * 2) | ((uint32_t)c << 8) | ((uint32_t)sl << 16) | ((uint32_t)q << 24);   // packed fields
+    }
+    if constexpr (W4NK) {
         const int R = tid >> 2, q = tid & 3, rho = R & 63;
         const int col = (R & 64) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
         const uint32_t n = (uint32_t)min(n0 + col, N - 1);
@@ -282,12 +297,15 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     };
     // K_W4NK: packed words and group scale of K step kt -> registers (requested before the activation loads
     // of the same step, so that waiting for them leaves exactly those MI loads in flight) ...
-    uint64_t w4_words = 0;
-    unsigned w4_scale = 0;
+    uint64_t w4_words = 0, w4_scale = 0;
     auto w4_request = [&](int kt) {
-        if constexpr (W4) {
+        if constexpr (W4NK) {
             w4_words = asm_load_b64(w4_off, (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 32);
             w4_scale = asm_load_u16(w4_soff, (const uint8_t*)p.b_s + (int64_t)(((kt0 + kt) * 64) / p.group) * 2);
+        }
+        if constexpr (W4M) {
+            w4_words = asm_load_b64(w4_off, (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 4 * (N >> 6) * 512);
+            w4_scale = asm_load_b64(w4_soff, (const uint8_t*)p.b_s + (int64_t)(((kt0 + kt) * 64) / p.group) * N * 2);
         }
     };
     // ... and from there, expanded, into the weight rows of stage kt
@@ -295,10 +313,35 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         if constexpr (W4) {
             __builtin_amdgcn_s_waitcnt(0x0F70 | MI);       // everything but the MI youngest (activation) loads
             __builtin_amdgcn_sched_barrier(0);
-            const v2h sc = w4_as_h2(w4_scale | (w4_scale << 16));
+        }
+        if constexpr (W4NK) {
+            const unsigned s16 = (unsigned)w4_scale;
+            const v2h sc = w4_as_h2(s16 | (s16 << 16));
             uint8_t* dst = lds + (kt % D_NSTAGE) * D_STAGE + D_A + w4_lds;
             *(v4i*)dst = w4_word_to_f16x8((unsigned)w4_words, sc);
             *(v4i*)(dst + ((w4_lds & 16u) ? -16 : 16)) = w4_word_to_f16x8((unsigned)(w4_words >> 32), sc);
+        }
+        if constexpr (W4M) {
+            const v2h k1032 = {(_Float16)1032.f, (_Float16)1032.f};
+            const v2h k16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+            const v2h k72 = {(_Float16)72.f, (_Float16)72.f};
+            const int j0 = (int)(w4_lds & 7u), ch8 = (int)(w4_lds & 8u), c = (int)((w4_lds >> 8) & 7u);
+            const int sl = (int)((w4_lds >> 16) & 3u), q = (int)(w4_lds >> 24);
+            uint8_t* bst = lds + (kt % D_NSTAGE) * D_STAGE + D_A;
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    const unsigned u = ((unsigned)(w4_words >> (32 * jj))) >> (8 * b);
+                    const unsigned s16 = (unsigned)(w4_scale >> (16 * (2 * jj + b))) & 0xffffu;
+                    const v2h sc = w4_as_h2(s16 | (s16 << 16));
+                    const int col = 16 * (j0 + jj) + 8 * b + c;                                 // column in the chunk
+                    const int R = (ch8 ? 64 : 0) + ((col >> 2) & 3) * 16 + (col >> 4) * 4 + (col & 3);   // its LDS row
+                    uint8_t* row = bst + R * 128 + 4 * q;
+                    const int sw = (R >> 1) & 7;
+                    *(v2h*)(row + ((2 * sl) ^ sw) * 16) = (w4_as_h2((u & 0x000f000fu) | 0x64006400u) - k1032) * sc;
+                    *(v2h*)(row + ((2 * sl + 1) ^ sw) * 16) = (w4_as_h2((u & 0x00f000f0u) | 0x64006400u) * k16 - k72) * sc;
+                }
         }
     };
     // loads per stage per thread: MI (A) + 2 (B, or words + scale for K_W4NK) + 1 (scale column);

@@ -618,6 +618,14 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
     if (M > 0x7fffffff / 2 || N > 0x7fffffff / 2 || K > 0x7fffffff / 2) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: dimension too large");
 
     hipStream_t st = (hipStream_t)stream;
+    if (M > 64 && M <= 512 && K % 64 == 0 && groupsize % 64 == 0) {
+        // mid-size M: the 128-column tile kernels expand the Marlin units themselves (see gemm_w4a16_nk)
+        llmk::DirectArgs p{};
+        p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.b_s = s; p.c = c; p.c_dtype = LLMK_F16;
+        p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1; p.group = groupsize;
+        if (llmk::dma_eligible(p, 2))
+            return llmk::launch_big_half<llmk::K_W4MARLIN, false>(p, st, "gemm_w4a16_marlin(fused tiles)", workspace, workspace_bytes);
+    }
     if (M > 64 && K % 64 == 0 && workspace && workspace_bytes >= N * K * 2 && !((uintptr_t)workspace & 15)) {
         // compute-bound: expand W once to fp16 [N, K], then run the tiled MFMA GEMM on it
         llmk::DirectArgs p{};

@@ -279,7 +279,7 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
 template <int KIND, bool GROUPED>
 int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
-    constexpr bool HAS_WIDE = KIND != K_W4NK;             // the 4-bit expansion exists in the 128-column kernels only
+    constexpr bool HAS_WIDE = KIND != K_W4NK && KIND != K_W4MARLIN;             // the 4-bit expansion exists in the 128-column kernels only
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
     auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm) + 255) / 256; };

@@ -159,6 +159,22 @@ def test_mul_large_tile_shapes(dev, M, N, K, gs):
     assert_close_scaled(C, g.w4a16_gemm(A, q4, s, gs), what="marlin large tiles")
 
 
+@pytest.mark.parametrize("M,N,K,gs", [(80, 192, 192, 64), (128, 4096, 4096, 128), (272, 1088, 8192, -1), (512, 320, 1024, 128),
+                                      (96, 28672, 512, 128), (144, 64, 14336, 128), (256, 4160, 2048, 256)])
+def test_mul_mid_m_fused_tiles(dev, M, N, K, gs):
+    """64 < M <= 512: the tile kernels expand the Marlin units themselves (odd chunk counts, one or several K
+    slices, group sizes from 64 to the whole column)."""
+    announce("marlin fused tiles", M, N, K, gs)
+    torch.manual_seed(M + N + K)
+    A = (torch.randn(M, K) * 0.3).half()
+    W = (torch.randn(K, N) * 0.05).half()
+    _, q4, s = mr.fake_quantize(W, gs)
+    B, sp = mr.pack(q4, s, K if gs == -1 else gs)
+    C = torch.zeros(M, N, dtype=torch.half, device=dev)
+    mul(A.to(dev), B.to(dev), C, sp.to(dev), torch.zeros(64, dtype=torch.int32, device=dev))
+    assert_close_scaled(C, g.w4a16_gemm(A, q4, s, gs), what="marlin fused tiles")
+
+
 @pytest.mark.parametrize("M,N,K,gs", [(65, 136, 128, 64), (128, 4096, 4096, 128), (200, 1000, 1152, 128), (256, 520, 8192, 256),
                                       (512, 264, 2048, 64), (100, 129, 14336, -1), (130, 4100, 4224, 128), (96, 28672, 1024, 128)])
 def test_w4a16_nk_mid_m_fused_tiles(dev, M, N, K, gs):
