@@ -135,16 +135,19 @@ int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, co
  * additionally N % 64 == 0 and groupsize % 16 == 0.
  * ref: fast_dequant/simple_marlin/marlin_w4a16_gemm.cu:283-326 (simple_marlin_cuda),
  *      marlin_w4a16_gemm.cpp:23-111 (mul).                                                    */
-/* bytes of fp32 split-K scratch llmk_gemm_w4a16_marlin uses for this shape (0 = none). Without it
- * (workspace NULL / too small) the kernel runs with fewer K slices. */
+/* bytes of scratch llmk_gemm_w4a16_marlin uses for this shape (0 = none): fp32 split-K partial sums, and for
+ * M > 64 room for the fp16 copy of W that the two-pass path of large M multiplies.  Without it (workspace
+ * NULL / too small) the kernels run with fewer K slices, large M on the weight-streaming kernel. */
 int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int llmk_gemm_w4a16_marlin(const void* a_f16, const int32_t* b, void* c_f16, const void* s_f16,
                            int64_t M, int64_t N, int64_t K, int groupsize,
                            void* workspace, int64_t workspace_bytes, void* stream);
 /* Same product for W stored [N, K/8] int32 by pack_weights_over_cols (nibble i of a word = k*8+i)
  * with s fp16 [N, K/g]; a/c fp16 or bf16 (dtype code).  fp16 only at present.  workspace is optional:
- * with N*K*2 bytes (16-byte aligned) M > 64 runs as dequantise + tiled MFMA GEMM; with
- * ceil(K/4096)*M*N*4 bytes M <= 64, K > 4096 runs as K ranges with fp32 partial sums. */
+ * M > 512 with N*K*2 bytes (16-byte aligned) runs as dequantise + tiled MFMA GEMM; 64 < M <= 512 (and
+ * 32 < M <= 64 with large weights) runs on tile kernels that expand the packed words themselves and use
+ * up to 8*M*N*4 bytes for split-K partial sums; M <= 64, K > 4096 with ceil(K/4096)*M*N*4 bytes runs as
+ * K ranges with fp32 partial sums. */
 int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s_f16,
                        int ac_dtype, int64_t M, int64_t N, int64_t K, int groupsize,
                        void* workspace, int64_t workspace_bytes, void* stream);

@@ -567,6 +567,19 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
     return LLMK_OK;
 }
 
+// Rows for which the 128-column tile kernels expand the 4-bit weights themselves: 65 to 512 always (measured
+// 1.3-2.8x faster than the separate expansion pass up to 256 rows, even to 1.4x at 512); 33 to 64 when the
+// weight matrix is large, where the tile kernel with split-K beats the weight-streaming kernels (which read
+// the activations once per 16 columns), provided the scratch for its partial sums is there.
+bool w4_tiles_expand(int64_t M, int64_t N, int64_t K, const void* workspace, int64_t workspace_bytes) {
+    if (M > 64) return M <= 512;
+    if (M <= 32 || K % 64) return false;
+    const int64_t nk = N * K;
+    if (!(K > 4096 ? nk >= ((int64_t)32 << 20) : nk >= ((int64_t)96 << 20))) return false;
+    const int z = llmk::splitk_factor_half(M, N, K);
+    return z <= 1 || (workspace && workspace_bytes >= (int64_t)z * M * N * 4 && !((uintptr_t)workspace & 15));
+}
+
 // launch shape of the Marlin-layout kernel for a given problem
 struct MarlinPlan {
     int mt, nw, mblocks, col_groups, z, steps_per_z;
@@ -598,7 +611,9 @@ extern "C" int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, 
         return ((N * K * 2 + 255) & ~(int64_t)255) + (z > 1 ? (int64_t)z * M * N * 4 : 0);
     }
     const MarlinPlan pl = marlin_plan(M, N, K);
-    return pl.z > 1 ? (int64_t)pl.z * M * N * 4 : 0;
+    const int64_t zt = M > 16 && K % 64 == 0 ? llmk::splitk_factor_half(M, N, K) : 1;   // tile kernels with split-K
+    const int64_t z = pl.z > zt ? pl.z : zt;
+    return z > 1 ? z * M * N * 4 : 0;
 }
 
 extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, const void* s, int64_t M, int64_t N,
@@ -618,7 +633,7 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
     if (M > 0x7fffffff / 2 || N > 0x7fffffff / 2 || K > 0x7fffffff / 2) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_marlin: dimension too large");
 
     hipStream_t st = (hipStream_t)stream;
-    if (M > 64 && M <= 512 && K % 64 == 0 && groupsize % 64 == 0) {
+    if (w4_tiles_expand(M, N, K, workspace, workspace_bytes) && K % 64 == 0 && groupsize % 64 == 0) {
         // mid-size M: the 128-column tile kernels expand the Marlin units themselves (see gemm_w4a16_nk)
         llmk::DirectArgs p{};
         p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.b_s = s; p.c = c; p.c_dtype = LLMK_F16;
@@ -700,7 +715,7 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
     const _Float16* A = (const _Float16*)a;
     const _Float16* S = (const _Float16*)s;
     _Float16* C = (_Float16*)c;
-    if (M > 64 && M <= 512 && K % 64 == 0 && groupsize % 64 == 0) {
+    if (w4_tiles_expand(M, N, K, workspace, workspace_bytes) && K % 64 == 0 && groupsize % 64 == 0) {
         // mid-size M: the 128-column tile kernels expand the packed words themselves (every weight byte is
         // read once; the separate expansion pass would write and re-read four times as much).  Measured
         // against the two-pass path: 1.3-2.8x faster up to M = 256, even to 1.4x at 512, slower from 2048

@@ -35,8 +35,8 @@ def w4a16_gemm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, gr
     if M > 64:
         # fp16 copy of W for the compute-bound path, split-K partials behind it for mid-size M
         ws = _lib.workspace(x.device, ((N * K * 2 + 255) // 256) * 256 + (8 * M * N * 4 if M <= 512 else 0))
-    elif K > 4096:
-        ws = _lib.workspace(x.device, -(-K // 4096) * M * N * 4)   # fp32 partial sums of the K ranges
+    elif K > 4096 or M > 16:
+        ws = _lib.workspace(x.device, max(8, -(-K // 4096)) * M * N * 4)   # fp32 partial sums of K ranges / K slices
     else:
         ws = None
     _lib.call("llmk_gemm_w4a16_nk", _lib.ptr(x), _lib.ptr(w_packed), _lib.ptr(y), _lib.ptr(scales),

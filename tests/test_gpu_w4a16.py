@@ -160,10 +160,11 @@ def test_mul_large_tile_shapes(dev, M, N, K, gs):
 
 
 @pytest.mark.parametrize("M,N,K,gs", [(80, 192, 192, 64), (128, 4096, 4096, 128), (272, 1088, 8192, -1), (512, 320, 1024, 128),
-                                      (96, 28672, 512, 128), (144, 64, 14336, 128), (256, 4160, 2048, 256)])
+                                      (96, 28672, 512, 128), (144, 64, 14336, 128), (256, 4160, 2048, 256),
+                                      (48, 4096, 14336, 128), (64, 28672, 4096, 128)])
 def test_mul_mid_m_fused_tiles(dev, M, N, K, gs):
-    """64 < M <= 512: the tile kernels expand the Marlin units themselves (odd chunk counts, one or several K
-    slices, group sizes from 64 to the whole column)."""
+    """64 < M <= 512, and 32 < M <= 64 with large weights: the tile kernels expand the Marlin units themselves
+    (odd chunk counts, one or several K slices, group sizes from 64 to the whole column)."""
     announce("marlin fused tiles", M, N, K, gs)
     torch.manual_seed(M + N + K)
     A = (torch.randn(M, K) * 0.3).half()
@@ -176,10 +177,11 @@ def test_mul_mid_m_fused_tiles(dev, M, N, K, gs):
 
 
 @pytest.mark.parametrize("M,N,K,gs", [(65, 136, 128, 64), (128, 4096, 4096, 128), (200, 1000, 1152, 128), (256, 520, 8192, 256),
-                                      (512, 264, 2048, 64), (100, 129, 14336, -1), (130, 4100, 4224, 128), (96, 28672, 1024, 128)])
+                                      (512, 264, 2048, 64), (100, 129, 14336, -1), (130, 4100, 4224, 128), (96, 28672, 1024, 128),
+                                      (48, 4096, 14336, 128), (64, 28672, 4096, 128), (33, 2400, 14336, 256)])
 def test_w4a16_nk_mid_m_fused_tiles(dev, M, N, K, gs):
-    """64 < M <= 512: the tile kernels expand the packed words themselves (one or several K slices, ragged rows
-    and columns, group sizes from 64 to the whole row)."""
+    """64 < M <= 512, and 32 < M <= 64 with large weights: the tile kernels expand the packed words themselves
+    (one or several K slices, ragged rows and columns, group sizes from 64 to the whole row)."""
     announce("w4a16 nk fused tiles", M, N, K, gs)
     torch.manual_seed(M + N + K)
     x = torch.randn(M, K).half()
