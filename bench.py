@@ -262,7 +262,7 @@ MOE_WORKLOADS = {"moe_mixtral_fp8_t4096": "fp8", "moe_mixtral_int8_t4096": "int8
 DEFAULT_WORKLOAD = "fp8_m4096_n4096_k4096"
 HEADLINE_SET = ["w4a16_m16_n4096_k4096", "w4a16_nk_m16_n4096_k4096", "w4a16_nk_m16_n28672_k4096", "fp8_m16_n4096_k4096", "fp8_m16_n28672_k4096", "fp8_m16_n4096_k14336",
                 "fp8_m16_n128256_k4096", "w4a16_nk_m16_n128256_k4096",
-                "w4a16_m4096_n4096_k4096", "w4a16_nk_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "w4a8_m16_n4096_k4096", "moe_mixtral_fp8_t4096"]
+                "w4a16_m4096_n4096_k4096", "w4a16_nk_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "int8_pt_m4096_n14336_k4096", "w4a8_m16_n4096_k4096", "moe_mixtral_fp8_t4096"]
 
 
 def run_case(case, dev, steps, warmup, eager=False):
