@@ -312,6 +312,28 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) { acc[mt] = (v4f){0.f, 0.f, 0.f, 0.f}; acci[mt] = (v4i){0, 0, 0, 0}; }
     };
+    // Per-token x per-channel kind: the scales of the outputs this thread finishes.  The row scale does not
+    // depend on the tile and is read once; the column scale of a tile is requested before the tile is
+    // multiplied, so that the store at its end does not wait for memory.
+    constexpr int NOUT = (MT * 256 + NW * 64 - 1) / (NW * 64);      // outputs per thread and tile
+    float rc_as[NOUT], rc_bs[NOUT];
+    if constexpr (KIND == K_I8_ROWCOL) {
+#pragma unroll
+        for (int q = 0; q < NOUT; ++q) {
+            const int o = (int)threadIdx.x + q * NW * 64;
+            const int m = m_start + 16 * (o >> 8) + ((o & 255) >> 4);
+            rc_as[q] = (p.c && o < MT * 256) ? ((const float*)p.a_s)[min(m, m_end - 1)] : 0.f;
+            rc_bs[q] = 0.f;
+        }
+    }
+    auto request_col_scales = [&](int tl) {
+        if constexpr (KIND == K_I8_ROWCOL) {
+            if (p.c) {
+#pragma unroll
+                for (int q = 0; q < NOUT; ++q) rc_bs[q] = ((const float*)p.b_s)[min(tl * 16 + ((int)threadIdx.x & 15), N - 1)];
+            }
+        }
+    };
     auto finish = [&](int tl) __attribute__((always_inline)) {
         float* rbuf = red + (RB == 2 ? parity : 0) * NW * MT * 256;
         parity ^= 1;
@@ -324,7 +346,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         }
         __syncthreads();
         const int n0 = tl * 16;
-        for (int o = threadIdx.x; o < MT * 256; o += NW * 64) {
+#pragma unroll
+        for (int q = 0; q < NOUT; ++q) {
+            const int o = (int)threadIdx.x + q * NW * 64;
+            if (o >= MT * 256) continue;
             const int mt = o >> 8, row16 = (o & 255) >> 4, col = o & 15;
             const int src = (mt * 64 + (row16 >> 2) * 16 + col) * 4 + (row16 & 3);
             const int m = m_start + 16 * mt + row16, n = n0 + col;
@@ -334,7 +359,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
 #pragma unroll
                 for (int w = 0; w < NW; ++w) sum += __float_as_int(rbuf[w * MT * 256 + src]);
                 if (p.c_i32) p.c_i32[(int64_t)m * N + n] = sum;
-                if (p.c) st_out(p.c, (int64_t)m * N + n, (float)sum * ((const float*)p.a_s)[m] * ((const float*)p.b_s)[n], p.c_dtype);
+                if (p.c) st_out(p.c, (int64_t)m * N + n, (float)sum * rc_as[q] * rc_bs[q], p.c_dtype);
             } else {
                 float sum = 0.f;
 #pragma unroll
@@ -356,6 +381,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
         if (tile + stride < ntiles) load_b(bnxt, tile + stride, wave);
         auto one = [&](BBatch& cur, BBatch& fill) __attribute__((always_inline)) {
             const int t2 = tile + 2 * stride;
+            request_col_scales(tile);          // ahead of the weight loads: waiting for it must not wait for them
             if (t2 < ntiles) load_b(fill, t2, wave);
             mul_batch(acur, cur, wave, acc, acci);
             finish(tile);
@@ -377,6 +403,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_direct_kernel(DirectArgs p) {
             const int nt = more ? tile : tile + stride;
             const bool any = nt < ntiles;
             const int fk = more ? nk : wave;
+            if (!more) request_col_scales(tile);   // ahead of the loads of the next batch (see above)
             if (any) { load_b(fb, nt, fk); load_a(fa, fk); }
             mul_batch(ca, cb, ks0, acc, acci);
             if (!more) finish(tile);
