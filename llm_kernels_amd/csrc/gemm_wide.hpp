@@ -36,7 +36,26 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
     const int KT = K >> 7;
-    const int n0 = blockIdx.x * W_BN;
+    int bx = blockIdx.x, by = blockIdx.y;
+    if constexpr (!GROUPED) {
+        // Workgroups go to the eight XCDs round robin by linear id, each XCD with its own L2, and 256 of them
+        // (one per CU) run at a time.  Within every such round give each XCD a compact block of 8 x 4 tiles of
+        // one strip of four tile rows instead of every eighth tile of the grid, so that its L2 holds few
+        // operand rows and all XCDs of a round share the four activation row tiles.
+        const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+        const int lin = by * gx + bx;
+        if (gy % 4 == 0) {
+            int lp = lin;
+            if (lin < (total & ~255)) {
+                const int w = lin & 255;
+                lp = (lin & ~255) + (w & 7) * 32 + (w >> 3);
+            }
+            const int strip = lp / (4 * gx), rr = lp % (4 * gx);
+            bx = rr / 4;
+            by = strip * 4 + rr % 4;
+        }
+    }
+    const int n0 = bx * W_BN;
 
     int m_start, m_end;
     const uint8_t* bbase = p.b;
@@ -57,7 +76,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         bbase += widx * (int64_t)N * K;
         bs_off = widx * (int64_t)((N + 127) / 128) * KT;
     } else {
-        m_start = blockIdx.y * W_BM;
+        m_start = by * W_BM;
         m_end = min(p.M, m_start + W_BM);
     }
 
@@ -106,7 +125,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     if constexpr (SCALED) {
         for (int i = tid; i < 2 * KT; i += W_THREADS) {
             const int c = i >= KT ? 1 : 0, kk = i - c * KT;
-            const int64_t blk = min(blockIdx.x * 2 + c, nblk - 1);
+            const int64_t blk = min(bx * 2 + c, nblk - 1);
             bsl[c * D_MAX_KT + kk] = ld_scale(p.b_s, bs_off + blk * KT + kk, p.s_dtype);
         }
     }
