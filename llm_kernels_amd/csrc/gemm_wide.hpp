@@ -5,8 +5,10 @@
 //
 // Workgroup: 512 threads = 8 waves, 2 along M x 4 along N; wave tile 128 rows x 64 columns =
 // 8 x 4 MFMA tiles (128 accumulator registers per lane).  Two LDS stages of 66560 bytes
-// (A 32 KB, B 32 KB, activation-scale column 1 KB): the loads of K step kt+2 are issued behind the
-// one barrier of step kt, which sits before its last tile row; they fly while step kt+1 is multiplied.
+// (A 32 KB, B 32 KB, activation-scale column 1 KB).  A step has two barriers: one in the middle, behind
+// which the weight rows of K step kt+2 are requested (every wave holds the weight fragments of step kt in
+// registers by then), and one before its last tile row, behind which the activation rows of step kt+2 are
+// requested and the fragments of step kt+1 fetched; the loads fly while step kt+1 is multiplied.
 //
 // Inside a step a wave keeps its four weight fragments in registers for the whole step and streams
 // the eight activation fragments through a two-deep register buffer.  The product of tile n is
@@ -21,6 +23,7 @@ namespace llmk {
 constexpr int W_BM = 256, W_BN = 256, W_THREADS = 512;
 constexpr int W_A = W_BM * 128, W_B = W_BN * 128, W_S = W_BM * 4;
 constexpr int W_STAGE = W_A + W_B + W_S;                   // 66560
+constexpr int W_EARLY_ROW = 5;                             // tile row in front of which the mid-step barrier sits
 constexpr int W_LDS = 2 * W_STAGE + 2 * D_MAX_KT * 4;      // 135168 bytes
 
 template <int KIND, bool GROUPED>
@@ -115,15 +118,18 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         if constexpr (SCALED) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
     };
 
-    // a quarter of the loads of a stage (part 0..3)
+    // The loads of a stage inside the loop, a quarter at a time (part 0..3): the weight rows behind the
+    // mid-step barrier, the activation rows and the scale column behind the barrier of the step.
     auto issue_part = [&](int kt, int part) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
         const uint8_t* ga = p.a + (int64_t)kt * 128;
-        const uint8_t* gb = bbase + (int64_t)kt * 128;
         const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
         dma16(st + (uint32_t)(wave * 4 + part) * 1024u, aoff[part], ga);
-        dma16(st + W_A + (uint32_t)(wave * 4 + part) * 1024u, boff[part], gb);
         if constexpr (SCALED) if (part == 3) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+    };
+    auto issue_b_part = [&](int kt, int part) {
+        const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
+        dma16(st + W_A + (uint32_t)(wave * 4 + part) * 1024u, boff[part], bbase + (int64_t)kt * 128);
     };
 
     // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 128 x 64 tile
@@ -190,9 +196,20 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             if (i + 1 < NR) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+            if (i == W_EARLY_ROW && ISSUE) {
+                // Every wave has had its weight fragments of this step in registers since the step began, so
+                // behind this barrier the weight half of the stage may be overwritten: the weight loads of
+                // step kt + 2 go out here, the activation loads behind the barrier of row 7.  Two bursts of
+                // loads per step instead of one measured 4-6 % faster (rows 4 and 5 best, 0 and 1 no gain).
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if (i == 7 && SYNC) {
                 __builtin_amdgcn_sched_barrier(0);
-                __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
+                // vmcnt(4): the four weight loads of step kt + 2 may stay in flight; lgkmcnt(0)
+                if constexpr (ISSUE) __builtin_amdgcn_s_waitcnt(0x0074);
+                else __builtin_amdgcn_s_waitcnt(0x0070);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -205,8 +222,9 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                 } else {
                     if (i < NR) acc[i][j] = mma_plain<KIND>(bf[j], af[i & 1], acc[i][j]);
                 }
+                if (i == W_EARLY_ROW && ISSUE) issue_b_part(kt + 2, j);
                 if (i == 7 && SYNC) {
-                    if (ISSUE) issue_part(kt + 2, j);      // a quarter of the stage behind each tile (measured 0.5-1 % faster than all at once)
+                    if (ISSUE) issue_part(kt + 2, j);      // a quarter behind each tile (0.5-1 % faster than all at once)
                     if (NR > 0) {
                         bf[j] = ldfrag(stage_b(kt + 1) + j * 2048);
                         if (j == 3) af[0] = ldfrag(stage_a(kt + 1));
