@@ -282,6 +282,25 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         w4_lds = (uint32_t)R * 128u + (uint32_t)((2 * q) ^ ((R >> 1) & 7)) * 16u;   // chunk 2q; chunk 2q+1 is at ^16
     }
 
+    // the same loads in two bursts for the block-scaled kinds on the taller tiles: activation rows before the
+    // step is multiplied, weight rows and scale column between its two phases (the buffer they go to was
+    // released by the barrier of the previous step; 2-5 % faster for int8, even for fp8)
+    auto issue_b_half = [&](int kt) {
+        const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
+        const uint8_t* gb = bbase + (int64_t)(kt0 + kt) * 128;
+        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
+        if constexpr (!W4) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) dma16(st + D_A + (uint32_t)(wave * 2 + i) * 1024u, boff[i], gb);
+        }
+        if constexpr (SCALED) dma4(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+    };
+    auto issue_a_half = [&](int kt) {
+        const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
+        const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) dma16(st + (uint32_t)(wave * MI + i) * 1024u, aoff[i], ga);
+    };
     auto issue = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
         const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
@@ -416,6 +435,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // The weight fragment is the MFMA row operand and the activation fragment the column operand, i.e.
     // the tile is produced transposed: a lane owns output row r and four consecutive columns per MFMA.
     // Branch-free so that the whole body is a single scheduling region.
+    int mid_kt = -1;                    // >= 0: stage whose second half of loads goes out between the phases
     auto compute = [&]() {
         if constexpr (!SCALED) {
 #pragma unroll
@@ -440,6 +460,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
                     __builtin_amdgcn_sched_group_barrier(0x008, KIND == K_FP8_BLOCK ? 1 : 2, 0);
                     __builtin_amdgcn_sched_group_barrier(0x002, KIND == K_FP8_BLOCK ? 4 : 8, 0);
                 }
+            if (mid_kt >= 0) { issue_b_half(mid_kt); mid_kt = -1; }
             // phase 2: Y <- lower tile rows of this step; retire X into the upper acc rows
 #pragma unroll
             for (int i = 0; i < H; ++i)
@@ -465,7 +486,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         for (; kt + 2 < KT; ++kt) {
             w4_expand(kt + 1);
             w4_request(kt + 2);
-            issue(kt + 2);
+            if constexpr (SCALED && MI >= 2) { issue_a_half(kt + 2); mid_kt = kt + 2; } else issue(kt + 2);
             load_frags(kt);
             compute();
             __builtin_amdgcn_s_waitcnt(WAIT_ONE_STAGE);
@@ -487,7 +508,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         for (; kt + 2 < KT; ++kt) {
             w4_expand(kt + 1);
             w4_request(kt + 2);
-            issue(kt + 2);
+            if constexpr (SCALED && MI >= 2) { issue_a_half(kt + 2); mid_kt = kt + 2; } else issue(kt + 2);
             compute();
             __builtin_amdgcn_sched_barrier(0);
             load_frags(kt);

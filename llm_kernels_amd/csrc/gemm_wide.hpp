@@ -323,7 +323,7 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
 }
 
 // Tile shape by estimated time: rounds of 256 workgroups times the measured cost of one round of each tile
-// shape (microseconds at K = 4096 for fp8; the ratios hold for the other kinds and K).  Ties go to the larger
+// shape (60 / 43 / 26 / 16 microseconds at K = 4096 for fp8; the ratios hold for the other kinds and K).  Ties go to the larger
 // tile (less operand re-reading).  Segments of a grouped GEMM are judged by their average length.
 template <int KIND, bool GROUPED>
 int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
@@ -332,7 +332,7 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
     auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm) + 255) / 256; };
-    const double t_wide = 64.0 * rounds(256, 256), t4 = 43.0 * rounds(256, 128), t2 = 26.0 * rounds(128, 128),
+    const double t_wide = 60.0 * rounds(256, 256), t4 = 43.0 * rounds(256, 128), t2 = 26.0 * rounds(128, 128),
                  t1 = 16.0 * rounds(64, 128);
     if constexpr (HAS_WIDE) {
         if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) return launch_wide<KIND, GROUPED>(p, stream, name);
