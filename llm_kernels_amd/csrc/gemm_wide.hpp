@@ -182,6 +182,24 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     // loop that neither fetches nor multiplies the tile rows from NR on (their accumulators are never
     // stored); the loop is instantiated for NR = 8, 4 and 0 so that it stays free of branches (a two-row variant
     // measured no faster: short tails are bound by the per-step barrier, not by the matrix pipe).
+    // every lane writes 16 consecutive outputs of each of its eight rows; row i of the wave tile:
+    const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
+    const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
+    const int nb = n0 + wn * 64 + 16 * g;
+    const int n_valid = N - nb;
+    auto store_row = [&](int i) {
+        const int m = m_start + wm * 128 + 16 * i + r;
+        if (m >= m_end || n_valid <= 0) return;
+        const int64_t off = (int64_t)m * N + nb;
+        if constexpr (KIND == K_I8_ROWCOL) {
+            rowcol_epilogue(p, acc[i], m, off, nb, n_valid);
+            if (!p.c) return;
+        }
+        if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
+        else if (p.c_dtype == LLMK_F16) store_row16<LLMK_F16>(p.c, off, acc[i], n_valid, vec_ok);
+        else store_row16<LLMK_F32>(p.c, off, acc[i], n_valid, vec_ok);
+    };
+
     auto step = [&](int kt, auto sync_c, auto issue_c, auto nr_c) {
         constexpr bool SYNC = decltype(sync_c)::value, ISSUE = decltype(issue_c)::value;
         constexpr int NR = decltype(nr_c)::value;
@@ -235,6 +253,11 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                 // tile row before its first use.
                 __builtin_amdgcn_sched_barrier(0);
             }
+            // last K step: the outputs of tile row i - 1 are final once row i has been issued; storing them
+            // here overlaps the conversion and the write with the rest of the step
+            if constexpr (!SYNC) {
+                if (i >= 1 && i <= NR) store_row(i - 1);
+            }
         }
         if constexpr (SCALED && NR == 8) sprev = sa[7];
     };
@@ -266,24 +289,10 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         run(std::integral_constant<int, 8>{});
     }
 
-    // ---- epilogue: every lane writes 16 consecutive outputs of each of its eight rows
-    const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
-    const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
-    const int nb = n0 + wn * 64 + 16 * g;
-    const int n_valid = N - nb;
+    // ---- epilogue: the rows not yet stored by the last K step
+    if (KT > 0) { store_row(7); return; }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int m = m_start + wm * 128 + 16 * i + r;
-        if (m >= m_end || n_valid <= 0) continue;
-        const int64_t off = (int64_t)m * N + nb;
-        if constexpr (KIND == K_I8_ROWCOL) {
-            rowcol_epilogue(p, acc[i], m, off, nb, n_valid);
-            if (!p.c) continue;
-        }
-        if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
-        else if (p.c_dtype == LLMK_F16) store_row16<LLMK_F16>(p.c, off, acc[i], n_valid, vec_ok);
-        else store_row16<LLMK_F32>(p.c, off, acc[i], n_valid, vec_ok);
-    }
+    for (int i = 0; i < 8; ++i) store_row(i);
 }
 
 template <int KIND, bool GROUPED>
