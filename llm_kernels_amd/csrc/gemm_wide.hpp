@@ -20,14 +20,20 @@
 
 namespace llmk {
 
-constexpr int W_BM = 256, W_BN = 256, W_THREADS = 512;
-constexpr int W_A = W_BM * 128, W_B = W_BN * 128, W_S = W_BM * 4;
-constexpr int W_STAGE = W_A + W_B + W_S;                   // 66560
-constexpr int W_EARLY_ROW = 5;                             // tile row in front of which the mid-step barrier sits
-constexpr int W_LDS = 2 * W_STAGE + 2 * D_MAX_KT * 4;      // 135168 bytes
+// R = tile rows (of 16) per wave: 8 gives the 256 x 256 tile described above, 4 a 128 x 256 tile (wave tile
+// 64 x 64) with the same loop for problems with too few rows for a round of the large tile.
+constexpr int W_BN = 256, W_THREADS = 512;
+constexpr int W_B = W_BN * 128, W_S = 256 * 4;
+constexpr int w_bm(int r) { return 32 * r; }
+constexpr int w_stage(int r) { return w_bm(r) * 128 + W_B + W_S; }        // 66560 / 50176
+constexpr int w_lds(int r) { return 2 * w_stage(r) + 2 * D_MAX_KT * 4; }  // 135168 / 102400 bytes
 
-template <int KIND, bool GROUPED>
+template <int KIND, bool GROUPED, int R = 8>
 __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
+    static_assert(R == 8 || (R == 4 && !GROUPED), "tile rows per wave");
+    constexpr int W_BM = w_bm(R), W_A = W_BM * 128, W_STAGE = w_stage(R);
+    constexpr int AL = R / 2;                    // activation loads per thread and stage
+    constexpr int W_EARLY_ROW = R == 8 ? 5 : 2;  // tile row in front of which the mid-step barrier sits
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -94,17 +100,22 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     // g, the four columns 16g + 4j + (0..3) and a lane ends up with 16 consecutive columns of a row.
     // The 16-byte chunk index is XOR-swizzled with ((R >> 1) & 7) on the global side.
     const int row8 = lane >> 3;
-    uint32_t aoff[4], boff[4];
+    uint32_t aoff[AL], boff[4];
+#pragma unroll
+    for (int i = 0; i < AL; ++i) {
+        const int row = 8 * (wave * AL + i) + row8;
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
+        aoff[i] = (uint32_t)min(m_start + row, m_end - 1) * (uint32_t)K + chunk;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int R = 8 * (wave * 4 + i) + row8;
-        const uint32_t chunk = (uint32_t)((lane & 7) ^ ((R >> 1) & 7)) * 16u;
-        aoff[i] = (uint32_t)min(m_start + R, m_end - 1) * (uint32_t)K + chunk;
-        const int rho = R & 63;
-        const int col = (R & 192) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
+        const int row = 8 * (wave * 4 + i) + row8;
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
+        const int rho = row & 63;
+        const int col = (row & 192) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
-    const uint32_t soff = (uint32_t)min(m_start + (wave & 3) * 64 + lane, m_end - 1) * (uint32_t)KT * 4u;
+    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT * 4u;
 
     auto issue = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
@@ -112,7 +123,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const uint8_t* gb = bbase + (int64_t)kt * 128;
         const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(st + (uint32_t)(wave * 4 + i) * 1024u, aoff[i], ga);
+        for (int i = 0; i < AL; ++i) dma16(st + (uint32_t)(wave * AL + i) * 1024u, aoff[i], ga);
 #pragma unroll
         for (int i = 0; i < 4; ++i) dma16(st + W_A + (uint32_t)(wave * 4 + i) * 1024u, boff[i], gb);
         if constexpr (SCALED) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
@@ -124,7 +135,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
         const uint8_t* ga = p.a + (int64_t)kt * 128;
         const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
-        dma16(st + (uint32_t)(wave * 4 + part) * 1024u, aoff[part], ga);
+        if (part < AL) dma16(st + (uint32_t)(wave * AL + part) * 1024u, aoff[part < AL ? part : 0], ga);
         if constexpr (SCALED) if (part == 3) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
     };
     auto issue_b_part = [&](int kt, int part) {
@@ -132,10 +143,10 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         dma16(st + W_A + (uint32_t)(wave * 4 + part) * 1024u, boff[part], bbase + (int64_t)kt * 128);
     };
 
-    // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 128 x 64 tile
-    v4f acc[8][4];
+    // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 16 R x 64 tile
+    v4f acc[R][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < R; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
@@ -170,7 +181,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     // Fragments of the step being multiplied.  bf and af[0] of step kt + 1 are fetched during the last
     // tile row of step kt, so that a step starts with its operands already in registers.
     v8i bf[4], af[2];
-    auto stage_a = [&](int kt) { return lds + (kt & 1) * W_STAGE + (wm * 128) * 128; };
+    auto stage_a = [&](int kt) { return lds + (kt & 1) * W_STAGE + (wm * 16 * R) * 128; };
     auto stage_b = [&](int kt) { return lds + (kt & 1) * W_STAGE + W_A + (wn * 64) * 128; };
 
     // One K step.  SYNC: another step follows; before the last tile row the wave waits for its share of
@@ -188,7 +199,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     const int nb = n0 + wn * 64 + 16 * g;
     const int n_valid = N - nb;
     auto store_row = [&](int i) {
-        const int m = m_start + wm * 128 + 16 * i + r;
+        const int m = m_start + wm * 16 * R + 16 * i + r;
         if (m >= m_end || n_valid <= 0) return;
         const int64_t off = (int64_t)m * N + nb;
         if constexpr (KIND == K_I8_ROWCOL) {
@@ -204,15 +215,15 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         constexpr bool SYNC = decltype(sync_c)::value, ISSUE = decltype(issue_c)::value;
         constexpr int NR = decltype(nr_c)::value;
         const uint8_t* As = stage_a(kt);
-        float sa[8];
+        float sa[R];
         if constexpr (SCALED && NR > 0) {
-            const float* Ss = (const float*)(lds + (kt & 1) * W_STAGE + W_A + W_B) + wm * 128 + r;
+            const float* Ss = (const float*)(lds + (kt & 1) * W_STAGE + W_A + W_B) + wm * 16 * R + r;
             const float bs = bsl[(wn >> 1) * D_MAX_KT + kt];
 #pragma unroll
             for (int i = 0; i < NR; ++i) sa[i] = Ss[i * 16] * bs;
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < R; ++i) {
             if (i + 1 < NR) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
             if (i == W_EARLY_ROW && ISSUE) {
                 // Every wave has had its weight fragments of this step in registers since the step began, so
@@ -223,7 +234,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                 __builtin_amdgcn_s_barrier();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (i == 7 && SYNC) {
+            if (i == R - 1 && SYNC) {
                 __builtin_amdgcn_sched_barrier(0);
                 // vmcnt(4): the four weight loads of step kt + 2 may stay in flight; lgkmcnt(0)
                 if constexpr (ISSUE) __builtin_amdgcn_s_waitcnt(0x0074);
@@ -236,12 +247,12 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                 if constexpr (SCALED) {
                     if (i < NR) t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
                     if (i > 0 && i <= NR) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
-                    else if (i == 0 && NR == 8) acc[7][j] += t[1][j] * sprev;
+                    else if (i == 0 && NR == R) acc[R - 1][j] += t[1][j] * sprev;
                 } else {
                     if (i < NR) acc[i][j] = mma_plain<KIND>(bf[j], af[i & 1], acc[i][j]);
                 }
                 if (i == W_EARLY_ROW && ISSUE) issue_b_part(kt + 2, j);
-                if (i == 7 && SYNC) {
+                if (i == R - 1 && SYNC) {
                     if (ISSUE) issue_part(kt + 2, j);      // a quarter behind each tile (0.5-1 % faster than all at once)
                     if (NR > 0) {
                         bf[j] = ldfrag(stage_b(kt + 1) + j * 2048);
@@ -259,7 +270,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                 if (i >= 1 && i <= NR) store_row(i - 1);
             }
         }
-        if constexpr (SCALED && NR == 8) sprev = sa[7];
+        if constexpr (SCALED && NR == R) sprev = sa[R - 1];
     };
 
     if (KT > 1) issue(1);
@@ -275,9 +286,9 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         for (; kt + 2 < KT; ++kt) step(kt, yes, yes, nr_c);
         if (kt + 1 < KT) { step(kt, yes, no, nr_c); ++kt; }
         if (kt < KT) step(kt, no, no, nr_c);
-        if constexpr (SCALED && decltype(nr_c)::value == 8) {
+        if constexpr (SCALED && decltype(nr_c)::value == R) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[7][j] += t[1][j] * sprev;
+            for (int j = 0; j < 4; ++j) acc[R - 1][j] += t[1][j] * sprev;
         }
     };
     if constexpr (GROUPED) {
@@ -286,19 +297,20 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         else if (live > 0) run(std::integral_constant<int, 4>{});
         else run(std::integral_constant<int, 0>{});
     } else {
-        run(std::integral_constant<int, 8>{});
+        run(std::integral_constant<int, R>{});
     }
 
     // ---- epilogue: the rows not yet stored by the last K step
-    if (KT > 0) { store_row(7); return; }
+    if (KT > 0) { store_row(R - 1); return; }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) store_row(i);
+    for (int i = 0; i < R; ++i) store_row(i);
 }
 
-template <int KIND, bool GROUPED>
+template <int KIND, bool GROUPED, int R = 8>
 int launch_wide(const DirectArgs& p, hipStream_t stream, const char* name) {
     static bool configured = false;
-    auto kern = gemm_wide_kernel<KIND, GROUPED>;
+    auto kern = gemm_wide_kernel<KIND, GROUPED, R>;
+    constexpr int W_BM = w_bm(R), W_LDS = w_lds(R);
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, W_LDS);
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, W_LDS, hipGetErrorString(e));
@@ -332,8 +344,8 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
 }
 
 // Tile shape by estimated time: rounds of 256 workgroups times the measured cost of one round of each tile
-// shape (60 / 43 / 26 / 16 microseconds at K = 4096 for fp8; the ratios hold for the other kinds and K).  Ties go to the larger
-// tile (less operand re-reading).  Segments of a grouped GEMM are judged by their average length.
+// shape (60 / 36 / 43 / 26 / 16 microseconds for 256 x 256, 128 x 256, 256 x 128, 128 x 128 and 64 x 128 at K = 4096
+// for fp8; the ratios hold for the other kinds and K).  Ties go to the larger tile (less operand re-reading).  Segments of a grouped GEMM are judged by their average length.
 template <int KIND, bool GROUPED>
 int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
@@ -344,7 +356,17 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     const double t_wide = 60.0 * rounds(256, 256), t4 = 43.0 * rounds(256, 128), t2 = 26.0 * rounds(128, 128),
                  t1 = 16.0 * rounds(64, 128);
     if constexpr (HAS_WIDE) {
-        if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) return launch_wide<KIND, GROUPED>(p, stream, name);
+        if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) {
+            // dense problems whose 256 x 256 tiles do not fill a round: the 128 x 256 tile of the same kernel
+            if constexpr (!GROUPED) {
+                if (36.0 * rounds(128, 256) < t_wide) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
+            }
+            return launch_wide<KIND, GROUPED>(p, stream, name);
+        }
+        if constexpr (!GROUPED) {
+            const double t_half = 36.0 * rounds(128, 256);
+            if (t_half < t4 && t_half <= t2 && t_half <= t1) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
+        }
     }
     if (t4 <= t2 && t4 <= t1) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
     if (t2 <= t1) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
