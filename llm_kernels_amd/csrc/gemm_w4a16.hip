@@ -231,13 +231,18 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const v4i* __restri
             }
     }
     __syncthreads();
-    const int row = tid >> 2, seg = tid & 3;
+    // eight lanes write one 128-byte line of a row per instruction
+    const int seg = tid & 7;
     const int k0 = blockIdx.y * 128;
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-        const int kl = seg * 32 + x * 8;
-        if (k0 + kl < K)
-            *(v8h*)(Wt + (int64_t)(64 * chunk + row) * K + k0 + kl) = *(const v8h*)&tile[row][kl];
+    for (int pass = 0; pass < 2; ++pass) {
+        const int row = pass * 32 + (tid >> 3);
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            const int kl = x * 64 + seg * 8;
+            if (k0 + kl < K)
+                *(v8h*)(Wt + (int64_t)(64 * chunk + row) * K + k0 + kl) = *(const v8h*)&tile[row][kl];
+        }
     }
 }
 
