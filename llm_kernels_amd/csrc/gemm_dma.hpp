@@ -176,6 +176,58 @@ __device__ __forceinline__ unsigned asm_load_u16(uint32_t voff, const void* sbas
     return v;
 }
 
+// ---- the same for runs of 8 consecutive outputs (two MFMA results), used by the 256-column kernel, whose lanes
+// own two such runs per row so that the four lane groups of a row write 64 contiguous bytes per instruction
+template <int ODT>
+__device__ __forceinline__ void store_run8(void* c, int64_t off, const v4f& a, const v4f& b, int n_valid, bool vec_ok) {
+    if (vec_ok && n_valid >= 8) {
+        if constexpr (ODT == LLMK_F32) {
+            v4f* dst = (v4f*)((float*)c + off);
+            dst[0] = a;
+            dst[1] = b;
+        } else {
+            v4i w;
+            w[0] = (int)(ODT == LLMK_F16 ? pack_f16x2(a[0], a[1]) : pack_bf16x2(a[0], a[1]));
+            w[1] = (int)(ODT == LLMK_F16 ? pack_f16x2(a[2], a[3]) : pack_bf16x2(a[2], a[3]));
+            w[2] = (int)(ODT == LLMK_F16 ? pack_f16x2(b[0], b[1]) : pack_bf16x2(b[0], b[1]));
+            w[3] = (int)(ODT == LLMK_F16 ? pack_f16x2(b[2], b[3]) : pack_bf16x2(b[2], b[3]));
+            *(v4i*)((unsigned short*)c + off) = w;
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (q < n_valid) FloatIO<ODT>::st(c, off + q, a[q]);
+            if (4 + q < n_valid) FloatIO<ODT>::st(c, off + 4 + q, b[q]);
+        }
+    }
+}
+__device__ __forceinline__ void store_run8_i32(int32_t* c, int64_t off, const v4f& a, const v4f& b, int n_valid, bool vec_ok) {
+    if (vec_ok && n_valid >= 8) {
+        v4f* dst = (v4f*)(c + off);
+        dst[0] = a;          // raw bits
+        dst[1] = b;
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (q < n_valid) c[off + q] = __float_as_int(a[q]);
+            if (4 + q < n_valid) c[off + 4 + q] = __float_as_int(b[q]);
+        }
+    }
+}
+__device__ __forceinline__ void rowcol_epilogue8(const DirectArgs& p, v4f& a, v4f& b, int m, int64_t off, int nb, int n_valid) {
+    if (p.c_i32) {
+        const bool vec_i = ((((uintptr_t)p.c_i32) & 15) == 0) && (p.N % 4 == 0);
+        store_run8_i32(p.c_i32, off, a, b, n_valid, vec_i);
+    }
+    if (!p.c) return;
+    const float as = ((const float*)p.a_s)[m];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        a[q] = (float)__float_as_int(a[q]) * as * ((const float*)p.b_s)[nb + min(q, n_valid - 1)];
+        b[q] = (float)__float_as_int(b[q]) * as * ((const float*)p.b_s)[nb + min(4 + q, n_valid - 1)];
+    }
+}
+
 // MI = 16-row tiles per wave along M (4, 2 or 1): the workgroup tile is 64*MI rows x 128 columns.
 template <int KIND, bool GROUPED, int MI>
 __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {

@@ -96,8 +96,10 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 
     // ---- source offsets of the 9 loads of a stage.  Load i of a wave fills LDS rows 8q .. 8q+7,
     // q = 4*wave + i.  A: LDS row R holds tile row R.  B: within each 64-row group, LDS row rho holds
-    // tile column 16*((rho & 15) >> 2) + 4*(rho >> 4) + (rho & 3), so that MFMA j yields, in lane group
-    // g, the four columns 16g + 4j + (0..3) and a lane ends up with 16 consecutive columns of a row.
+    // tile column 32*(rho >> 5) + 8*((rho & 15) >> 2) + 4*((rho >> 4) & 1) + (rho & 3), so that MFMA j yields,
+    // in lane group g, the four columns 32*(j >> 1) + 8g + 4*(j & 1) + (0..3): a lane ends up with two runs
+    // of 8 consecutive columns of a row, and the four lane groups of a row write 64 contiguous bytes per
+    // store instruction (1-2 % faster than 16 columns per lane, whose stores leave 16-byte gaps).
     // The 16-byte chunk index is XOR-swizzled with ((R >> 1) & 7) on the global side.
     const int row8 = lane >> 3;
     uint32_t aoff[AL], boff[4];
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const int row = 8 * (wave * 4 + i) + row8;
         const uint32_t chunk = (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
         const int rho = row & 63;
-        const int col = (row & 192) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
+        const int col = (row & 192) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
     const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT * 4u;
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         dma16(st + W_A + (uint32_t)(wave * 4 + part) * 1024u, boff[part], bbase + (int64_t)kt * 128);
     };
 
-    // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 16 R x 64 tile
+    // acc[i][j][q] = C[row 16i + r][col 32*(j >> 1) + 8g + 4*(j & 1) + q] of the wave's 16 R x 64 tile
     v4f acc[R][4];
 #pragma unroll
     for (int i = 0; i < R; ++i)
@@ -184,33 +186,37 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     auto stage_a = [&](int kt) { return lds + (kt & 1) * W_STAGE + (wm * 16 * R) * 128; };
     auto stage_b = [&](int kt) { return lds + (kt & 1) * W_STAGE + W_A + (wn * 64) * 128; };
 
+    // every lane writes two runs of 8 consecutive outputs of each of its rows; row i of the wave tile:
+    const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
+    const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
+    auto store_row = [&](int i) {
+        const int m = m_start + wm * 16 * R + 16 * i + r;
+        if (m >= m_end) return;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int nbh = n0 + wn * 64 + 32 * h + 8 * g;
+            const int nv = N - nbh;
+            if (nv <= 0) continue;
+            const int64_t off = (int64_t)m * N + nbh;
+            if constexpr (KIND == K_I8_ROWCOL) {
+                rowcol_epilogue8(p, acc[i][2 * h], acc[i][2 * h + 1], m, off, nbh, nv);
+                if (!p.c) continue;
+            }
+            if (p.c_dtype == LLMK_BF16) store_run8<LLMK_BF16>(p.c, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
+            else if (p.c_dtype == LLMK_F16) store_run8<LLMK_F16>(p.c, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
+            else store_run8<LLMK_F32>(p.c, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
+        }
+    };
+
     // One K step.  SYNC: another step follows; before the last tile row the wave waits for its share of
     // the next stage and for its own LDS reads, and meets the others at the barrier.  Behind the barrier
     // the next stage is complete and nobody reads the current one any more, so the loads of step kt + 2
-    // (ISSUE) may overwrite it, and the fragments of step kt + 1 are fetched while row 7 is multiplied.
-    // NR = tile rows (of 16) this wave multiplies.  Dense GEMM: always 8.  Grouped GEMM: the last m-tile of
+    // (ISSUE) may overwrite it, and the fragments of step kt + 1 are fetched while the last row is multiplied.
+    // NR = tile rows (of 16) this wave multiplies.  Dense GEMM: always R.  Grouped GEMM: the last m-tile of
     // a segment is ragged, and a wave whose rows lie (partly) behind the segment end runs a variant of the
     // loop that neither fetches nor multiplies the tile rows from NR on (their accumulators are never
     // stored); the loop is instantiated for NR = 8, 4 and 0 so that it stays free of branches (a two-row variant
     // measured no faster: short tails are bound by the per-step barrier, not by the matrix pipe).
-    // every lane writes 16 consecutive outputs of each of its eight rows; row i of the wave tile:
-    const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
-    const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
-    const int nb = n0 + wn * 64 + 16 * g;
-    const int n_valid = N - nb;
-    auto store_row = [&](int i) {
-        const int m = m_start + wm * 16 * R + 16 * i + r;
-        if (m >= m_end || n_valid <= 0) return;
-        const int64_t off = (int64_t)m * N + nb;
-        if constexpr (KIND == K_I8_ROWCOL) {
-            rowcol_epilogue(p, acc[i], m, off, nb, n_valid);
-            if (!p.c) return;
-        }
-        if (p.c_dtype == LLMK_BF16) store_row16<LLMK_BF16>(p.c, off, acc[i], n_valid, vec_ok);
-        else if (p.c_dtype == LLMK_F16) store_row16<LLMK_F16>(p.c, off, acc[i], n_valid, vec_ok);
-        else store_row16<LLMK_F32>(p.c, off, acc[i], n_valid, vec_ok);
-    };
-
     auto step = [&](int kt, auto sync_c, auto issue_c, auto nr_c) {
         constexpr bool SYNC = decltype(sync_c)::value, ISSUE = decltype(issue_c)::value;
         constexpr int NR = decltype(nr_c)::value;
