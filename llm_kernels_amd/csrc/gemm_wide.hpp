@@ -30,7 +30,7 @@ constexpr int w_lds(int r) { return 2 * w_stage(r) + 2 * D_MAX_KT * 4; }  // 135
 
 template <int KIND, bool GROUPED, int R = 8>
 __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
-    static_assert(R == 8 || (R == 4 && !GROUPED), "tile rows per wave");
+    static_assert(R == 8 || R == 4, "tile rows per wave");
     constexpr int W_BM = w_bm(R), W_A = W_BM * 128, W_STAGE = w_stage(R);
     constexpr int AL = R / 2;                    // activation loads per thread and stage
     constexpr int W_EARLY_ROW = R == 8 ? 5 : 2;  // tile row in front of which the mid-step barrier sits
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     // NR = tile rows (of 16) this wave multiplies.  Dense GEMM: always R.  Grouped GEMM: the last m-tile of
     // a segment is ragged, and a wave whose rows lie (partly) behind the segment end runs a variant of the
     // loop that neither fetches nor multiplies the tile rows from NR on (their accumulators are never
-    // stored); the loop is instantiated for NR = 8, 4 and 0 so that it stays free of branches (a two-row variant
+    // stored); the loop is instantiated for NR = R, R / 2 and 0 so that it stays free of branches (a two-row variant
     // measured no faster: short tails are bound by the per-step barrier, not by the matrix pipe).
     auto step = [&](int kt, auto sync_c, auto issue_c, auto nr_c) {
         constexpr bool SYNC = decltype(sync_c)::value, ISSUE = decltype(issue_c)::value;
@@ -298,9 +298,9 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         }
     };
     if constexpr (GROUPED) {
-        const int live = m_end - m_start - wm * 128;       // rows of this wave inside the segment (wave-uniform)
-        if (live > 64) run(std::integral_constant<int, 8>{});
-        else if (live > 0) run(std::integral_constant<int, 4>{});
+        const int live = m_end - m_start - wm * 16 * R;    // rows of this wave inside the segment (wave-uniform)
+        if (live > 8 * R) run(std::integral_constant<int, R>{});
+        else if (live > 0) run(std::integral_constant<int, R / 2>{});
         else run(std::integral_constant<int, 0>{});
     } else {
         run(std::integral_constant<int, R>{});
@@ -363,16 +363,12 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
                  t1 = 16.0 * rounds(64, 128);
     if constexpr (HAS_WIDE) {
         if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) {
-            // dense problems whose 256 x 256 tiles do not fill a round: the 128 x 256 tile of the same kernel
-            if constexpr (!GROUPED) {
-                if (36.0 * rounds(128, 256) < t_wide) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
-            }
+            // problems whose 256 x 256 tiles do not fill a round: the 128 x 256 tile of the same kernel
+            if (36.0 * rounds(128, 256) < t_wide) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
             return launch_wide<KIND, GROUPED>(p, stream, name);
         }
-        if constexpr (!GROUPED) {
-            const double t_half = 36.0 * rounds(128, 256);
-            if (t_half < t4 && t_half <= t2 && t_half <= t1) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
-        }
+        const double t_half = 36.0 * rounds(128, 256);
+        if (t_half < t4 && t_half <= t2 && t_half <= t1) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
     }
     if (t4 <= t2 && t4 <= t1) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
     if (t2 <= t1) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
