@@ -6,6 +6,7 @@ from oracle import gemm_ref as g, marlin_ref as mr, quant_ref as q, bitpack_ref 
 from llm_kernels_amd.fast_dequant.simple_marlin.utils import QuantUtils
 from llm_kernels_amd.fast_dequant.simple_marlin.marlin import mul
 from llm_kernels_amd.fast_dequant import w4a16
+from llm_kernels_amd import _lib
 from helpers import announce, assert_close_scaled
 
 pytestmark = pytest.mark.gpu
@@ -206,3 +207,29 @@ def test_w4a16_nk_large_tile_shapes(dev, M, N, K, gs):
     y = w4a16.w4a16_gemm(x.to(dev), torch.from_numpy(packed).to(dev), s.to(dev), gs)
     ref = g.w4a16_gemm(x, qn.t().int().contiguous(), s.t().contiguous(), gs)
     assert_close_scaled(y, ref, what="w4a16 nk large tiles")
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 1024, 4096), (48, 4096, 14336), (300, 520, 1152), (16, 264, 8320)])
+def test_w4a16_without_scratch(dev, M, N, K):
+    """The scratch of both w4a16 entry points is optional: without it the kernels run with one K slice (or the
+    weight-streaming variant) and must agree with the oracle all the same."""
+    announce("w4a16 without scratch", M, N, K)
+    torch.manual_seed(M + N)
+    x = torch.randn(M, K).half()
+    qn, s = q.w4a16_quant_nk(torch.randn(N, K) * 0.02, 128)
+    packed, _ = bp.pack_cols(qn.numpy(), 4, 32)
+    xd, pd, sd = x.to(dev), torch.from_numpy(packed).to(dev), s.to(dev)
+    y = torch.empty(M, N, dtype=torch.half, device=dev)
+    _lib.call("llmk_gemm_w4a16_nk", _lib.ptr(xd), _lib.ptr(pd), _lib.ptr(y), _lib.ptr(sd), _lib.dt(xd.dtype),
+              M, N, K, 128, None, 0, _lib.stream(xd))
+    assert_close_scaled(y, g.w4a16_gemm(x, qn.t().int().contiguous(), s.t().contiguous(), 128), what="nk without scratch")
+    if M % 16 == 0 and N % 64 == 0:
+        A = (torch.randn(M, K) * 0.3).half()
+        W = (torch.randn(K, N) * 0.05).half()
+        _, q4, sm = mr.fake_quantize(W, 128)
+        B, sp = mr.pack(q4, sm, 128)
+        Ad, Bd, spd = A.to(dev), B.to(dev), sp.to(dev)
+        C = torch.zeros(M, N, dtype=torch.half, device=dev)
+        _lib.call("llmk_gemm_w4a16_marlin", _lib.ptr(Ad), _lib.ptr(Bd), _lib.ptr(C), _lib.ptr(spd),
+                  M, N, K, 128, None, 0, _lib.stream(Ad))
+        assert_close_scaled(C, g.w4a16_gemm(A, q4, sm, 128), what="marlin without scratch")
