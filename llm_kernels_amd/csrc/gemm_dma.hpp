@@ -42,54 +42,6 @@ __device__ __forceinline__ void dma4(uint32_t lds_addr, uint32_t voff, const voi
 #define LLMK_WAIT_VMCNT_0 0x0F70
 
 
-// 16 consecutive outputs of one row -> memory (vector stores when the row segment is 16-byte aligned)
-template <int ODT>
-__device__ __forceinline__ void store_row16(void* c, int64_t off, const v4f (&v)[4], int n_valid, bool vec_ok) {
-    if (vec_ok && n_valid >= 16) {
-        if constexpr (ODT == LLMK_F32) {
-            v4f* dst = (v4f*)((float*)c + off);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) dst[j] = v[j];
-        } else {
-            v4i lo, hi;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                v4i w;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float x = v[2 * j + (q >> 1)][2 * (q & 1)], y = v[2 * j + (q >> 1)][2 * (q & 1) + 1];
-                    w[q] = (int)(ODT == LLMK_F16 ? pack_f16x2(x, y) : pack_bf16x2(x, y));
-                }
-                if (j == 0) lo = w; else hi = w;
-            }
-            v4i* dst = (v4i*)((unsigned short*)c + off);
-            dst[0] = lo;
-            dst[1] = hi;
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (4 * j + q < n_valid) FloatIO<ODT>::st(c, off + 4 * j + q, v[j][q]);
-    }
-}
-
-// 16 consecutive int32 accumulators of one row -> memory
-__device__ __forceinline__ void store_row16_i32(int32_t* c, int64_t off, const v4f (&v)[4], int n_valid, bool vec_ok) {
-    if (vec_ok && n_valid >= 16) {
-        v4f* dst = (v4f*)(c + off);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) dst[j] = v[j];          // raw bits
-    } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (4 * j + q < n_valid) c[off + 4 * j + q] = __float_as_int(v[j][q]);
-    }
-}
-
 // Unscaled kinds accumulate inside the MFMA over the whole K range: two 16x16x32 half-precision MFMAs, or two
 // 16x16x64 int8 MFMAs whose int32 accumulators travel as raw bits in the fp32 accumulator registers.
 template <int KIND>
@@ -116,28 +68,6 @@ __device__ __forceinline__ v4f mma_plain(const v8i& x, const v8i& y, v4f c) {
         c = mfma_bf16_16x16x32(x0, y0, c);
         return mfma_bf16_16x16x32(x1, y1, c);
     }
-}
-
-// Per-token x per-channel int8, a lane's 16 consecutive outputs of row m: raw accumulators (as bits) ->
-// float(acc) * a_s[m] * b_s[n], in that order, like the weight-streaming kernel.
-__device__ __forceinline__ void rowcol_scale(const DirectArgs& p, v4f (&v)[4], int m, int nb, int n_valid) {
-    const float as = ((const float*)p.a_s)[m];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float bs = ((const float*)p.b_s)[nb + min(4 * j + q, n_valid - 1)];
-            v[j][q] = (float)__float_as_int(v[j][q]) * as * bs;
-        }
-}
-
-// the same with the optional store of the raw accumulators in front
-__device__ __forceinline__ void rowcol_epilogue(const DirectArgs& p, v4f (&v)[4], int m, int64_t off, int nb, int n_valid) {
-    if (p.c_i32) {
-        const bool vec_i = ((((uintptr_t)p.c_i32) & 15) == 0) && (p.N % 4 == 0);
-        store_row16_i32(p.c_i32, off, v, n_valid, vec_i);
-    }
-    if (p.c) rowcol_scale(p, v, m, nb, n_valid);
 }
 
 // ---- 4-bit weights inside the tile kernel (K_W4NK) ----
@@ -176,8 +106,9 @@ __device__ __forceinline__ unsigned asm_load_u16(uint32_t voff, const void* sbas
     return v;
 }
 
-// ---- the same for runs of 8 consecutive outputs (two MFMA results), used by the 256-column kernel, whose lanes
-// own two such runs per row so that the four lane groups of a row write 64 contiguous bytes per instruction
+// ---- epilogue helpers.  A lane owns two runs of 8 consecutive outputs (two MFMA results each) per row, so that
+// the four lane groups of a row write 64 contiguous bytes per store instruction (vector stores when the row
+// segment is 16-byte aligned).
 template <int ODT>
 __device__ __forceinline__ void store_run8(void* c, int64_t off, const v4f& a, const v4f& b, int n_valid, bool vec_ok) {
     if (vec_ok && n_valid >= 8) {
@@ -292,8 +223,9 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // ---- per-thread source offsets (bytes, 32 bit) of the 7 loads of a stage.
     // Load i of a wave fills LDS rows 8q .. 8q+7 with q = wave*4+i (A) or wave*2+i (B), q & 1 == i & 1.
     // A: LDS row R holds tile row R.  B: within each 64-row half, LDS row rho holds tile column
-    // 16*((rho & 15) >> 2) + 4*(rho >> 4) + (rho & 3): MFMA j then produces, in lane group g, the four
-    // columns 16g + 4j + (0..3), so that a lane ends up with 16 consecutive columns of one output row.
+    // 32*(rho >> 5) + 8*((rho & 15) >> 2) + 4*((rho >> 4) & 1) + (rho & 3): MFMA j then produces, in lane group g,
+    // the four columns 32*(j >> 1) + 8g + 4*(j & 1) + (0..3), so that a lane ends up with two runs of 8 consecutive
+    // columns of one output row and a store instruction writes 64 contiguous bytes per row.
     const int row8 = lane >> 3;
     uint32_t aoff[MI], boff[2];
 #pragma unroll
@@ -306,7 +238,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     for (int i = 0; i < 2; ++i) {
         const uint32_t chunk = (uint32_t)((lane & 7) ^ (((i & 1) * 4 + (row8 >> 1)) & 7)) * 16u;
         const int R = 8 * (wave * 2 + i) + row8, rho = R & 63;
-        const int col = (R & 64) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
+        const int col = (R & 64) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
     const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
@@ -327,7 +259,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     }
     if constexpr (W4NK) {
         const int R = tid >> 2, q = tid & 3, rho = R & 63;
-        const int col = (R & 64) + 16 * ((rho & 15) >> 2) + 4 * (rho >> 4) + (rho & 3);
+        const int col = (R & 64) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
         const uint32_t n = (uint32_t)min(n0 + col, N - 1);
         w4_off = n * (uint32_t)(p.K >> 1) + (uint32_t)q * 8u;                  // bytes into the packed matrix
         w4_soff = n * (uint32_t)(p.K / p.group) * 2u;                          // bytes into the scale matrix
@@ -407,7 +339,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
                     const unsigned s16 = (unsigned)(w4_scale >> (16 * (2 * jj + b))) & 0xffffu;
                     const v2h sc = w4_as_h2(s16 | (s16 << 16));
                     const int col = 16 * (j0 + jj) + 8 * b + c;                                 // column in the chunk
-                    const int R = (ch8 ? 64 : 0) + ((col >> 2) & 3) * 16 + (col >> 4) * 4 + (col & 3);   // its LDS row
+                    const int R = (ch8 ? 64 : 0) + (col >> 5) * 32 + ((col >> 2) & 1) * 16 + ((col >> 3) & 3) * 4 + (col & 3);   // its LDS row
                     uint8_t* row = bst + R * 128 + 4 * q;
                     const int sw = (R >> 1) & 7;
                     *(v2h*)(row + ((2 * sl) ^ sw) * 16) = (w4_as_h2((u & 0x000f000fu) | 0x64006400u) - k1032) * sc;
@@ -419,7 +351,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // imm = vmcnt | no expcnt/lgkmcnt wait
     constexpr int WAIT_ONE_STAGE = 0x0F70 | (MI + 2 + (SCALED ? 1 : 0));
 
-    // acc[i][j][q] = C[row 16i + r][col 16g + 4j + q] of the wave's 64 x 64 tile
+    // acc[i][j][q] = C[row 16i + r][col 32*(j >> 1) + 8g + 4*(j & 1) + q] of the wave's 64 x 64 tile
     v4f acc[MI][4];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -594,26 +526,30 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         for (int j = 0; j < 4; ++j) acc[0][j] += tx[0][j] * sy[0];
     }
 
-    // ---- epilogue: every lane writes 16 consecutive outputs of each of its four rows
+    // ---- epilogue: every lane writes two runs of 8 consecutive outputs of each of its rows
     const bool split = !GROUPED && p.ksplit > 1;
     void* cout = split ? (void*)(p.partial + (int64_t)blockIdx.z * p.M * N) : p.c;
     const int cdt = split ? LLMK_F32 : p.c_dtype;
     const int esz = cdt == LLMK_F32 ? 4 : 2;
     const bool vec_ok = ((((uintptr_t)cout) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
-    const int nb = n0 + wn * 64 + 16 * g;
-    const int n_valid = N - nb;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
         const int m = m_start + wm * WR + 16 * i + r;
-        if (m >= m_end || n_valid <= 0) continue;
-        const int64_t off = (int64_t)m * N + nb;
-        if constexpr (KIND == K_I8_ROWCOL) {
-            rowcol_epilogue(p, acc[i], m, off, nb, n_valid);
-            if (!p.c) continue;
+        if (m >= m_end) continue;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int nbh = n0 + wn * 64 + 32 * h + 8 * g;
+            const int nv = N - nbh;
+            if (nv <= 0) continue;
+            const int64_t off = (int64_t)m * N + nbh;
+            if constexpr (KIND == K_I8_ROWCOL) {
+                rowcol_epilogue8(p, acc[i][2 * h], acc[i][2 * h + 1], m, off, nbh, nv);
+                if (!p.c) continue;
+            }
+            if (cdt == LLMK_BF16) store_run8<LLMK_BF16>(cout, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
+            else if (cdt == LLMK_F16) store_run8<LLMK_F16>(cout, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
+            else store_run8<LLMK_F32>(cout, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
         }
-        if (cdt == LLMK_BF16) store_row16<LLMK_BF16>(cout, off, acc[i], n_valid, vec_ok);
-        else if (cdt == LLMK_F16) store_row16<LLMK_F16>(cout, off, acc[i], n_valid, vec_ok);
-        else store_row16<LLMK_F32>(cout, off, acc[i], n_valid, vec_ok);
     }
 }
 
