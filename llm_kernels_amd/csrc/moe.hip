@@ -57,14 +57,23 @@ template <int DT> __device__ __forceinline__ float rnd(float v) {
 // tensor dtype, product in the tensor dtype, optional per-expert scale in the tensor dtype)
 constexpr int AMQ_UNROLL = 4;      // groups per thread of the fused activation + quantisation kernel
 
+// 1 / (1 + e^-x).  For 16-bit tensors the result is rounded to 8 or 11 significant bits right after, so the
+// hardware exp2 and reciprocal (1 ulp each in fp32) are used: large |x| gives exp2 -> inf or 0 and the
+// quotient 0 or 1, as the exact expression does.  fp32 tensors keep the library routines.
+template <int IDT>
+__device__ __forceinline__ float sigmoid_f(float x) {
+    if constexpr (IDT == LLMK_F32) return 1.0f / (1.0f + expf(-x));
+    else return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+
 template <int IDT>
 __device__ __forceinline__ float gated_act(float gv, float up, int act, bool has_scale, float scale) {
     if (act == 0) {
-        gv = gv * (1.0f / (1.0f + expf(-gv)));
+        gv = gv * sigmoid_f<IDT>(gv);
     } else {
         const float kAlpha = 0.7978845608028654f;
         const float u = kAlpha * (gv + 0.044715f * gv * gv * gv);
-        const float th = 2.0f * (1.0f / (1.0f + expf(-2.0f * u))) - 1.0f;
+        const float th = 2.0f * sigmoid_f<IDT>(2.0f * u) - 1.0f;
         gv = 0.5f * gv * (1.0f + th);
     }
     gv = rnd<IDT>(gv);
@@ -174,6 +183,34 @@ __global__ void post_reorder_kernel(const void* __restrict__ down, void* __restr
                                     const void* __restrict__ topk_ids, int ids_bytes, const void* __restrict__ topk_w,
                                     int start_e, int end_e, int topk, int64_t hidden) {
     const int64_t t = blockIdx.x;
+    if constexpr (DT != LLMK_F32) {
+        // 16-bit rows of whole 16-byte chunks: 8 columns per lane and load
+        if (hidden % EPL == 0 && (((uintptr_t)down | (uintptr_t)out) & 15) == 0) {
+            for (int64_t c = (int64_t)threadIdx.x * EPL; c < hidden; c += (int64_t)blockDim.x * EPL) {
+                float sum[EPL] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                for (int j = 0; j < topk; ++j) {
+                    const int64_t e = ld_id(topk_ids, t * topk + j, ids_bytes);
+                    if (e < start_e || e > end_e) continue;
+                    const int64_t dst = src2dst[t * topk + j];
+                    const float w = rnd<DT>(FloatIO<WDT>::ld(topk_w, t * topk + j));
+                    float v[EPL];
+                    load8<DT>(down, dst * hidden + c, v);
+#pragma unroll
+                    for (int k = 0; k < EPL; ++k) sum[k] = rnd<DT>(sum[k] + rnd<DT>(v[k] * w));
+                }
+                uint4 o;
+                if constexpr (DT == LLMK_BF16) {
+                    o.x = pack_bf16x2(sum[0], sum[1]); o.y = pack_bf16x2(sum[2], sum[3]);
+                    o.z = pack_bf16x2(sum[4], sum[5]); o.w = pack_bf16x2(sum[6], sum[7]);
+                } else {
+                    o.x = pack_f16x2(sum[0], sum[1]); o.y = pack_f16x2(sum[2], sum[3]);
+                    o.z = pack_f16x2(sum[4], sum[5]); o.w = pack_f16x2(sum[6], sum[7]);
+                }
+                *(uint4*)((unsigned short*)out + t * hidden + c) = o;
+            }
+            return;
+        }
+    }
     for (int64_t c = threadIdx.x; c < hidden; c += blockDim.x) {
         float sum = 0.f;
         for (int j = 0; j < topk; ++j) {
