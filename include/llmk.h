@@ -178,6 +178,16 @@ int llmk_comm_dequant(const void* y, int kind, const void* s, int s_dtype, void*
 int llmk_moe_seg_indptr(const int64_t* sorted_ids, int64_t* seg_indptr, int64_t num_toks,
                         int num_experts, void* stream);
 int llmk_moe_src2dst(const int64_t* reorder_ids, int32_t* src2dst, int64_t num_toks, void* stream);
+/* ref: moe/group_gemm_kernel.py:48-78 (run_moe_ep_preproess) in one launch: stable sort of the num_toks
+ * flattened expert ids (int32 / int64 by ids_bytes; sorted_ids has the same type), src2dst[i] = position of
+ * id i in the sorted order, seg_indptr[e + 1] = number of ids <= e.  Every workgroup places 1024 ids and
+ * reads the whole id list to do so: the entry point is for the id counts of one forward pass and fails
+ * beyond the limits below;
+ * ids outside [0, num_experts) are ordered as one leading (negative) and one trailing group. */
+#define LLMK_MOE_PREPROCESS_MAX_EXPERTS 512
+#define LLMK_MOE_PREPROCESS_MAX_IDS 32768
+int llmk_moe_ep_preprocess(const void* topk_ids, int ids_bytes, int64_t num_toks, int num_experts,
+                           void* sorted_ids, int32_t* src2dst, int64_t* seg_indptr, void* stream);
 /* ids_bytes: 4 or 8 (topk_ids int32 / int64).  a1_scales may be NULL (fp32 per expert). */
 int llmk_moe_pre_reorder(const void* x, int x_dtype, void* out, int out_dtype, const int32_t* src2dst,
                          const void* topk_ids, int ids_bytes, const float* a1_scales,

@@ -52,6 +52,7 @@ SIGNATURES = {
     "llmk_comm_dequant": [_p, _i, _p, _i, _p, _i, _l, _i, _p],
     "llmk_moe_seg_indptr": [_p, _p, _l, _i, _p],
     "llmk_moe_src2dst": [_p, _p, _l, _p],
+    "llmk_moe_ep_preprocess": [_p, _i, _l, _i, _p, _p, _p, _p],
     "llmk_moe_pre_reorder": [_p, _i, _p, _i, _p, _p, _i, _p, _i, _i, _i, _l, _l, _p],
     "llmk_moe_act_and_mul": [_p, _i, _p, _i, _p, _i, _p, _i, _i, _l, _l, _i, _p],
     "llmk_moe_act_and_mul_quant": [_p, _i, _p, _p, _i, _i, _p, _i, _p, _i, _i, _l, _l, _i, _p],

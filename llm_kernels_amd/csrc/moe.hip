@@ -30,6 +30,112 @@ __device__ __forceinline__ int64_t ld_id(const void* p, int64_t i, int bytes) {
     return bytes == 8 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
 }
 
+// Stable counting sort of the flattened expert ids, with the segment pointers and the source -> destination
+// map as by-products: what torch.sort(stable) + seg_indptr_kernel + src2dst_kernel produce in eight launches.
+// Bucket 0 takes negative ids, bucket e + 1 expert e, bucket E + 1 ids >= E (both out-of-range buckets keep
+// their arrival order; a well-formed input leaves them empty).
+// Workgroup g places the ids [1024 g, 1024 g + 1024).  It counts, per bucket, all ids (-> bucket starts) and
+// the ids in front of its chunk, by reading the whole id list (at most PP_MAX_IDS ids, from L2); a lane's
+// position is then bucket start + ids of the bucket in earlier chunks + those in the lower waves of the
+// chunk + its rank among the equal ids of its own wave.  No workgroup waits for another.
+constexpr int PP_THREADS = 1024, PP_WAVES = PP_THREADS / 64, PP_MAX_EXPERTS = 512, PP_BUCKETS = PP_MAX_EXPERTS + 2;
+
+__global__ __launch_bounds__(PP_THREADS) void ep_preprocess_kernel(const void* __restrict__ ids, int ids_bytes, int n, int E,
+                                                                   void* __restrict__ sorted_out, int32_t* __restrict__ src2dst,
+                                                                   int64_t* __restrict__ seg_indptr) {
+    __shared__ int tot[PP_BUCKETS];      // ids per bucket, then the bucket's first position
+    __shared__ int pre[PP_BUCKETS];      // ids per bucket in front of this workgroup's chunk
+    __shared__ int wcount[PP_WAVES][PP_BUCKETS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nb = E + 2;
+    const int c0 = blockIdx.x * PP_THREADS;
+    auto bucket_at = [&](int i) {
+        if (i >= n) return -1;
+        const int64_t id = ld_id(ids, i, ids_bytes);
+        return id < 0 ? 0 : (id >= E ? E + 1 : (int)id + 1);
+    };
+    for (int b = tid; b < nb; b += PP_THREADS) { tot[b] = 0; pre[b] = 0; }
+    for (int i = tid; i < PP_WAVES * PP_BUCKETS; i += PP_THREADS) (&wcount[0][0])[i] = 0;
+    __syncthreads();
+    constexpr int U = 4;                 // rounds whose loads are in flight together
+    if (nb <= 64) {
+        // few buckets: lane k of every wave counts bucket k from ballots (one LDS atomic per id would
+        // serialise on the few addresses)
+        int acc_t = 0, acc_p = 0;
+        for (int r0 = 0; r0 < n; r0 += U * PP_THREADS) {
+            int b[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) b[u] = bucket_at(r0 + u * PP_THREADS + tid);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool before = r0 + u * PP_THREADS < c0;        // whole rounds lie in front of the chunk or not
+                for (int k = 0; k < nb; ++k) {
+                    const int c = __popcll(__ballot(b[u] == k));
+                    if (lane == k) { acc_t += c; if (before) acc_p += c; }
+                }
+            }
+        }
+        if (lane < nb) { atomicAdd(&tot[lane], acc_t); atomicAdd(&pre[lane], acc_p); }
+    } else {
+        for (int r0 = 0; r0 < n; r0 += U * PP_THREADS) {
+            int b[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) b[u] = bucket_at(r0 + u * PP_THREADS + tid);
+#pragma unroll
+            for (int u = 0; u < U; ++u) if (b[u] >= 0) {
+                atomicAdd(&tot[b[u]], 1);
+                if (r0 + u * PP_THREADS < c0) atomicAdd(&pre[b[u]], 1);
+            }
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // exclusive scan of the bucket counts: a run of buckets per lane, then a scan over the lanes
+        const int per = (nb + 63) / 64, b0 = lane * per;
+        int sum = 0;
+        for (int k = 0; k < per; ++k) if (b0 + k < nb) sum += tot[b0 + k];
+        int incl = sum;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int t = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += t;
+        }
+        int run = incl - sum;
+        for (int k = 0; k < per; ++k) if (b0 + k < nb) {
+            const int c = tot[b0 + k];
+            tot[b0 + k] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    // seg_indptr[e + 1] = number of ids <= e = start of bucket e + 2; seg_indptr[0] = 0
+    if (blockIdx.x == 0)
+        for (int e = tid; e <= E; e += PP_THREADS) seg_indptr[e] = e == 0 ? 0 : (int64_t)tot[e + 1];
+
+    // rank of a lane among the lanes of its wave with the same bucket, one leader per bucket publishes the count
+    const int i = c0 + tid;
+    const int b = bucket_at(i);
+    int rank = 0;
+    uint64_t todo = __ballot(b >= 0);
+    while (todo) {                                       // one pass per distinct bucket of the wave
+        const int l = __ffsll((unsigned long long)todo) - 1;
+        const int v = __builtin_amdgcn_readlane(b, l);
+        const uint64_t m = __ballot(b == v);
+        if (b == v) {
+            rank = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == l) wcount[wave][b] = __popcll(m);
+        }
+        todo &= ~m;
+    }
+    __syncthreads();
+    if (b >= 0) {
+        int pos = tot[b] + pre[b] + rank;
+        for (int w = 0; w < wave; ++w) pos += wcount[w][b];
+        const int64_t id = (b >= 1 && b <= E) ? (int64_t)(b - 1) : ld_id(ids, i, ids_bytes);
+        if (ids_bytes == 8) ((int64_t*)sorted_out)[pos] = id; else ((int32_t*)sorted_out)[pos] = (int32_t)id;
+        src2dst[i] = pos;
+    }
+}
+
 // one workgroup per token: copy (x * 1/a1_scale[e]) into each destination row of its local experts
 template <int IDT, int ODT>
 __global__ void pre_reorder_kernel(const void* __restrict__ x, void* __restrict__ out, const int32_t* __restrict__ src2dst,
@@ -243,6 +349,21 @@ extern "C" int llmk_moe_src2dst(const int64_t* reorder_ids, int32_t* src2dst, in
     if (!reorder_ids || !src2dst) LLMK_FAIL(LLMK_ERR_ARG, "moe_src2dst: null pointer");
     src2dst_kernel<<<(unsigned)cdiv64(num_toks, 256), 256, 0, (hipStream_t)stream>>>(reorder_ids, src2dst, num_toks);
     LLMK_CHECK_LAUNCH("moe_src2dst");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_moe_ep_preprocess(const void* topk_ids, int ids_bytes, int64_t num_toks, int num_experts,
+                                      void* sorted_ids, int32_t* src2dst, int64_t* seg_indptr, void* stream) {
+    if (num_experts < 0 || num_toks < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_ep_preprocess: negative size");
+    if (num_experts > LLMK_MOE_PREPROCESS_MAX_EXPERTS || num_toks > LLMK_MOE_PREPROCESS_MAX_IDS)
+        LLMK_FAIL(LLMK_ERR_SHAPE, "moe_ep_preprocess: %lld ids of %d experts exceed the limits %d / %d of the one-workgroup sort",
+                  (long long)num_toks, num_experts, LLMK_MOE_PREPROCESS_MAX_IDS, LLMK_MOE_PREPROCESS_MAX_EXPERTS);
+    if (ids_bytes != 4 && ids_bytes != 8) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_ep_preprocess: ids_bytes %d", ids_bytes);
+    if (!seg_indptr || (num_toks && (!topk_ids || !sorted_ids || !src2dst))) LLMK_FAIL(LLMK_ERR_ARG, "moe_ep_preprocess: null pointer");
+    static_assert(LLMK_MOE_PREPROCESS_MAX_EXPERTS == PP_MAX_EXPERTS, "header limit and kernel table size differ");
+    const unsigned grid = (unsigned)(num_toks > 0 ? cdiv64(num_toks, PP_THREADS) : 1);
+    ep_preprocess_kernel<<<grid, PP_THREADS, 0, (hipStream_t)stream>>>(topk_ids, ids_bytes, (int)num_toks, num_experts, sorted_ids, src2dst, seg_indptr);
+    LLMK_CHECK_LAUNCH("moe_ep_preprocess");
     return LLMK_OK;
 }
 

@@ -17,14 +17,28 @@ def _cdiv(a, b):
     return (a + b - 1) // b
 
 
+# limits of the one-workgroup sort behind llmk_moe_ep_preprocess (LLMK_MOE_PREPROCESS_MAX_* of the C header)
+PREPROCESS_MAX_IDS = 32768
+PREPROCESS_MAX_EXPERTS = 512
+
+
 def run_moe_ep_preproess(topk_ids: torch.Tensor, num_experts: int):
     """Stable sort of the flattened expert ids -> (sorted ids, src2dst int32 [T*topk], seg_indptr int64 [E+1])."""
     _lib.require_gpu(topk_ids)
-    reorder_topk_ids, reorder_ids = torch.sort(topk_ids.view(-1), stable=True)
     n = topk_ids.numel()
+    st = _lib.stream(topk_ids)
+    if (n <= PREPROCESS_MAX_IDS and num_experts <= PREPROCESS_MAX_EXPERTS and topk_ids.is_contiguous()
+            and topk_ids.dtype in (torch.int32, torch.int64)):
+        # the id counts of one forward pass: one launch instead of the eight of sort + pointers + map
+        reorder_topk_ids = torch.empty(n, device=topk_ids.device, dtype=topk_ids.dtype)
+        seg_indptr = torch.empty(num_experts + 1, device=topk_ids.device, dtype=torch.int64)
+        src2dst = torch.empty(n, device=topk_ids.device, dtype=torch.int32)
+        _lib.call("llmk_moe_ep_preprocess", _lib.ptr(topk_ids), _ids_bytes(topk_ids), n, int(num_experts),
+                  _lib.ptr(reorder_topk_ids), _lib.ptr(src2dst), _lib.ptr(seg_indptr), st)
+        return reorder_topk_ids, src2dst, seg_indptr
+    reorder_topk_ids, reorder_ids = torch.sort(topk_ids.view(-1), stable=True)
     seg_indptr = torch.zeros(num_experts + 1, device=topk_ids.device, dtype=torch.int64)
     src2dst = torch.empty(n, device=topk_ids.device, dtype=torch.int32)
-    st = _lib.stream(topk_ids)
     sorted64 = reorder_topk_ids if reorder_topk_ids.dtype == torch.int64 else reorder_topk_ids.to(torch.int64)
     _lib.call("llmk_moe_seg_indptr", _lib.ptr(sorted64), _lib.ptr(seg_indptr), n, num_experts, st)
     _lib.call("llmk_moe_src2dst", _lib.ptr(reorder_ids), _lib.ptr(src2dst), n, st)

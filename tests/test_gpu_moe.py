@@ -33,6 +33,45 @@ def test_preprocess_random_incl_empty_experts(dev, T, E, topk):
     assert seg[-1].item() == T * topk and seg[E].item() == seg[E - 1].item()
 
 
+@pytest.mark.parametrize("n,E,dtype", [(8192, 8, torch.int64), (32768, 512, torch.int32), (1025, 256, torch.int64),
+                                       (1023, 3, torch.int32), (64, 160, torch.int64), (5000, 1, torch.int64),
+                                       (0, 8, torch.int64)])
+def test_preprocess_one_launch_equals_sort(dev, n, E, dtype):
+    """The one-workgroup counting sort returns what the stable sort + segment pointers + map return: many
+    rounds, every wave holding many distinct ids (E = 512), a single bucket, ragged last round, no ids."""
+    announce("moe preprocess one launch", n, E, dtype)
+    torch.manual_seed(n + E)
+    ids = torch.randint(0, E, (n,), dtype=dtype)
+    if n > 100:
+        ids[n // 3: n // 3 + 70] = E - 1                        # a run longer than a wave of one id
+    rids, s2d, seg = gk.run_moe_ep_preproess(ids.to(dev), E)
+    orids, order = torch.sort(ids, stable=True)
+    os2d = torch.empty(n, dtype=torch.int32)
+    os2d[order] = torch.arange(n, dtype=torch.int32)
+    oseg = torch.zeros(E + 1, dtype=torch.int64)
+    oseg[1:] = torch.cumsum(torch.bincount(ids.long(), minlength=E), 0)
+    assert rids.dtype == dtype and torch.equal(rids.cpu(), orids)
+    assert torch.equal(s2d.cpu(), os2d) and torch.equal(seg.cpu(), oseg)
+
+
+def test_preprocess_beyond_one_workgroup(dev):
+    """More ids than the one-launch sort takes: the wrapper goes through torch.sort, the entry point refuses."""
+    announce("moe preprocess large")
+    from llm_kernels_amd import _lib
+    n, E = gk.PREPROCESS_MAX_IDS + 5, 8
+    torch.manual_seed(3)
+    ids = torch.randint(0, E, (n,))
+    rids, s2d, seg = gk.run_moe_ep_preproess(ids.to(dev), E)
+    orids, os2d, oseg = m.run_moe_ep_preprocess(ids, E)
+    assert torch.equal(rids.cpu(), orids) and torch.equal(s2d.cpu(), os2d) and torch.equal(seg.cpu(), oseg)
+    d = ids.to(dev)
+    with pytest.raises(RuntimeError, match="exceed the limits"):
+        _lib.call("llmk_moe_ep_preprocess", _lib.ptr(d), 8, n, E, _lib.ptr(rids), _lib.ptr(s2d), _lib.ptr(seg), None)
+    with pytest.raises(RuntimeError, match="exceed the limits"):
+        _lib.call("llmk_moe_ep_preprocess", _lib.ptr(d), 8, 16, gk.PREPROCESS_MAX_EXPERTS + 1, _lib.ptr(rids),
+                  _lib.ptr(s2d), _lib.ptr(seg), None)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_reorder_and_activation_kernels(dev, dtype):
     announce("moe aux", dtype)
