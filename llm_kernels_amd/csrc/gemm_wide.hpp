@@ -65,21 +65,43 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
             by = strip * H + rr % H;
         }
     }
-    const int n0 = bx * W_BN;
-
     int m_start, m_end;
     const uint8_t* bbase = p.b;
     int64_t bs_off = 0;
     if constexpr (GROUPED) {
-        int tile = blockIdx.y, e = 0, cum = 0;
+        int e = 0;
         int64_t s0 = p.seg_indptr[0];
         bool found = false;
-        for (; e < p.E; ++e) {
-            const int64_t s1 = p.seg_indptr[e + 1];
-            const int t = (int)((s1 - s0 + W_BM - 1) / W_BM);
-            if (tile < cum + t) { found = true; m_start = (int)s0 + (tile - cum) * W_BM; m_end = min((int)s1, m_start + W_BM); break; }
-            cum += t;
-            s0 = s1;
+        const int gx = gridDim.x;
+        if (gx % 8 == 0) {
+            // XCD x (workgroup id mod 8) owns the column tiles x, x + 8, ...; it walks them segment by
+            // segment, and for every column tile all row tiles of the segment back to back, so the workgroups
+            // that share a weight tile run at the same time on the L2 that holds it.
+            const int lin = blockIdx.y * gx + blockIdx.x, x = lin & 7, cx = gx >> 3;
+            int s = lin >> 3;
+            for (; e < p.E; ++e) {
+                const int64_t s1 = p.seg_indptr[e + 1];
+                const int t = (int)((s1 - s0 + W_BM - 1) / W_BM);
+                if (s < t * cx) {
+                    const int bl = s / t, rt = s - bl * t;
+                    found = true;
+                    bx = bl * 8 + x;
+                    m_start = (int)s0 + rt * W_BM;
+                    m_end = min((int)s1, m_start + W_BM);
+                    break;
+                }
+                s -= t * cx;
+                s0 = s1;
+            }
+        } else {
+            int tile = blockIdx.y, cum = 0;
+            for (; e < p.E; ++e) {
+                const int64_t s1 = p.seg_indptr[e + 1];
+                const int t = (int)((s1 - s0 + W_BM - 1) / W_BM);
+                if (tile < cum + t) { found = true; m_start = (int)s0 + (tile - cum) * W_BM; m_end = min((int)s1, m_start + W_BM); break; }
+                cum += t;
+                s0 = s1;
+            }
         }
         if (!found) return;
         const int64_t widx = p.weight_indices ? p.weight_indices[e] : e;
@@ -89,6 +111,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         m_start = by * W_BM;
         m_end = min(p.M, m_start + W_BM);
     }
+    const int n0 = bx * W_BN;
 
     // weight scales of the tile's two 128-column blocks, for every K step
     float* bsl = (float*)(lds + 2 * W_STAGE);
