@@ -159,6 +159,40 @@ def test_grouped_gemm(dev, kind, T, E, N, K):
     assert_close_scaled(c, ref, what="grouped " + kind)
 
 
+@pytest.mark.parametrize("M,N,K", [(8192, 2048, 256), (8192, 2304, 384), (8192, 3840, 256), (4096, 2048, 384)])
+def test_grouped_gemm_large_tiles_exact(dev, M, N, K):
+    """Shapes that the dispatch gives to the 256- and 128-row tiles of the large grouped kernel, with a number
+    of column tiles that is and is not a multiple of the XCD count (the tile order differs), segments of very
+    different length (one empty, one shorter than a tile, ragged ends) and permuted weight indices.  int8 with
+    unit scales and small integers: every output must be the exact integer product; rows behind the last
+    segment keep their fill value."""
+    announce("grouped large tiles", M, N, K)
+    E = 4
+    torch.manual_seed(M + N)
+    used = M - 7                                                # the last 7 rows belong to no segment
+    seg = torch.tensor([0, 3000 if M > 4096 else 1300, 3000 if M > 4096 else 1300, 3041 if M > 4096 else 1341, used])
+    widx = torch.tensor([2, 0, 3, 1])
+    a = torch.randint(-15, 16, (M, K), dtype=torch.int8)
+    b = torch.randint(-15, 16, (E, N, K), dtype=torch.int8)
+    a_s = torch.ones(M, K // 128, dtype=torch.float32)
+    b_s = torch.ones(E, (N + 127) // 128, K // 128, dtype=torch.float32)
+    c = torch.full((M, N), 5.0, dtype=torch.float32, device=dev)
+    _lib_call_grouped_i8(dev, a, a_s, b, b_s, c, seg, widx)
+    out = c.cpu()
+    for e in range(E):
+        lo, hi = int(seg[e]), int(seg[e + 1])
+        ref = a[lo:hi].double() @ b[widx[e]].double().T
+        assert torch.equal(out[lo:hi].double(), ref), "segment %d" % e
+    assert torch.all(out[used:] == 5.0)
+
+
+def _lib_call_grouped_i8(dev, a, a_s, b, b_s, c, seg, widx):
+    """grouped_gemm_triton on activations that are already int8 with their 1 x 128 scales."""
+    d = [t.to(dev).contiguous() for t in (a, a_s, b, b_s, seg.long(), widx.long())]
+    gk.grouped_gemm_triton(d[0], d[2], c, b.shape[0], True, d[4], d[5], False, d[1], d[3], [128, 128])
+    torch.cuda.synchronize()
+
+
 def test_grouped_gemm_single_expert_equals_dense_and_weight_indices(dev):
     announce("grouped single expert")
     torch.manual_seed(4)
