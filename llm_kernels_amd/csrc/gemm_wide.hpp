@@ -381,7 +381,10 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     constexpr bool HAS_WIDE = KIND != K_W4NK && KIND != K_W4MARLIN;             // the 4-bit expansion exists in the 128-column kernels only
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
-    auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * ((rows + bm - 1) / bm) + 255) / 256; };
+    // a segment of a grouped GEMM rarely ends on a tile boundary: count one ragged tile per segment on top of
+    // the full ones (with the plain ceiling, segments of 128 +- a few rows looked like one 128-row tile each and
+    // went to a tile shape that needed two; -8 % on the Mixtral forward at 256 and 512 tokens)
+    auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * (GROUPED ? rows / bm + 1 : (rows + bm - 1) / bm) + 255) / 256; };
     const double t_wide = 60.0 * rounds(256, 256), t4 = 43.0 * rounds(256, 128), t2 = 26.0 * rounds(128, 128),
                  t1 = 16.0 * rounds(64, 128);
     if constexpr (HAS_WIDE) {
