@@ -390,7 +390,10 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     if constexpr (HAS_WIDE) {
         if (t_wide <= t4 && t_wide <= t2 && t_wide <= t1) {
             // problems whose 256 x 256 tiles do not fill a round: the 128 x 256 tile of the same kernel
-            if (36.0 * rounds(128, 256) < t_wide) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
+            // (a tie goes to the 128-row tile for block-scaled int8, whose per-step conversions leave the tall
+            // tile less of its advantage: grouped Mixtral down projection -3 %; +1 % for fp8)
+            const double t_half = 36.0 * rounds(128, 256);
+            if (t_half < t_wide || (KIND == K_I8_BLOCK && GROUPED && t_half == t_wide)) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
             return launch_wide<KIND, GROUPED>(p, stream, name);
         }
         const double t_half = 36.0 * rounds(128, 256);
