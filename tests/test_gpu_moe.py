@@ -54,6 +54,32 @@ def test_preprocess_one_launch_equals_sort(dev, n, E, dtype):
     assert torch.equal(s2d.cpu(), os2d) and torch.equal(seg.cpu(), oseg)
 
 
+def test_preprocess_ids_outside_the_expert_range(dev):
+    """Ids below 0 or at / above num_experts (padding conventions of some routers): the launch must stay inside
+    its tables and still return a permutation whose in-range part is the stable sort; negative ids lead,
+    too-large ids trail, and seg_indptr[e + 1] counts the ids <= e as the reference's binary search does."""
+    announce("moe preprocess out-of-range ids")
+    n, E = 3000, 8
+    torch.manual_seed(9)
+    ids = torch.randint(0, E, (n,))
+    ids[::17] = -1
+    ids[5::29] = E + 3
+    ids[7::31] = E
+    rids, s2d, seg = gk.run_moe_ep_preproess(ids.to(dev), E)
+    rids, s2d, seg = rids.cpu(), s2d.cpu().long(), seg.cpu()
+    assert sorted(s2d.tolist()) == list(range(n))                   # a permutation
+    assert torch.equal(rids[s2d], ids)                               # every id sits where src2dst says
+    neg, big = int((ids < 0).sum()), int((ids >= E).sum())
+    assert (rids[:neg] < 0).all() and (rids[n - big:] >= E).all()
+    mid = rids[neg:n - big]
+    assert torch.equal(mid, torch.sort(ids[(ids >= 0) & (ids < E)], stable=True)[0])
+    inr = torch.nonzero((ids >= 0) & (ids < E)).flatten()            # stable: equal ids keep their order
+    for e in range(E):
+        pos = s2d[inr[ids[inr] == e]]
+        assert (pos[1:] > pos[:-1]).all()
+    assert seg.tolist() == [0] + [int((ids <= e).sum()) for e in range(E)]
+
+
 def test_preprocess_beyond_one_workgroup(dev):
     """More ids than the one-launch sort takes: the wrapper goes through torch.sort, the entry point refuses."""
     announce("moe preprocess large")
