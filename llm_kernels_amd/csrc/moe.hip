@@ -54,7 +54,7 @@ __global__ __launch_bounds__(PP_THREADS) void ep_preprocess_kernel(const void* _
         return id < 0 ? 0 : (id >= E ? E + 1 : (int)id + 1);
     };
     for (int b = tid; b < nb; b += PP_THREADS) { tot[b] = 0; pre[b] = 0; }
-    for (int i = tid; i < PP_WAVES * PP_BUCKETS; i += PP_THREADS) (&wcount[0][0])[i] = 0;
+    for (int i = tid; i < PP_WAVES * nb; i += PP_THREADS) wcount[i / nb][i % nb] = 0;
     __syncthreads();
     constexpr int U = 4;                 // rounds whose loads are in flight together
     if (nb <= 64) {

@@ -20,6 +20,19 @@ def softmax_topk_router(router_logits: torch.Tensor, top_k: int = 2, renormalize
     return ids, w
 
 
+_widx_cache = {}
+
+
+def _weight_indices(E, dev):
+    """arange(E) on the device (reference sglang_moe_all_gather_all_reduce.py:327), built once per (E, device):
+    the grouped GEMM only reads it, and a launch per forward is 5 us of a decode-sized forward."""
+    key = (E, dev.type, dev.index)
+    t = _widx_cache.get(key)
+    if t is None:
+        t = _widx_cache[key] = torch.arange(0, E, device=dev, dtype=torch.int64)
+    return t
+
+
 def ep_moe_forward(hidden_states: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor,
                    w13_weight: torch.Tensor, w2_weight: torch.Tensor,
                    w13_weight_scale: Optional[torch.Tensor] = None, w2_weight_scale: Optional[torch.Tensor] = None,
@@ -42,7 +55,7 @@ def ep_moe_forward(hidden_states: torch.Tensor, topk_ids: torch.Tensor, topk_wei
 
     reorder_topk_ids, src2dst, seg_indptr = run_moe_ep_preproess(topk_ids, num_experts)
     seg_cur = seg_indptr[start_expert_id:end_expert_id + 2]
-    widx = torch.arange(0, E, device=dev, dtype=torch.int64)
+    widx = _weight_indices(E, dev)
     quantised = block_shape is not None and w13_weight.dtype in (torch.int8, torch.float8_e4m3fn)
     fused = bool(fuse_quant and quantised and H % 128 == 0 and (w13_weight.shape[1] // 2) % 128 == 0
                  and dt in (torch.float16, torch.bfloat16))
