@@ -7,7 +7,10 @@ converter returns the values in natural order, like the reference's `uint4_to_fp
 """
 import torch
 
-from .. import _lib
+try:
+    from .. import _lib
+except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
+    import _lib
 
 
 def pack_uint4(values: torch.Tensor) -> torch.Tensor:

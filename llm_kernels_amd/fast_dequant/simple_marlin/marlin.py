@@ -2,7 +2,10 @@
 marlin_w4a16_gemm.cpp:23-111).  Same argument list and error behaviour (RuntimeError)."""
 import torch
 
-from ... import _lib
+try:
+    from ... import _lib
+except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
+    import _lib
 
 
 def mul(A, B, C, s, workspace, thread_k=-1, thread_n=-1, sms=-1, max_par=16):

@@ -6,8 +6,12 @@ k = 8*word + i).  The simple-Marlin layout has its own entry point (simple_marli
 """
 import torch
 
-from .. import _lib
-from ..quantization.bitpack import pack_weights_over_cols
+try:
+    from .. import _lib
+    from ..quantization.bitpack import pack_weights_over_cols
+except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
+    import _lib
+    from quantization.bitpack import pack_weights_over_cols
 
 
 def quantize_nk(w: torch.Tensor, group_size: int = 128):

@@ -10,7 +10,12 @@ from typing import List, Optional
 
 import torch
 
-from .. import _lib
+try:
+    from .. import _lib
+    from ..quantization import fp8_kernel as _fp8_kernel, int8_kernel as _int8_kernel
+except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
+    import _lib
+    from quantization import fp8_kernel as _fp8_kernel, int8_kernel as _int8_kernel
 
 
 def _cdiv(a, b):
@@ -209,10 +214,7 @@ def grouped_gemm_triton(
             assert scale_a is not None, 'quantised activations need scale_a'
             scale_a = scale_a.contiguous()
         else:
-            if b.dtype == torch.int8:
-                from ..quantization.int8_kernel import act_quant as per_token_group_quant
-            else:
-                from ..quantization.fp8_kernel import act_quant as per_token_group_quant
+            per_token_group_quant = (_int8_kernel if b.dtype == torch.int8 else _fp8_kernel).act_quant
             a, scale_a = per_token_group_quant(a.contiguous(), block_k)
         assert _cdiv(a.shape[-1], block_k) == scale_a.shape[-1]
         assert _cdiv(b.shape[-2], block_n) == scale_b.shape[-2]

@@ -10,7 +10,10 @@ from typing import Tuple
 
 import torch
 
-from .. import _lib
+try:
+    from .. import _lib
+except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
+    import _lib
 
 
 def int8_quant(x: torch.Tensor, block_size: int = 32) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -7,7 +7,10 @@ HIP-backed functions so that existing call sites keep working.
 """
 import torch
 
-from .. import _lib
+try:
+    from .. import _lib
+except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
+    import _lib
 
 _PACK_DTYPE = {8: torch.uint8, 16: torch.int16, 32: torch.int32, 64: torch.int64}
 _OUT_BYTES = {torch.uint8: 1, torch.int8: 1, torch.int16: 2, torch.int32: 4, torch.int64: 8}

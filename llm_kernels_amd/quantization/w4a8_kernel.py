@@ -9,7 +9,10 @@ from typing import Tuple
 
 import torch
 
-from .. import _lib
+try:
+    from .. import _lib
+except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
+    import _lib
 from .bitpack import pack_weights_over_rows
 
 PACKING_BITS = 32

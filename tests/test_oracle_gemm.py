@@ -120,3 +120,53 @@ def test_silu_rounding_points_bf16():
     g32 = gu[:, :2].float()
     exp = ((g32 * torch.sigmoid(g32)).bfloat16() * gu[:, 2:])
     assert torch.equal(out, exp)
+
+
+def test_gelu_branch_equals_torch_tanh_gelu():
+    """moe_ref.silu_and_mul(act='gelu') restates group_gemm_kernel.py:214-228; in fp32 (no rounding points)
+    it must be torch's tanh-approximated GELU times up."""
+    torch.manual_seed(8)
+    g32 = torch.cat([torch.randn(7, 64) * 3, torch.tensor([[0.0, 1.0, -1.0, 10.0, -10.0, 0.5, -0.5, 25.0] * 8])])
+    up = torch.randn(8, 64)
+    out, mask = m.silu_and_mul(torch.cat([g32, up], 1), torch.zeros(8, dtype=torch.long), None, 0, 0, act="gelu")
+    assert mask.all()
+    want = torch.nn.functional.gelu(g32.double(), approximate="tanh") * up.double()
+    assert torch.allclose(out.double(), want, rtol=2e-6, atol=2e-7)
+    # known values: gelu(0) = 0, gelu(x) -> x for large x, -> 0 for very negative x
+    one = torch.ones(1, 3)
+    o2, _ = m.silu_and_mul(torch.cat([torch.tensor([[0.0, 25.0, -25.0]]), one], 1), torch.tensor([0]), None, 0, 0,
+                           act="gelu")
+    assert o2.tolist() == [[0.0, 25.0, 0.0]] or o2.abs().tolist() == [[0.0, 25.0, 0.0]]
+
+
+def test_pre_reorder_scale_branch_hand_rows():
+    """group_gemm_kernel.py:100-115: row * (1 / a1_scales[e - start]) for local experts only."""
+    x = torch.tensor([[2.0, 4.0, -8.0, 1.0], [3.0, 6.0, 9.0, -12.0]])
+    topk_ids = torch.tensor([[1, 2], [3, 1]])            # experts 1..2 are local, 3 is not
+    src2dst = torch.tensor([0, 2, 3, 1], dtype=torch.int32)
+    a1 = torch.tensor([2.0, 4.0])                        # scales of experts 1 and 2
+    out = m.pre_reorder(x, src2dst, topk_ids, a1, 1, 2, 2)
+    assert out[0].tolist() == [1.0, 2.0, -4.0, 0.5]      # token 0 -> expert 1: / 2
+    assert out[2].tolist() == [0.5, 1.0, -2.0, 0.25]     # token 0 -> expert 2: / 4
+    assert out[1].tolist() == [1.5, 3.0, 4.5, -6.0]      # token 1 -> expert 1: / 2
+    assert out[3].tolist() == [0.0, 0.0, 0.0, 0.0]       # token 1 -> expert 3: not local, row untouched
+    # rounding point: the product is formed in fp32 and cast once to the output dtype
+    xb = torch.tensor([[1.0078125, 3.0]]).bfloat16()
+    ob = m.pre_reorder(xb, torch.tensor([0], dtype=torch.int32), torch.tensor([[0]]), torch.tensor([3.0]), 0, 0, 1)
+    assert torch.equal(ob, (xb.float() * (1.0 / 3.0)).bfloat16())
+
+
+def test_silu_and_mul_scale_branch_hand_rows():
+    """group_gemm_kernel.py:145-166: (1 / scale[e - start]) is cast to the tensor dtype first, then
+    silu(gate) (cast) * up (rounded) * scale (rounded)."""
+    # silu(20) = 20 in fp32 to 8 digits; up = 3; expert 2 -> 1/4, expert 1 -> 1/2
+    gu = torch.tensor([[20.0, 3.0], [20.0, 3.0], [20.0, 3.0]]).bfloat16()
+    rids = torch.tensor([1, 2, 3])
+    out, mask = m.silu_and_mul(gu, rids, torch.tensor([2.0, 4.0]), 1, 2)
+    assert mask.tolist() == [True, True, False]
+    assert out.flatten().tolist() == [30.0, 15.0, 0.0]
+    # 1/3 is rounded to bf16 before the multiplication (not applied as an fp32 factor)
+    gu2 = torch.tensor([[20.0, 1.0]]).bfloat16()
+    o2, _ = m.silu_and_mul(gu2, torch.tensor([0]), torch.tensor([3.0]), 0, 0)
+    third = torch.tensor(1.0 / 3.0).bfloat16()
+    assert o2.item() == (torch.tensor(20.0).bfloat16() * third).item() != torch.tensor(20.0 / 3.0).bfloat16().item()

@@ -134,3 +134,90 @@ def test_rowwise():
     x = torch.randn(9, 384)
     y, s = q.int8_quant_rowwise(x)
     assert (y.abs().amax(1) == 127).all() and s.dtype == torch.float32
+
+
+# ----------------------------------------------------------------- fp8 128x128 weight quantizer
+def _e4m3_table():
+    """Every finite e4m3fn value from the bit layout (1 sign, 4 exponent bits with bias 7, 3 mantissa bits;
+    exponent 15 with mantissa 7 is NaN), without going through torch's fp8 type."""
+    vals = {}
+    for code in range(256):
+        sgn = -1.0 if code & 0x80 else 1.0
+        e, mnt = (code >> 3) & 0xF, code & 7
+        if e == 15 and mnt == 7:
+            continue
+        v = mnt * 2.0 ** -9 if e == 0 else (1 + mnt / 8.0) * 2.0 ** (e - 7)
+        vals[code] = sgn * v
+    return vals
+
+
+def _e4m3_rne(v, table):
+    """Nearest table value, ties to the even mantissa (brute force over the 254 finite codes)."""
+    best = None
+    for code, t in table.items():
+        d = abs(t - v)
+        if best is None or d < best[0] or (d == best[0] and (code & 1) == 0 and (best[1] & 1) == 1):
+            best = (d, code)
+    return best[1]
+
+
+def test_e4m3_cast_is_rne_onto_the_bit_layout_table():
+    """Pins the cast that act_quant_fp8 / weight_quant_fp8 rely on: torch's CPU fp32 -> e4m3fn conversion
+    equals round-to-nearest-even onto the value table derived from the bit layout (ties included)."""
+    table = _e4m3_table()
+    assert len(table) == 254 and table[0x7E] == 448.0 and table[0x38] == 1.0 and table[0xC0] == -2.0
+    torch.manual_seed(11)
+    v = torch.cat([torch.randn(300) * 100, torch.randn(100) * 0.01,
+                   torch.tensor([0.0, 17.0, 19.0, 0.0029296875, 432.0, 448.0, -448.0, 1.0625, 1.1875])])
+    v = v.clamp(-448, 448)
+    got = v.to(torch.float8_e4m3fn).view(torch.uint8).tolist()
+    for x, c in zip(v.tolist(), got):
+        want = _e4m3_rne(x, table)
+        if x == 0.0:
+            assert c in (0x00, 0x80)
+        else:
+            assert table[c] == table[want], (x, c, want)
+    # 17 lies midway between 16 (mantissa 0) and 18 (mantissa 1): ties go to the even mantissa
+    assert torch.tensor([17.0, 19.0]).to(torch.float8_e4m3fn).float().tolist() == [16.0, 20.0]
+
+
+def test_weight_quant_fp8_hand_block():
+    # one block whose absmax is 448 -> s = 1 exactly and the codes are the plain e4m3 encodings
+    w = torch.zeros(128, 128)
+    w[0, 0], w[0, 1], w[0, 2], w[5, 7], w[127, 127] = 448.0, 1.0, -2.0, 17.0, 0.0009765625
+    y, s = q.weight_quant_fp8(w)
+    assert s.shape == (1, 1) and s.dtype == torch.float32 and s.item() == 1.0
+    yb = y.view(torch.uint8)
+    assert [yb[0, 0].item(), yb[0, 1].item(), yb[0, 2].item()] == [0x7E, 0x38, 0xC0]
+    assert y.float()[5, 7].item() == 16.0              # tie -> even mantissa
+    assert yb[127, 127].item() == 0x00                 # 2^-10 is half the smallest subnormal: tie -> 0
+    assert int((yb != 0).sum()) == 4
+    # absmax 224 -> s = 0.5, the same codes for inputs scaled by 0.5
+    y2, s2 = q.weight_quant_fp8(w * 0.5)
+    assert s2.item() == 0.5 and torch.equal(y2.view(torch.uint8), yb)
+
+
+def test_weight_quant_fp8_blocks_ragged_by_brute_force():
+    """200 x 300 (ragged in both directions): block membership, scale and codes of every block against an
+    independent slice-by-slice evaluation; every block's absmax element maps to +-448."""
+    torch.manual_seed(12)
+    w = torch.randn(200, 300) * 0.02
+    y, s = q.weight_quant_fp8(w, 128)
+    assert y.shape == w.shape and y.dtype == torch.float8_e4m3fn and s.shape == (2, 3) and s.dtype == torch.float32
+    table = _e4m3_table()
+    yb = y.view(torch.uint8)
+    for bi in range(2):
+        for bj in range(3):
+            r0, r1, c0, c1 = bi * 128, min(200, bi * 128 + 128), bj * 128, min(300, bj * 128 + 128)
+            blk = w[r0:r1, c0:c1]
+            sc = blk.abs().max() / 448.0                       # fp32
+            assert s[bi, bj] == sc
+            assert torch.equal(yb[r0:r1, c0:c1], (blk / sc).to(torch.float8_e4m3fn).view(torch.uint8))
+            assert y[r0:r1, c0:c1].float().abs().max() == 448.0
+            # a few elements of the block through the brute-force encoder
+            for (i, j) in [(0, 0), (r1 - r0 - 1, c1 - c0 - 1), ((r1 - r0) // 2, (c1 - c0) // 3)]:
+                v = (blk[i, j] / sc).item()
+                assert table[yb[r0 + i, c0 + j].item()] == table[_e4m3_rne(v, table)]
+    d = q.weight_dequant_block(y, s, 128)
+    assert ((d - w).abs() <= torch.maximum(w.abs() * 2 ** -4, s.repeat_interleave(128, 0)[:200]
+                                           .repeat_interleave(128, 1)[:, :300] * 2 ** -10) * 1.001).all()
