@@ -105,6 +105,16 @@ int llmk_weight_dequant_w4a8(const int32_t* packed, const void* s_f16, const int
 int llmk_gemm_fp8_block(const void* a_e4m3, const float* a_s, const void* b_e4m3, const float* b_s,
                         void* c, int c_dtype, int64_t M, int64_t N, int64_t K,
                         void* workspace, int64_t workspace_bytes, void* stream);
+/* llmk_gemm_fp8_block for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and
+ * results (bit for bit) as llmk_gemm_fp8_block called with a workspace of llmk_gemm_workspace_bytes(M, N, K)
+ * bytes, but the scratch is a device array built into the library (LLMK_STATIC_SCRATCH_BYTES per GPU, held
+ * until the process ends); the call itself allocates and frees nothing.  Shapes whose scratch exceeds the
+ * array fail with LLMK_ERR_SHAPE.  All calls on one GPU share the array: calls that may overlap on
+ * different streams of that GPU race, issue them on one stream. */
+#define LLMK_STATIC_SCRATCH_BYTES (32 << 20)
+int llmk_gemm_fp8_block_static(const void* a_e4m3, const float* a_s, const void* b_e4m3, const float* b_s,
+                               void* c, int c_dtype, int64_t M, int64_t N, int64_t K, void* stream);
 /* ref: quantization/int8_kernel.py:174-257 (scales fp16 in the reference; s_dtype F16/BF16/F32) */
 int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const void* b_s,
                        int s_dtype, void* c, int c_dtype, int64_t M, int64_t N, int64_t K,

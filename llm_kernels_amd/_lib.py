@@ -38,6 +38,7 @@ SIGNATURES = {
     "llmk_weight_dequant_i8_block": [_p, _p, _i, _p, _i, _l, _l, _i, _p],
     "llmk_weight_dequant_w4a8": [_p, _p, _p, _p, _p, _l, _l, _i, _i, _p],
     "llmk_gemm_fp8_block": [_p, _p, _p, _p, _p, _i, _l, _l, _l, _p, _l, _p],
+    "llmk_gemm_fp8_block_static": [_p, _p, _p, _p, _p, _i, _l, _l, _l, _p],
     "llmk_gemm_i8_block": [_p, _p, _p, _p, _i, _p, _i, _l, _l, _l, _p, _l, _p],
     "llmk_gemm_i8_rowcol": [_p, _p, _p, _p, _p, _i, _p, _l, _l, _l, _p],
     "llmk_gemm_w4a8": [_p, _p, _p, _p, _i, _p, _p, _p, _i, _l, _l, _l, _i, _p, _l, _p],

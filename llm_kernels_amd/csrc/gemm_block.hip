@@ -1,4 +1,6 @@
 // Dense block-scaled fp8 / int8 GEMM entry points.
+#include <mutex>
+
 #include "gemm_wide.hpp"
 
 using namespace llmk;
@@ -102,4 +104,56 @@ extern "C" int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8
     // large M: the tile kernels accumulate int32 over the whole K range inside the MFMA and scale in the epilogue
     if (M > 64 && dma_eligible(p)) return launch_dma<K_I8_ROWCOL, false>(p, (hipStream_t)stream, "gemm_i8_rowcol(tiled)");
     return launch_direct<K_I8_ROWCOL, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_rowcol");
+}
+
+// ------------------------------------------------------------------ llmk_gemm_fp8_block without a scratch argument
+// For callers that cannot allocate device memory (HIP graph capture, serving loops, harnesses that forbid
+// hipMalloc): the fp32 partial sums of the split-K / K-range kernels live in a file-scope device array instead
+// of a caller-provided buffer.  Every GPU the library runs on holds its own copy of the array until the
+// process ends; its address on a device is looked up once, with that device current, and only that address
+// (never the array's name, which is a host-side stand-in) is handed to kernels.
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[LLMK_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void** out, const char* name) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: hipGetDevice: %s", name, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) LLMK_FAIL(LLMK_ERR_ARG, "%s: device ordinal %d out of range", name, dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", name, dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return LLMK_OK;
+}
+
+}  // namespace
+
+extern "C" int llmk_gemm_fp8_block_static(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                                          int c_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+    int rc = check_common("gemm_fp8_block_static", a, b, M, N, K, c_dtype);
+    if (rc) return rc;
+    const int64_t need = llmk_gemm_workspace_bytes(M, N, K);
+    if (need > (int64_t)LLMK_STATIC_SCRATCH_BYTES)
+        LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_fp8_block_static: M=%lld N=%lld K=%lld needs %lld bytes of scratch, the built-in "
+                  "buffer holds %lld; use llmk_gemm_fp8_block with a caller-provided workspace",
+                  (long long)M, (long long)N, (long long)K, (long long)need, (long long)LLMK_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (need > 0) {
+        rc = static_scratch(&ws, "gemm_fp8_block_static");
+        if (rc) return rc;
+    }
+    // Every plane of partial sums is written in full by the first kernel before the summing kernel reads it,
+    // so nothing in the array has to start at zero; what a previous (possibly larger) call left is never read.
+    return llmk_gemm_fp8_block(a, a_s, b, b_s, c, c_dtype, M, N, K, ws, need > 0 ? need : 0, stream);
 }

@@ -41,6 +41,9 @@ def test_version_and_error_paths_without_gpu():
     assert rc == -1 and b"multiple of 64" in lib.llmk_last_error()
     rc = lib.llmk_gemm_w4a16_marlin(None, None, None, None, 15, 64, 64, 16, None, 0, None)
     assert rc == -1
+    # the entry point with the built-in scratch refuses shapes beyond it before touching the GPU
+    rc = lib.llmk_gemm_fp8_block_static(256, 256, 256, 256, 256, 2, 16, 128256, 20480, None)
+    assert rc == -1 and b"built-in" in lib.llmk_last_error()
     rc = lib.llmk_pack_rows(None, 1, None, 4, 4, 3, 32, None)
     assert rc == -2
     rc = lib.llmk_act_quant_i8(None, 0, None, None, 4, 100, 0, None)
