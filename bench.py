@@ -143,6 +143,7 @@ class MoECase:
 
 
 CPU_BUDGET_S = 10.0       # the CPU baseline repeats its pass until this much time has gone by
+CPU_BUDGET_HEADLINE_S, CPU_BUDGET_OTHER_S = 10.0, 1.5
 
 
 def _timed_passes(run, budget):
@@ -282,50 +283,86 @@ HEADLINE_SET = ["w4a16_m16_n4096_k4096", "w4a16_nk_m16_n4096_k4096", "w4a16_nk_m
                 "w4a16_m4096_n4096_k4096", "w4a16_nk_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "int8_pt_m4096_n14336_k4096", "w4a8_m16_n4096_k4096", "moe_mixtral_fp8_t4096", "moe_mixtral_fp8_t16"]
 
 
+PREROLL_MS = 150.0        # untimed replays of the captured steps before anything is timed (clock and cache state settle)
+TIMED_REPLAYS = 7         # every replay times exactly `steps` steps; the median replay is reported
+_flush_buf = None
+
+
+def _flush_caches(dev):
+    """Read and write 1 GiB on the current stream: afterwards neither the L2s nor the 256 MB memory-side cache
+    hold any operand of the case, whatever --steps is.  (It also keeps the GPU busy while the host queues the
+    timed replay, so the events bracket GPU work only.)"""
+    global _flush_buf
+    if _flush_buf is None:
+        _flush_buf = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
+    _flush_buf.add_(1)
+
+
 def run_case(case, dev, steps, warmup, eager=False):
-    """Returns (wall seconds, HIP-event milliseconds) for exactly `steps` steps.
+    """Times exactly `steps` steps, TIMED_REPLAYS times over; returns a dict of timings.
 
     The steps are captured once into a HIP graph and replayed, so that the timed region is bound by the
     GPU and not by the Python launch path (decode-sized kernels last a few microseconds).  Events are
-    recorded on the stream the replay runs on.
+    recorded on the stream the replay runs on.  Before anything is timed the captured steps are replayed
+    for PREROLL_MS, so the first case of a process is not measured on idle clocks.  HBM-bound cases give every
+    step of a replay its own copy of the weights where that is possible (steps <= copies; otherwise a copy
+    returns only after 512 MB of other copies went by) and every timed replay starts behind a 1 GiB
+    read-modify-write, so no step finds its weights in a cache.
     """
     case.setup(dev)
     for i in range(warmup):
         case.launch(i)
     torch.cuda.synchronize()
     graph = None
+
+    def replay():
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                case.launch(warmup + i)
+
     if not eager:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             for i in range(steps):
                 case.launch(warmup + i)
-        graph.replay()                   # untimed replay (first replay uploads the graph)
+        graph.replay()                   # first replay uploads the graph
         torch.cuda.synchronize()
+    # pre-roll
+    t0 = time.perf_counter()
+    n_pre = 0
+    while n_pre < 2 or (time.perf_counter() - t0) * 1e3 < PREROLL_MS:
+        replay()
+        n_pre += 1
+        if n_pre % 8 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    preroll_ms = (time.perf_counter() - t0) * 1e3
     # wall clock: exactly `steps` steps between two host synchronisations (includes the host-side cost of
     # launching the graph, about 0.2 ms per replay)
-    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(steps):
-            case.launch(warmup + i)
+    replay()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    # HIP events: the same `steps` steps again, queued behind an untimed replay that is not waited for, so
-    # that the launch of the timed replay hides behind it and the events bracket GPU work only
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    if graph is not None:
-        graph.replay()
-    e0.record()
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(steps):
-            case.launch(warmup + i)
-    e1.record()
-    torch.cuda.synchronize()
-    return wall, e0.elapsed_time(e1)
+    # HIP events around each timed replay.  The replay is queued behind GPU work that is not waited for (the
+    # cache flush for HBM-bound cases, an untimed replay otherwise), so its launch cost hides behind that work.
+    cold = case.bound == "hbm"
+    ev = []
+    for _ in range(TIMED_REPLAYS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if cold:
+            _flush_caches(dev)
+        else:
+            replay()
+        e0.record()
+        replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ev.append(e0.elapsed_time(e1))
+    ev.sort()
+    return {"wall": wall, "ev_ms": ev[len(ev) // 2], "ev_ms_min": ev[0], "ev_ms_max": ev[-1],
+            "preroll_ms": preroll_ms, "preroll_replays": n_pre, "cold": cold}
 
 
 def measured_traffic(workload):
@@ -337,8 +374,8 @@ def measured_traffic(workload):
         return None
 
 
-def record(case, wall, ev_ms, steps):
-    dur = ev_ms / 1e3 / steps                       # average launch-to-launch duration from HIP events
+def record(case, t, steps):
+    dur = t["ev_ms"] / 1e3 / steps                  # average launch-to-launch duration from HIP events, median replay
     tflops = case.flops / dur / 1e12
     gbs = case.bytes / dur / 1e9
     if case.bound == "hbm":
@@ -349,8 +386,31 @@ def record(case, wall, ev_ms, steps):
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": pk, "unit": "TFLOP/s",
                 "frac": round(tflops / pk, 4), "traffic": measured_traffic(case.name)}
     return {"workload": case.name, "M": case.M, "N": case.N, "K": case.K, "us_per_launch": round(dur * 1e6, 2),
+            "us_per_launch_min": round(t["ev_ms_min"] * 1e3 / steps, 2), "us_per_launch_max": round(t["ev_ms_max"] * 1e3 / steps, 2),
+            "timed_replays": TIMED_REPLAYS, "preroll_ms": round(t["preroll_ms"], 1), "preroll_replays": t["preroll_replays"],
+            "cache_flushed_before_each_replay": t["cold"],
             "tflops": round(tflops, 2), "gbs": round(gbs, 1), "alg_bytes": case.bytes, "flops": case.flops,
-            "weight_copies_rotated": case.nbuf, "wall_ms_per_step": round(wall * 1e3 / steps, 4), "roofline": roof}
+            "weight_copies_rotated": case.nbuf, "wall_ms_per_step": round(t["wall"] * 1e3 / steps, 4), "roofline": roof}
+
+
+def cpu_baseline(case, budget):
+    """The oracle's dequantize-then-matmul on the host cores for a bounded sample of the case."""
+    global CPU_BUDGET_S
+    CPU_BUDGET_S = budget
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    max_rows = 512 if case.op == "moe" else 4096       # bounded sample of the same workload
+    dt, rows = case.cpu_seconds(max_rows)
+    if case.op == "copy":
+        return {"value": round(case.bytes / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "host memcpy of the same size"}
+    cpu_flops = case.flops * rows / case.T if case.op == "moe" else 2.0 * rows * case.N * case.K
+    return {"value": round(cpu_flops / dt / 1e12, 4), "unit": "TFLOP/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
+                      "1 warm-up + %d timed passes of %.3f s each, weight dequantisation included in every pass"
+                      % (rows, case.T if case.op == "moe" else case.M, getattr(case, "cpu_passes", 1), dt)}
 
 
 def main():
@@ -387,8 +447,8 @@ def main():
             WORKLOADS[args.workload] = (m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4)))
         op, M, N, K = WORKLOADS[args.workload]
         case = Case(args.workload, op, M, N, K)
-    wall, ev_ms = run_case(case, dev, args.steps, args.warmup, args.eager)
-    rec = record(case, wall, ev_ms, args.steps)
+    t = run_case(case, dev, args.steps, args.warmup, args.eager)
+    rec = record(case, t, args.steps)
 
     cases = []
     if not args.headline_only and args.workload in WORKLOADS:
@@ -396,28 +456,14 @@ def main():
             if name == args.workload:
                 continue
             c = MoECase(name, *MOE_WORKLOADS[name]) if name in MOE_WORKLOADS else Case(name, *WORKLOADS[name])
-            w2, e2 = run_case(c, dev, args.steps, args.warmup, args.eager)
-            cases.append(record(c, w2, e2, args.steps))
+            r2 = record(c, run_case(c, dev, args.steps, args.warmup, args.eager), args.steps)
+            if not args.no_cpu:
+                r2["cpu_baseline"] = cpu_baseline(c, CPU_BUDGET_OTHER_S)
+            cases.append(r2)
             del c
             torch.cuda.empty_cache()
 
-    cpu = None
-    if not args.no_cpu:
-        cores = os.cpu_count() or 1
-        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-        torch.set_num_threads(cores)
-        max_rows = 512 if op == "moe" else 4096       # bounded sample of the same workload
-        dt, rows = case.cpu_seconds(max_rows)
-        if op == "copy":
-            cpu = {"value": round(case.bytes / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
-                   "sample": "host memcpy of the same size"}
-        else:
-            cpu_flops = case.flops * rows / case.T if op == "moe" else 2.0 * rows * N * K
-            cpu = {"value": round(cpu_flops / dt / 1e12, 4), "unit": "TFLOP/s",
-                   "cores": torch.get_num_threads(), "kind": "port",
-                   "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
-                             "1 warm-up + %d timed passes of %.3f s each, weight dequantisation included in every pass"
-                             % (rows, M, getattr(case, "cpu_passes", 1), dt)}
+    cpu = None if args.no_cpu else cpu_baseline(case, CPU_BUDGET_HEADLINE_S)
 
     out = {
         "metric": "w4a16/fp8 GEMM TFLOPS & % roofline (HBM at M=16, MFMA at M=4096)",
@@ -425,7 +471,11 @@ def main():
         "ms_per_step": round(rec["us_per_launch"] / 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": case.dtype, "data": "synthetic",
         "config": {"workload": args.workload, "M": M, "N": N, "K": K, "weight_copies_rotated": case.nbuf,
-                   "us_per_launch_hip_events": rec["us_per_launch"], "wall_ms_per_step": rec["wall_ms_per_step"], "alg_bytes": rec["alg_bytes"],
+                   "us_per_launch_hip_events": rec["us_per_launch"], "us_per_launch_min": rec["us_per_launch_min"],
+                   "us_per_launch_max": rec["us_per_launch_max"], "timed_replays": TIMED_REPLAYS,
+                   "preroll_ms": rec["preroll_ms"], "preroll_replays": rec["preroll_replays"],
+                   "cache_flushed_before_each_replay": rec["cache_flushed_before_each_replay"],
+                   "wall_ms_per_step": rec["wall_ms_per_step"], "alg_bytes": rec["alg_bytes"],
                    "flops": rec["flops"], "launch": "eager" if args.eager else "hip_graph"},
         "roofline": rec["roofline"], "cpu_baseline": cpu,
     }
