@@ -70,6 +70,13 @@ int llmk_act_quant_fp8(const void* x, int x_dtype, void* y_e4m3, float* s, int64
 int llmk_act_quant_i8(const void* x, int x_dtype, int8_t* y, void* s_f16, int64_t n_groups,
                       int block, int round_mode, void* stream);
 
+/* One group per row of x [rows, cols] (any cols >= 1): s[row] = max|x[row]| / 127 in fp32 (stored fp32),
+ * y = round-half-away(x / s) int8.  The per-token activation / per-output-channel weight quantizer of the
+ * W8A8 scheme with one scale per row; the reference has no function of this shape, its nearest relative is
+ * the 1 x 128 group kernel quantization/int8_kernel.py:9-31 (same arithmetic, group = whole row). */
+int llmk_quant_i8_rowwise(const void* x, int x_dtype, int8_t* y, float* s, int64_t rows, int64_t cols,
+                          void* stream);
+
 /* block x block weight quantizers over W [M, N].
  * ref: quantization/int8_kernel.py:59-113 (qmax 127, half-away, no clamp)
  *      quantization/w4a8_kernel.py:196-225 (qmax 119, half-up, clamp +-119)
@@ -227,6 +234,13 @@ int llmk_moe_post_reorder(const void* down_out, void* out, int dtype, const int3
                           const void* topk_ids, int ids_bytes, const void* topk_weights, int w_dtype,
                           int start_expert, int end_expert, int topk, int64_t T, int64_t hidden,
                           void* stream);
+/* Per-expert scalar scales (the `use_fp8_w8a8` branch without block_shape that the reference keeps commented
+ * out, moe/group_gemm_kernel.py:417-420) written in the block-scale layout of llmk_grouped_gemm, in one launch
+ * and without reading anything back: scale_a[r, 0:K/128] = sa[e] for the rows r of segment e (0 for rows
+ * outside every segment), scale_b[w, :, :] = sb[w] for the Eb weight matrices.  sa [E], sb [Eb] fp32. */
+int llmk_moe_expert_scales(const float* sa, const float* sb, const int64_t* seg_indptr, int E, int Eb,
+                           int64_t M, int64_t N, int64_t K, void* scale_a, void* scale_b, int s_dtype,
+                           void* stream);
 /* C[seg[e]:seg[e+1], :] = A[seg[e]:seg[e+1], :] x B[weight_indices[e]]^T  for e < E.
  * a [M,K], b [E,N,K], c [M,N]; scale_a [M,K/128], scale_b [E,ceil(N/128),K/128] for the
  * block-scaled kinds (s_dtype = dtype code of both), NULL otherwise.  workspace: optional scratch of

@@ -31,6 +31,7 @@ SIGNATURES = {
     "llmk_unpack_cols": [_p, _i, _p, _i, _l, _l, _i, _i, _p],
     "llmk_act_quant_fp8": [_p, _i, _p, _p, _l, _i, _p],
     "llmk_act_quant_i8": [_p, _i, _p, _p, _l, _i, _i, _p],
+    "llmk_quant_i8_rowwise": [_p, _i, _p, _p, _l, _l, _p],
     "llmk_weight_quant_i8_block": [_p, _i, _p, _p, _l, _l, _i, _f, _i, _i, _p],
     "llmk_weight_quant_fp8_block": [_p, _i, _p, _p, _l, _l, _i, _p],
     "llmk_weight_quant_w4a8_level2": [_p, _p, _p, _l, _l, _i, _p],
@@ -59,6 +60,7 @@ SIGNATURES = {
     "llmk_moe_act_and_mul_quant": [_p, _i, _p, _p, _i, _i, _p, _i, _p, _i, _i, _l, _l, _i, _p],
     "llmk_moe_pre_reorder_quant": [_p, _i, _p, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _l, _l, _p],
     "llmk_moe_post_reorder": [_p, _p, _i, _p, _p, _i, _p, _i, _i, _i, _i, _l, _l, _p],
+    "llmk_moe_expert_scales": [_p, _p, _p, _i, _i, _l, _l, _l, _p, _p, _i, _p],
     "llmk_grouped_gemm": [_p, _p, _p, _i, _i, _i, _l, _l, _l, _p, _p, _p, _p, _i, _p, _l, _p],
 }
 _RESTYPE = {"llmk_last_error": _c.c_char_p, "llmk_gemm_workspace_bytes": _l,

@@ -39,18 +39,59 @@ def _compile(src):
     return obj
 
 
+def _assembly(src):
+    """Device assembly of one source (same flags as the object), for the static check of check_asm.py."""
+    out = os.path.join(OBJ, os.path.basename(src)[:-4] + ".s")
+    cmd = [hipcc(), *FLAGS, "-S", "--cuda-device-only", src, "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc -S failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    return out
+
+
+def _has_asm_register_loads(src):
+    """True when the source (or a header of csrc/ it includes) issues register loads from inline asm."""
+    seen, todo = set(), [src]
+    while todo:
+        p = todo.pop()
+        if p in seen or not os.path.exists(p):
+            continue
+        seen.add(p)
+        text = open(p).read()
+        if "asm_load_" in text:
+            return True
+        for line in text.splitlines():
+            line = line.strip()
+            if line.startswith('#include "'):
+                todo.append(os.path.join(CSRC, line.split('"')[1]))
+    return False
+
+
 def build(jobs=None, verbose=True):
+    from . import check_asm
     os.makedirs(OBJ, exist_ok=True)
     srcs = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
     jobs = jobs or min(8, len(srcs))
+    # Kernels that load registers from inline asm are only correct while the compiler never touches the
+    # destination before the hand-placed wait: prove it on the assembly of this very build, or fail.
+    asm_srcs = [s for s in srcs if _has_asm_register_loads(s)]
     with cf.ThreadPoolExecutor(jobs) as ex:
+        asm_jobs = [ex.submit(_assembly, s) for s in asm_srcs]
         objs = list(ex.map(_compile, srcs))
+        checked = 0
+        for j in asm_jobs:
+            n, problems = check_asm.check_file(j.result())
+            checked += n
+            if problems:
+                raise RuntimeError("hand-issued register loads are not safe in this build:\n  " + "\n  ".join(problems[:20]))
+    if asm_srcs and checked == 0:
+        raise RuntimeError("check_asm found no hand-issued loads in %s: the check no longer sees them" % asm_srcs)
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
     if verbose:
-        print("built", LIB, "from", len(srcs), "sources")
+        print("built", LIB, "from", len(srcs), "sources;", checked, "hand-issued register loads verified in the assembly")
     return LIB
 
 

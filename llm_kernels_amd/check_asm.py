@@ -1,0 +1,155 @@
+"""Static check of the device assembly for the hand-issued register loads.
+
+Some tile kernels issue global loads that land in VGPRs from inline asm, so that they share the hand-counted
+vmcnt scheme of the direct-to-LDS loads.  The compiler believes such a destination register holds its value
+as soon as the asm statement has been issued; the code is only correct while nothing reads, copies, spills or
+overwrites that register before an `s_waitcnt vmcnt(n)` that really covers the load.  This module proves that
+property on the generated assembly, for every path of the control-flow graph:
+
+  for every vector-memory load between `;;#ASMSTART` / `;;#ASMEND` whose destination is a VGPR (not an LDS
+  load), on every path from the load: no instruction names a destination register until an `s_waitcnt` whose
+  vmcnt is <= the number of vector-memory instructions issued after the load on that path (loads return in
+  order, so the load has then landed).
+
+It also refuses kernels with register spills or a private (scratch) segment among those that contain such
+loads.  build.py runs it on every source and fails the build when it does not hold.
+"""
+import re
+import sys
+
+_LABEL = re.compile(r"^([.\w$]+):")
+_REG1 = re.compile(r"\bv(\d+)\b")
+_REGR = re.compile(r"\bv\[(\d+):(\d+)\]")
+_VMCNT = re.compile(r"vmcnt\((\d+)\)")
+_VM_PREFIX = ("global_load", "global_store", "global_atomic", "buffer_load", "buffer_store", "buffer_atomic",
+              "flat_load", "flat_store", "flat_atomic", "scratch_load", "scratch_store")
+
+
+def _regs(text):
+    out = set(int(m) for m in _REG1.findall(text))
+    for a, b in _REGR.findall(text):
+        out.update(range(int(a), int(b) + 1))
+    return out
+
+
+class _Func:
+    def __init__(self, name):
+        self.name = name
+        self.ins = []          # (opcode, operand text, in_asm_block)
+        self.labels = {}       # label -> index of the next instruction
+
+
+def _parse(path):
+    funcs, cur, in_asm = [], None, False
+    meta = {}                  # kernel name -> {"spill": n, "private": n}
+    meta_name = None
+    for raw in open(path, errors="replace"):
+        line = raw.split("//")[0].rstrip()
+        s = line.strip()
+        if s.startswith("- ."):                  # first key of a YAML list item in the kernel metadata
+            s = s[2:]
+        if s.startswith(".name:"):
+            meta_name = s.split(":", 1)[1].strip()
+            meta.setdefault(meta_name, {})
+        elif meta_name and s.startswith(".vgpr_spill_count:"):
+            meta[meta_name]["spill"] = int(s.split(":")[1])
+        elif meta_name and s.startswith(".sgpr_spill_count:"):
+            meta[meta_name]["sspill"] = int(s.split(":")[1])
+        elif meta_name and s.startswith(".private_segment_fixed_size:"):
+            meta[meta_name]["private"] = int(s.split(":")[1])
+        if s.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if s.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        m = _LABEL.match(line)
+        if m and not line[0].isspace():
+            lab = m.group(1)
+            if not lab.startswith(".L"):
+                cur = _Func(lab)
+                funcs.append(cur)
+            elif cur is not None:
+                cur.labels[lab] = len(cur.ins)
+            continue
+        if cur is None or not s or s.startswith(".") or s.startswith(";"):
+            continue
+        code = s.split(";")[0].strip()
+        if not code:
+            continue
+        parts = code.split(None, 1)
+        cur.ins.append((parts[0], parts[1] if len(parts) > 1 else "", in_asm))
+    return funcs, meta
+
+
+def _is_vm(op):
+    return op.startswith(_VM_PREFIX)
+
+
+def check_file(path):
+    """Returns (number of hand-issued register loads checked, list of violation strings)."""
+    funcs, meta = _parse(path)
+    problems, checked = [], 0
+    for f in funcs:
+        loads = [i for i, (op, args, in_asm) in enumerate(f.ins)
+                 if in_asm and op.startswith(("global_load", "buffer_load", "flat_load")) and "_lds_" not in op]
+        if not loads:
+            continue
+        md = meta.get(f.name, {})
+        if md.get("spill", 0) or md.get("private", 0):
+            problems.append("%s: kernel with hand-issued register loads has %d spilled VGPRs and %d bytes of scratch"
+                            % (f.name, md.get("spill", 0), md.get("private", 0)))
+        for li in loads:
+            checked += 1
+            dest = _regs(f.ins[li][1].split(",")[0])
+            if not dest:
+                problems.append("%s: cannot parse the destination of `%s %s`" % (f.name, *f.ins[li][:2]))
+                continue
+            best = {}                      # instruction index -> fewest younger vector-memory instructions seen
+            stack = [(li + 1, 0)]
+            while stack:
+                i, younger = stack.pop()
+                while True:
+                    if i >= len(f.ins):
+                        problems.append("%s: load at #%d: ran off the function without a covering s_waitcnt" % (f.name, li))
+                        break
+                    if i in best and best[i] <= younger:
+                        break
+                    best[i] = younger
+                    op, args, _ = f.ins[i]
+                    if op == "s_waitcnt":
+                        m = _VMCNT.search(args)
+                        if m and int(m.group(1)) <= younger:
+                            break                                   # the load has landed on this path
+                    elif op == "s_endpgm":
+                        break                                       # never consumed on this path
+                    if op != "s_waitcnt" and dest & _regs(args):
+                        problems.append("%s: `%s %s` touches v%s of the hand-issued load #%d (`%s`) before a covering "
+                                        "s_waitcnt" % (f.name, op, args, sorted(dest & _regs(args)), li, f.ins[li][1]))
+                        break
+                    if _is_vm(op):
+                        younger += 1
+                    if op == "s_branch":
+                        i = f.labels.get(args.strip(), len(f.ins))
+                        continue
+                    if op.startswith("s_cbranch"):
+                        tgt = f.labels.get(args.strip())
+                        if tgt is not None:
+                            stack.append((tgt, younger))
+                    if op in ("s_setpc_b64", "s_swappc_b64"):
+                        problems.append("%s: indirect jump after a hand-issued load" % f.name)
+                        break
+                    i += 1
+    return checked, problems
+
+
+if __name__ == "__main__":
+    total, bad = 0, []
+    for p in sys.argv[1:]:
+        n, pr = check_file(p)
+        total += n
+        bad += pr
+    print("%d hand-issued register loads checked, %d problems" % (total, len(bad)))
+    for b in bad[:40]:
+        print("  " + b)
+    sys.exit(1 if bad else 0)

@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <atomic>
 
 #include "../../include/llmk.h"
 
@@ -134,3 +135,19 @@ __device__ __forceinline__ v4f mfma_bf16_16x16x32(v8bf a, v8bf b, v4f c) {
 }
 
 static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ------------------------------------------------------------------ one-time launch set-up (host)
+// Opt a kernel into more than 64 KB of dynamic LDS, once per device.  `done` is a bit mask of the device
+// ordinals already configured (one static mask per launch site); the call is idempotent, so two threads that
+// race here merely both make it.
+static inline int llmk_reserve_lds(const void* kern, int bytes, std::atomic<uint64_t>& done, const char* name) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: hipGetDevice: %s", name, hipGetErrorString(e));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return LLMK_OK;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+    done.fetch_or(bit, std::memory_order_release);
+    return LLMK_OK;
+}

@@ -434,7 +434,8 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
             if (p.kc_steps > NW * U || !p.partial) LLMK_FAIL(LLMK_ERR_ARG, "%s: bad K range setup", name);
             const int nz = (steps + p.kc_steps - 1) / p.kc_steps;
             const size_t smem_r = (size_t)2 * NW * 256 * sizeof(float) + (size_t)16 * p.kc_steps * sizeof(float);
-            static int slots_r = 0;
+            static std::atomic<int> slots_r_cache{0};     // same value on every MI355X; recomputing it is harmless
+            int slots_r = slots_r_cache.load(std::memory_order_relaxed);
             if (slots_r == 0) {
                 int dev = 0, cus = 0, per_cu = 0;
                 hipError_t e = hipGetDevice(&dev);
@@ -443,6 +444,7 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
                     e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, 1, NW, false, true, SDT, false, true>, NW * 64, smem_r);
                 if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
                 slots_r = max(1, cus * max(1, per_cu));
+                slots_r_cache.store(slots_r, std::memory_order_relaxed);
             }
             const int rows = mtiles * nz;
             int gx = min(ntiles, max(1, slots_r / min(rows, slots_r)));
@@ -462,7 +464,8 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
     // long K: consecutive steps per wave, one load for the four weight scales of a batch (measured faster at
     // K = 14336, slower at K = 4096 where the interleaved order spreads the first requests over more channels)
     const bool vec = CAN_VEC && !resident && steps % 4 == 0;
-    static int slots[2] = {0, 0};             // resident workgroups on the whole device, per kernel variant
+    static std::atomic<int> slots_cache[2];   // resident workgroups on the whole device, per kernel variant
+    int slots[2] = {slots_cache[0].load(std::memory_order_relaxed), slots_cache[1].load(std::memory_order_relaxed)};
     if (slots[resident] == 0) {
         int dev = 0, cus = 0, per_cu = 0;
         hipError_t e = hipGetDevice(&dev);
@@ -472,6 +475,7 @@ int launch_direct_sdt(const DirectArgs& p, hipStream_t stream, const char* name)
                          : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_direct_kernel<KIND, MT, NW, GROUPED, false, SDT>, NW * 64, 64 * 1024);
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: occupancy query failed: %s", name, hipGetErrorString(e));
         slots[resident] = max(1, cus * max(1, per_cu));
+        slots_cache[resident].store(slots[resident], std::memory_order_relaxed);
     }
     int gx = min(ntiles, max(1, slots[resident] / min(mtiles, slots[resident])));
     // every workgroup the same number of column tiles (the slowest one sets the time): fewer workgroups

@@ -94,7 +94,10 @@ __device__ __forceinline__ v4i w4_word_to_f16x8(unsigned w, v2h sc) {
 }
 // Register loads issued from inline asm like the direct-to-LDS loads, so that they take part in the same
 // hand-counted vmcnt scheme (a compiler-tracked load would make the compiler wait for every load in flight).
-// The destination is only read behind an explicit s_waitcnt.
+// The destination is only read behind an explicit s_waitcnt that names it as a read-write operand.  The
+// compiler takes the register for ready as soon as the load is issued, so the scheme holds only while it
+// neither copies, spills nor reuses the register before that wait: check_asm.py proves exactly that on the
+// assembly of every build (all control-flow paths from each such load), and the build fails otherwise.
 __device__ __forceinline__ uint64_t asm_load_b64(uint32_t voff, const void* sbase) {
     uint64_t v;
     asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
@@ -300,11 +303,14 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     };
     // K_W4NK: packed words and group scale of K step kt -> registers (requested before the activation loads
     // of the same step, so that waiting for them leaves exactly those MI loads in flight) ...
+    // (the group scale is one halfword for the row-packed layout and four for a Marlin half unit: separate
+    // variables of the exact register width, so that no widening move is ever placed between load and wait)
     uint64_t w4_words = 0, w4_scale = 0;
+    unsigned w4_scale16 = 0;
     auto w4_request = [&](int kt) {
         if constexpr (W4NK) {
             w4_words = asm_load_b64(w4_off, (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 32);
-            w4_scale = asm_load_u16(w4_soff, (const uint8_t*)p.b_s + (int64_t)(((kt0 + kt) * 64) / p.group) * 2);
+            w4_scale16 = asm_load_u16(w4_soff, (const uint8_t*)p.b_s + (int64_t)(((kt0 + kt) * 64) / p.group) * 2);
         }
         if constexpr (W4M) {
             w4_words = asm_load_b64(w4_off, (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 4 * (N >> 6) * 512);
@@ -314,11 +320,15 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // ... and from there, expanded, into the weight rows of stage kt
     auto w4_expand = [&](int kt) {
         if constexpr (W4) {
-            __builtin_amdgcn_s_waitcnt(0x0F70 | MI);       // everything but the MI youngest (activation) loads
+            // everything but the MI youngest (activation) loads.  The two registers pass through the wait as
+            // read-write operands: the compiler must have them in VGPRs here and takes every later use from
+            // this statement, so no use can be scheduled above the wait.
+            if constexpr (W4NK) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(w4_words), "+v"(w4_scale16) : "n"(MI) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%2)" : "+v"(w4_words), "+v"(w4_scale) : "n"(MI) : "memory");
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (W4NK) {
-            const unsigned s16 = (unsigned)w4_scale;
+            const unsigned s16 = w4_scale16;
             const v2h sc = w4_as_h2(s16 | (s16 << 16));
             uint8_t* dst = lds + (kt % D_NSTAGE) * D_STAGE + D_A + w4_lds;
             *(v4i*)dst = w4_word_to_f16x8((unsigned)w4_words, sc);
@@ -599,13 +609,9 @@ inline bool dma_eligible(const DirectArgs& p, int esz = 1) {
 // a_s must be fp32 here (p.a_s); p.s_dtype describes b_s only.
 template <int KIND, bool GROUPED, int MI>
 int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
-    static bool configured = false;
+    static std::atomic<uint64_t> configured{0};
     auto kern = gemm_dma_kernel<KIND, GROUPED, MI>;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, d_lds(MI));
-        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, d_lds(MI), hipGetErrorString(e));
-        configured = true;
-    }
+    if (int rc = llmk_reserve_lds((const void*)kern, d_lds(MI), configured, name)) return rc;
     constexpr int BM = 64 * MI;
     const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, BM) : (p.M + BM - 1) / BM;
     const bool split = !GROUPED && p.ksplit > 1 && p.partial;

@@ -142,13 +142,9 @@ __global__ __launch_bounds__(T_THREADS) void gemm_tiled_kernel(DirectArgs p) {
 
 template <int KIND, bool GROUPED, int SDT>
 int launch_tiled_sdt(const DirectArgs& p, hipStream_t stream, const char* name) {
-    static bool configured = false;
+    static std::atomic<uint64_t> configured{0};
     auto kern = gemm_tiled_kernel<KIND, GROUPED, SDT>;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, T_LDS);
-        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, T_LDS, hipGetErrorString(e));
-        configured = true;
-    }
+    if (int rc = llmk_reserve_lds((const void*)kern, T_LDS, configured, name)) return rc;
     const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, T_BM) : (p.M + T_BM - 1) / T_BM;
     dim3 grid((unsigned)((p.N + T_BN - 1) / T_BN), (unsigned)tiles_m);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;

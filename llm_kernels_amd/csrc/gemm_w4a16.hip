@@ -535,7 +535,8 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
     const int ntiles = (N + 16 * NT - 1) / (16 * NT), mtiles = (M + 16 * MT - 1) / (16 * MT);
     const bool resident = steps <= 8 * U;
     const size_t smem = (size_t)2 * 8 * NT * MT * 256 * sizeof(float);
-    static int slots[2] = {0, 0};
+    static std::atomic<int> slots_cache[2];
+    int slots[2] = {slots_cache[0].load(std::memory_order_relaxed), slots_cache[1].load(std::memory_order_relaxed)};
     if (slots[resident] == 0) {
         int dev = 0, cus = 0, per_cu = 0;
         hipError_t e = hipGetDevice(&dev);
@@ -545,6 +546,7 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
                          : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, w4a16_nk_stream_kernel<MT, NT, false>, 512, smem);
         if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a16_nk: occupancy query failed: %s", hipGetErrorString(e));
         slots[resident] = max(1, cus * max(1, per_cu));
+        slots_cache[resident].store(slots[resident], std::memory_order_relaxed);
     }
     const int rows = mtiles * nz;
     int gx = min(ntiles, max(1, slots[resident] / min(rows, slots[resident])));
@@ -678,13 +680,9 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
     const bool a_lds = a_bytes <= 144 * 1024 && (int64_t)pl.col_groups * pl.mblocks * pl.z <= 512;
     const size_t smem = a_lds && a_bytes > red_bytes ? a_bytes : red_bytes;
     if (smem > 64 * 1024) {
-        static bool configured = false;
-        if (!configured) {
-            hipError_t e = hipFuncSetAttribute((const void*)w4a16_marlin_kernel<1, 8, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            if (e == hipSuccess) e = hipFuncSetAttribute((const void*)w4a16_marlin_kernel<1, 8, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a16_marlin: cannot reserve LDS: %s", hipGetErrorString(e));
-            configured = true;
-        }
+        static std::atomic<uint64_t> cfg_a{0}, cfg_b{0};
+        if (int rc = llmk_reserve_lds((const void*)w4a16_marlin_kernel<1, 8, true, true>, 160 * 1024, cfg_a, "gemm_w4a16_marlin")) return rc;
+        if (int rc = llmk_reserve_lds((const void*)w4a16_marlin_kernel<1, 8, false, true>, 160 * 1024, cfg_b, "gemm_w4a16_marlin")) return rc;
     }
 #define LLMK_MARLIN_LAUNCH(MT, NW)                                                                              \
     do {                                                                                                        \

@@ -326,18 +326,16 @@ int launch_w4a8_stream(W4A8Args p, void* workspace, int64_t workspace_bytes, hip
     const size_t smem = (size_t)2 * 8 * MT * 256 * 4 + (size_t)MT * 16 * steps * 8 + (size_t)2 * 2 * (rounds * 8192 + 64);
     auto k1 = w4a8_stream_kernel<MT, SDT, 1>;
     auto k2 = w4a8_stream_kernel<MT, SDT, 2>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot reserve LDS: %s", hipGetErrorString(e));
-        configured = true;
-    }
-    static int cus = 0;
+    static std::atomic<uint64_t> cfg1{0}, cfg2{0};
+    if (int rc = llmk_reserve_lds((const void*)k1, 160 * 1024, cfg1, "gemm_w4a8")) return rc;
+    if (int rc = llmk_reserve_lds((const void*)k2, 160 * 1024, cfg2, "gemm_w4a8")) return rc;
+    static std::atomic<int> cus_cache{0};
+    int cus = cus_cache.load(std::memory_order_relaxed);
     if (cus == 0) {
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot query the device");
+        cus_cache.store(cus, std::memory_order_relaxed);
     }
     const int rows = mtiles * nz;                                      // workgroup rows that share the column tiles
     int gx = min(ntiles, max(1, cus / min(rows, cus)));                // one workgroup per CU (LDS bound)

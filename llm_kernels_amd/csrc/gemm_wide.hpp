@@ -337,14 +337,10 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 
 template <int KIND, bool GROUPED, int R = 8>
 int launch_wide(const DirectArgs& p, hipStream_t stream, const char* name) {
-    static bool configured = false;
+    static std::atomic<uint64_t> configured{0};
     auto kern = gemm_wide_kernel<KIND, GROUPED, R>;
     constexpr int W_BM = w_bm(R), W_LDS = w_lds(R);
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, W_LDS);
-        if (e != hipSuccess) LLMK_FAIL(LLMK_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", name, W_LDS, hipGetErrorString(e));
-        configured = true;
-    }
+    if (int rc = llmk_reserve_lds((const void*)kern, W_LDS, configured, name)) return rc;
     const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, W_BM) : (p.M + W_BM - 1) / W_BM;
     dim3 grid((unsigned)((p.N + W_BN - 1) / W_BN), (unsigned)tiles_m);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;

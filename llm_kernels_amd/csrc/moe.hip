@@ -345,7 +345,41 @@ __global__ void post_reorder_kernel(const void* __restrict__ down, void* __restr
     }
 }
 
+// ---------------------------------------------------------------- per-expert scalar scales -> block-scale layout
+// scale_a[r, :] = sa[e(r)] for the rows of segment e, scale_b[w, :, :] = sb[w]; rows outside every segment get 0.
+// Blocks [0, M) write one activation-scale row each, blocks [M, M + Eb) one expert's weight scales.
+template <int SDT>
+__global__ void expert_scales_kernel(const float* __restrict__ sa, const float* __restrict__ sb,
+                                     const int64_t* __restrict__ seg, int E, int64_t M, int kb, int64_t nbkb,
+                                     void* __restrict__ scale_a, void* __restrict__ scale_b) {
+    const int64_t blk = blockIdx.x;
+    if (blk < M) {
+        float v = 0.f;
+        for (int e = 0; e < E; ++e)
+            if (blk >= seg[e] && blk < seg[e + 1]) { v = sa[e]; break; }
+        for (int i = threadIdx.x; i < kb; i += blockDim.x) FloatIO<SDT>::st(scale_a, blk * kb + i, v);
+    } else {
+        const int64_t w = blk - M;
+        const float v = sb[w];
+        for (int64_t i = threadIdx.x; i < nbkb; i += blockDim.x) FloatIO<SDT>::st(scale_b, w * nbkb + i, v);
+    }
+}
+
 }  // namespace
+
+extern "C" int llmk_moe_expert_scales(const float* sa, const float* sb, const int64_t* seg_indptr, int E, int Eb,
+                                      int64_t M, int64_t N, int64_t K, void* scale_a, void* scale_b, int s_dtype,
+                                      void* stream) {
+    if (M < 0 || N < 0 || K < 0 || E < 0 || Eb < 0 || K % 128) LLMK_FAIL(LLMK_ERR_SHAPE, "moe_expert_scales: bad shape");
+    if (M + Eb == 0 || K == 0) return LLMK_OK;
+    if (!sa || !sb || !seg_indptr || !scale_a || !scale_b) LLMK_FAIL(LLMK_ERR_ARG, "moe_expert_scales: null pointer");
+    const int kb = (int)(K / 128);
+    const int64_t nbkb = ((N + 127) / 128) * kb;
+    LLMK_DISPATCH_FLOAT(s_dtype, SDT, (expert_scales_kernel<SDT><<<(unsigned)(M + Eb), 64, 0, (hipStream_t)stream>>>(
+        sa, sb, seg_indptr, E, M, kb, nbkb, scale_a, scale_b)));
+    LLMK_CHECK_LAUNCH("moe_expert_scales");
+    return LLMK_OK;
+}
 
 extern "C" int llmk_moe_seg_indptr(const int64_t* sorted_ids, int64_t* seg_indptr, int64_t num_toks, int num_experts,
                                    void* stream) {

@@ -62,6 +62,54 @@ __global__ void block_dequant_kernel(const uint8_t* __restrict__ y, const void* 
     for (int j = 0; j < EPL; ++j) FloatIO<ODT>::st(x, off + j, v[j]);
 }
 
+// ---------------------------------------------------------------- one group per row (per-token / per-channel int8)
+// One 256-thread workgroup per row of any length: absmax over the row, s = absmax / 127 in fp32 (stored
+// fp32), y = round-half-away(x / s).  The second pass re-reads the row, which the first pass left in cache.
+template <int DT>
+__global__ __launch_bounds__(256) void row_quant_i8_kernel(const void* __restrict__ x, int8_t* __restrict__ y,
+                                                           float* __restrict__ s, int64_t cols, bool vec) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x, base = row * cols;
+    const int t = threadIdx.x;
+    float m = 0.f;
+    if (vec) {
+        for (int64_t c = (int64_t)t * EPL; c < cols; c += 256 * EPL) {
+            float v[EPL];
+            load8<DT>(x, base + c, v);
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) m = fmaxf(m, fabsf(v[j]));
+        }
+    } else {
+        for (int64_t c = t; c < cols; c += 256) m = fmaxf(m, fabsf(FloatIO<DT>::ld(x, base + c)));
+    }
+    m = wave_max(m);
+    if ((t & 63) == 0) red[t >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float sc = m / 127.f;
+    const bool fast = div_by_ok(sc);
+    const float r = fast ? 1.0f / sc : 0.f;
+    if (vec) {
+        for (int64_t c = (int64_t)t * EPL; c < cols; c += 256 * EPL) {
+            float v[EPL];
+            load8<DT>(x, base + c, v);
+            unsigned w[2] = {0, 0};
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) {
+                const int qi = (int)roundf(fast ? div_by(v[j], sc, r) : v[j] / sc);
+                w[j >> 2] |= ((unsigned)(qi & 0xff)) << (8 * (j & 3));
+            }
+            *(uint2*)(y + base + c) = make_uint2(w[0], w[1]);
+        }
+    } else {
+        for (int64_t c = t; c < cols; c += 256) {
+            const float v = FloatIO<DT>::ld(x, base + c);
+            y[base + c] = (int8_t)(int)roundf(fast ? div_by(v, sc, r) : v / sc);
+        }
+    }
+    if (t == 0) s[row] = sc;
+}
+
 // ---------------------------------------------------------------- block x block weight quant
 // one 256-thread workgroup per (BLOCK x BLOCK) tile, BLOCK <= 128, BLOCK % 8 == 0.
 // thread t: column chunk (t % 16) * 8, rows t / 16 + 16 * j.
@@ -265,6 +313,19 @@ extern "C" int llmk_act_quant_i8(const void* x, int x_dtype, int8_t* y, void* s,
     LPG_SWITCH(block, CALL)
 #undef CALL
     LLMK_CHECK_LAUNCH("act_quant_i8");
+    return LLMK_OK;
+}
+
+extern "C" int llmk_quant_i8_rowwise(const void* x, int x_dtype, int8_t* y, float* s, int64_t rows, int64_t cols,
+                                     void* stream) {
+    if (rows < 0 || cols < 0 || rows > 0x7fffffff) LLMK_FAIL(LLMK_ERR_SHAPE, "quant_i8_rowwise: bad shape");
+    if (rows == 0) return LLMK_OK;
+    if (!y || !s || (cols && !x)) LLMK_FAIL(LLMK_ERR_ARG, "quant_i8_rowwise: null pointer");
+    const int esz = x_dtype == LLMK_F32 ? 4 : 2;
+    // 8 elements per lane when every row starts on a 16-byte (input) and 8-byte (output) boundary
+    const bool vec = cols % EPL == 0 && (((uintptr_t)x) & 15) == 0 && (((uintptr_t)y) & 7) == 0 && (cols * esz) % 16 == 0;
+    LLMK_DISPATCH_FLOAT(x_dtype, DT, (row_quant_i8_kernel<DT><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(x, y, s, cols, vec)));
+    LLMK_CHECK_LAUNCH("quant_i8_rowwise");
     return LLMK_OK;
 }
 

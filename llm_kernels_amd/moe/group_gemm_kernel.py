@@ -226,15 +226,17 @@ def grouped_gemm_triton(
         assert a.dtype == b.dtype, 'per-expert scaling takes activations already in the weight dtype'
         assert a.shape[-1] % 128 == 0, 'K must be a multiple of 128'
         kb = a.shape[-1] // 128
-        sdt = torch.float32 if b.dtype == torch.float8_e4m3fn else torch.float16
-        seg64 = seg_indptr.to(torch.int64)
-        rows = (seg64[1:batch_size + 1] - seg64[:batch_size])
-        sa = scale_a.to(torch.float32).flatten()[:batch_size]
-        row_scale = torch.zeros(a.shape[0], device=a.device, dtype=torch.float32)
-        row_scale[seg64[0]:seg64[batch_size]] = torch.repeat_interleave(sa, rows)
-        scale_a = row_scale.to(sdt).unsqueeze(1).expand(-1, kb).contiguous()
         nb = _cdiv(b.shape[1], 128)
-        scale_b = scale_b.to(sdt).flatten().view(-1, 1, 1).expand(-1, nb, kb).contiguous()
+        sdt = torch.float32 if b.dtype == torch.float8_e4m3fn else torch.float16
+        seg64 = (seg_indptr if seg_indptr.dtype == torch.int64 else seg_indptr.to(torch.int64)).contiguous()
+        sa = scale_a.to(torch.float32).flatten().contiguous()
+        sb = scale_b.to(torch.float32).flatten().contiguous()
+        assert sa.numel() >= batch_size and sb.numel() >= b.shape[0], 'one activation scale per segment, one weight scale per expert'
+        scale_a = torch.empty(a.shape[0], kb, device=a.device, dtype=sdt)
+        scale_b = torch.empty(b.shape[0], nb, kb, device=a.device, dtype=sdt)
+        # one launch, nothing read back (usable under graph capture)
+        _lib.call("llmk_moe_expert_scales", _lib.ptr(sa), _lib.ptr(sb), _lib.ptr(seg64), int(batch_size), b.shape[0],
+                  a.shape[0], b.shape[1], b.shape[2], _lib.ptr(scale_a), _lib.ptr(scale_b), _lib.dt(sdt), _lib.stream(a))
     elif quantised_w:
         raise AssertionError('quantised weights need block_shape=[128, 128] and scale_b, or use_fp8_w8a8 with per-expert scales')
     assert a.is_contiguous() and b.is_contiguous() and c.is_contiguous(), 'Input tensors must be contiguous'

@@ -46,7 +46,8 @@ def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> t
     _lib.require_gpu(x, s)
     M, N = x.size()
     y = torch.empty_like(x, dtype=torch.get_default_dtype())
-    _lib.call("llmk_weight_dequant_fp8_block", _lib.ptr(x), _lib.ptr(s.float()), _lib.ptr(y), _lib.dt(y.dtype),
+    s32 = s if s.dtype == torch.float32 else s.float()     # held until the launch is queued; no copy for fp32 scales
+    _lib.call("llmk_weight_dequant_fp8_block", _lib.ptr(x), _lib.ptr(s32), _lib.ptr(y), _lib.dt(y.dtype),
               M, N, block_size, _lib.stream(x))
     return y
 

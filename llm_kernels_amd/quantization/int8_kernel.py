@@ -68,13 +68,16 @@ def int8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor, b_s: torch.Te
 
 # ----------------------------------------------------------------------------- per-token x per-channel
 def _rowwise_quant(x: torch.Tensor):
-    # one group per row: the 1 x block kernel needs a power-of-two block, so rows go through torch here
-    xf = x.float()
-    amax = xf.abs().amax(dim=-1)
-    s = amax / torch.full_like(amax, 127.0)                       # tensor divisor: a true IEEE division on every device
-    v = xf / s.unsqueeze(-1)
-    t = torch.trunc(v)
-    y = (t + torch.sign(v) * ((v - t).abs() >= 0.5)).to(torch.int8)
+    """One scale per row of the last dimension: s = max|row| / 127 (fp32), y = round-half-away(x / s)."""
+    assert x.is_contiguous(), 'Input tensor must be contiguous'
+    _lib.require_gpu(x)
+    if x.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        x = x.float()
+    cols = x.size(-1)
+    rows = x.numel() // cols if cols else 0
+    y = torch.empty_like(x, dtype=torch.int8)
+    s = x.new_empty(x.size()[:-1], dtype=torch.float32)
+    _lib.call("llmk_quant_i8_rowwise", _lib.ptr(x), _lib.dt(x.dtype), _lib.ptr(y), _lib.ptr(s), rows, cols, _lib.stream(x))
     return y, s
 
 

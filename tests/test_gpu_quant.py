@@ -95,3 +95,34 @@ def test_w4a8_weight_quant_dequant(dev, shape):
     assert d.dtype == torch.float16 and torch.equal(d.cpu(), q.w4a8_weight_dequant(oq, os_, os4, oz4))
     cos = torch.nn.functional.cosine_similarity(d.float().flatten().cpu(), w.float().flatten(), dim=0)
     assert cos > 0.98
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 1), (5, 100), (16, 4096), (7, 14336), (3, 4, 333), (130, 1000), (2, 4104)])
+def test_rowwise_int8_quantizer(dev, dtype, shape):
+    """Per-token / per-channel int8 (one fp32 scale per row, any row length): integers and scales bit-exact,
+    ties away from zero included."""
+    announce("rowwise int8", dtype, shape)
+    torch.manual_seed(7)
+    x = torch.randn(*shape).to(dtype)
+    flat = x.view(-1, shape[-1])
+    if shape[-1] >= 8:
+        flat[0, :8] = torch.tensor([0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 127.0, -127.0]).to(dtype)   # absmax 127 -> s = 1: ties
+    y, s = int8_kernel.act_quant_per_token(x.to(dev))
+    oy, os_ = q.int8_quant_rowwise(flat)
+    assert y.dtype == torch.int8 and s.dtype == torch.float32 and y.shape == x.shape and s.shape == x.shape[:-1]
+    assert torch.equal(s.cpu().view(-1), os_)
+    assert torch.equal(y.cpu().view(-1, shape[-1]), oy)
+    y2, s2 = int8_kernel.weight_quant_per_channel(x.to(dev))
+    assert torch.equal(y2, y) and torch.equal(s2, s)
+
+
+def test_rowwise_int8_quantizer_zero_row_is_nan_free_of_crash(dev):
+    """An all-zero row gives s = 0 and 0/0 in the division, as the 1 x 128 quantizers do; other rows are untouched."""
+    announce("rowwise int8 zero row")
+    x = torch.zeros(2, 256)
+    x[1] = torch.linspace(-1, 1, 256)
+    y, s = int8_kernel.act_quant_per_token(x.to(dev))
+    oy, os_ = q.int8_quant_rowwise(x)
+    assert s.cpu()[0].item() == 0.0 and torch.equal(s.cpu(), os_)
+    assert torch.equal(y.cpu()[1], oy[1])
