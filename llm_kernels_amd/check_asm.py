@@ -8,8 +8,8 @@ property on the generated assembly, for every path of the control-flow graph:
 
   for every vector-memory load between `;;#ASMSTART` / `;;#ASMEND` whose destination is a VGPR (not an LDS
   load), on every path from the load: no instruction names a destination register until an `s_waitcnt` whose
-  vmcnt is <= the number of vector-memory instructions issued after the load on that path (loads return in
-  order, so the load has then landed).
+  vmcnt is <= the number of vector-memory loads issued after the load on that path (loads return in order
+  among themselves, so the load has then landed; stores are not counted, they may complete at any time).
 
 It also refuses kernels with register spills or a private (scratch) segment among those that contain such
 loads.  build.py runs it on every source and fails the build when it does not hold.
@@ -21,8 +21,9 @@ _LABEL = re.compile(r"^([.\w$]+):")
 _REG1 = re.compile(r"\bv(\d+)\b")
 _REGR = re.compile(r"\bv\[(\d+):(\d+)\]")
 _VMCNT = re.compile(r"vmcnt\((\d+)\)")
-_VM_PREFIX = ("global_load", "global_store", "global_atomic", "buffer_load", "buffer_store", "buffer_atomic",
-              "flat_load", "flat_store", "flat_atomic", "scratch_load", "scratch_store")
+# Only loads count as "younger": loads return in order among themselves, while a store may be acknowledged
+# before or after the loads around it, so a pending store can never vouch for a load having landed.
+_VM_PREFIX = ("global_load", "buffer_load", "flat_load", "scratch_load")
 
 
 def _regs(text):

@@ -3,6 +3,7 @@
 // nibble -> fp16 without integer->float converts: (q | 0x6400) is the fp16 number 1024 + q,
 // ((q << 4) | 0x6400) is 1024 + 16 q; one packed subtract / fma gives q - 8 exactly.
 #include "gemm_wide.hpp"
+#include "stream_ring.hpp"
 
 namespace {
 
@@ -359,6 +360,8 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     struct BBatch {
         v4i w[NT][U];
         unsigned short s[NT][U];
+        uint2 sv[NT];          // VS: the four scales of the batch as loaded (unpacked when the batch is multiplied:
+                               // any arithmetic on a value still in flight would wait for it right away)
     };
     struct ABatch {
         v4i a[U][MT][4];
@@ -367,26 +370,30 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     // consecutive steps and, with 128-wide groups, fetches their four scales with one load.
     auto step_of = [&](int ks0, int u) { return VS ? (ks0 - wave) + wave * U + u : ks0 + u * NW; };
     auto clamp_step = [&](int ks) { return min(ks, steps - 1); };
+    // Addresses are a wave-uniform base (tile, K step: scalar registers) plus one 32-bit offset per lane, so that
+    // a load needs no 64-bit per-lane address arithmetic and no address registers that could collide with
+    // the destinations of loads still in flight.  Rows past N in the last tile repeat the last row.
     auto load_b = [&](BBatch& t, int tile, int ks0) __attribute__((always_inline)) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            const int nrow = min((tile * NT + nt) * 16 + r, N - 1);
-            const int32_t* brow = B + (int64_t)nrow * kwords + (k0 >> 3) + 4 * g;
+            const int rowbase = (tile * NT + nt) * 16;
+            const uint32_t lo = (uint32_t)min(r, N - 1 - rowbase) * (uint32_t)(kwords * 4) + 16u * (uint32_t)g;
+            const char* tb = (const char*)B + ((int64_t)rowbase * kwords + (k0 >> 3)) * 4;
 #pragma unroll
-            for (int u = 0; u < U; ++u) t.w[nt][u] = *(const v4i*)(brow + clamp_step(step_of(ks0, u)) * 16);
+            for (int u = 0; u < U; ++u) t.w[nt][u] = *(const v4i*)(tb + (int64_t)clamp_step(step_of(ks0, u)) * 64 + lo);
         }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            const int nrow = min((tile * NT + nt) * 16 + r, N - 1);
-            const unsigned short* srow = (const unsigned short*)S + (int64_t)nrow * ngroups;
+            const int rowbase = (tile * NT + nt) * 16;
+            const uint32_t lo = (uint32_t)min(r, N - 1 - rowbase) * (uint32_t)(ngroups * 2);
+            const char* sb = (const char*)S + (int64_t)rowbase * ngroups * 2;
             if constexpr (VS) {
                 static_assert(U == 4, "four scales per load");
-                const uint2 q = *(const uint2*)(srow + (k0 >> 7) + min(step_of(ks0, 0), steps - U));
-                t.s[nt][0] = (unsigned short)q.x; t.s[nt][1] = (unsigned short)(q.x >> 16);
-                t.s[nt][2] = (unsigned short)q.y; t.s[nt][3] = (unsigned short)(q.y >> 16);
+                t.sv[nt] = *(const uint2*)(sb + (int64_t)((k0 >> 7) + min(step_of(ks0, 0), steps - U)) * 2 + lo);
             } else {
 #pragma unroll
-                for (int u = 0; u < U; ++u) t.s[nt][u] = srow[(k0 + clamp_step(step_of(ks0, u)) * 128) / groupsize];
+                for (int u = 0; u < U; ++u)
+                    t.s[nt][u] = *(const unsigned short*)(sb + (int64_t)((k0 + clamp_step(step_of(ks0, u)) * 128) / groupsize) * 2 + lo);
             }
         }
     };
@@ -421,7 +428,10 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
             const bool valid = step_of(ks0, u) < steps;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const float sc = valid ? f16_to_f32(tb.s[nt][u]) : 0.f;
+                unsigned short sraw;
+                if constexpr (VS) sraw = (unsigned short)((u < 2 ? tb.sv[nt].x : tb.sv[nt].y) >> (16 * (u & 1)));
+                else sraw = tb.s[nt][u];
+                const float sc = valid ? f16_to_f32(sraw) : 0.f;
                 v4f t[MT];
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) t[mt] = (v4f){0.f, 0.f, 0.f, 0.f};
@@ -446,11 +456,14 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     const int stride = gridDim.x;
     ABatch acur, anxt;
     BBatch bcur, bnxt, bnx2;
+    // Every load of the ring is issued unconditionally (a tile index past the end is clamped to the last tile,
+    // whose lines are then in cache): with loads under a condition the compiler cannot tell how many are in
+    // flight and waits for all of them, the one just requested included, before it touches any.
     if (tile < ntiles) {
         // activations first (mostly L2 hits): they are permuted while the weights are still on their way
         load_a(acur, wave);
         load_b(bcur, tile, wave);
-        if (RESIDENT && tile + stride < ntiles) load_b(bnxt, tile + stride, wave);
+        if (RESIDENT) load_b(bnxt, min(tile + stride, ntiles - 1), wave);
         __builtin_amdgcn_sched_barrier(0);
         if (RESIDENT) perm_a(acur);
     }
@@ -490,8 +503,7 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     // would wait for them).
     if constexpr (RESIDENT) {
         auto one = [&](BBatch& cur, BBatch& fill) __attribute__((always_inline)) {
-            const int t2 = tile + 2 * stride;
-            if (t2 < ntiles) load_b(fill, t2, wave);
+            load_b(fill, min(tile + 2 * stride, ntiles - 1), wave);
             mul(acur, cur, wave, acc);
             finish(tile);
             tile += stride;
@@ -526,6 +538,161 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
     }
 }
 
+// Ring variant of the weight-streaming kernel for 128-wide groups, at most 16 rows per workgroup and a K range
+// of at most 32 steps (steps % 4 == 0): wave w owns the four consecutive 128-K steps 4w .. 4w + 3 of every
+// 16-column tile, its activation fragments stay in registers, and the packed words and group scales of the
+// next DEPTH - 1 tiles are in flight in a ring of registers filled by hand-issued loads (see stream_ring.hpp:
+// one s_waitcnt per tile that leaves exactly the younger tiles outstanding).
+template <int DEPTH>
+__global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
+    const _Float16* __restrict__ A, const int32_t* __restrict__ B, const _Float16* __restrict__ S,
+    _Float16* __restrict__ C, int M, int N, int Kfull, int Kc, float* __restrict__ partial) {
+    using namespace llmk;
+    constexpr int NW = 8, LPT = 5;                       // loads per tile and lane: four word vectors + the scales
+    extern __shared__ float red[];                       // [2][NW][64][4]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int k0 = (int)blockIdx.z * Kc, K = min(Kc, Kfull - k0);
+    const int steps = K >> 7, ngroups = Kfull >> 7, kwords = Kfull >> 3;
+    const int m0 = blockIdx.y * 16;
+    const int ntiles = (N + 15) >> 4;
+    const bool wvalid = 4 * wave < steps;                // waves past the K range multiply by zero scales
+    const int s0 = wvalid ? 4 * wave : 0;                // first step of this wave
+
+    // ---- activations, requested first: row i of the wave's K slice (512 elements = 1 KiB) is one fully
+    // coalesced load.  (Fetching the MFMA fragments straight from global memory costs 2 us per launch: every
+    // 16-lane group of such a load touches 16 different cache lines, 16 bytes of each.)  They pass through a
+    // wave-private LDS area once and stay in registers as fragments for every tile.
+    v4i a[16];
+    {
+        // load 4 u + q: rows 4 q .. 4 q + 3 of the 256-byte slab of step u (a 16-lane group reads 256 contiguous bytes)
+        const char* ab = (const char*)A + ((int64_t)k0 + s0 * 128) * 2;
+        const uint32_t rowb = (uint32_t)(Kfull * 2), lrow = (uint32_t)(lane >> 4), lcol = 16u * (uint32_t)(lane & 15);
+#define LLMK_LDA(u, q) a[4 * u + q] = ring_load_b128<u * 256>((uint32_t)min(m0 + 4 * q + (int)lrow, M - 1) * rowb + lcol, ab)
+        LLMK_LDA(0, 0); LLMK_LDA(0, 1); LLMK_LDA(0, 2); LLMK_LDA(0, 3);
+        LLMK_LDA(1, 0); LLMK_LDA(1, 1); LLMK_LDA(1, 2); LLMK_LDA(1, 3);
+        LLMK_LDA(2, 0); LLMK_LDA(2, 1); LLMK_LDA(2, 2); LLMK_LDA(2, 3);
+        LLMK_LDA(3, 0); LLMK_LDA(3, 1); LLMK_LDA(3, 2); LLMK_LDA(3, 3);
+#undef LLMK_LDA
+    }
+    // ---- ring of weight tiles
+    v4i w[DEPTH][4];
+    v2i sv[DEPTH];
+    const char* bb = (const char*)B + ((int64_t)(k0 >> 3) + s0 * 16) * 4;
+    const char* sb = (const char*)S + ((int64_t)(k0 >> 7) + s0) * 2;
+    auto issue = [&](v4i (&tw)[4], v2i& ts, int tile) __attribute__((always_inline)) {
+        const int rowbase = tile * 16;
+        const uint32_t row = (uint32_t)min(r, N - 1 - rowbase);             // rows past N repeat the last row
+        const uint32_t vo = row * (uint32_t)(kwords * 4) + 16u * (uint32_t)g;
+        const char* tb = bb + (int64_t)rowbase * kwords * 4;
+        tw[0] = ring_load_b128<0>(vo, tb);
+        tw[1] = ring_load_b128<64>(vo, tb);
+        tw[2] = ring_load_b128<128>(vo, tb);
+        tw[3] = ring_load_b128<192>(vo, tb);
+        ts = ring_load_b64<0>(row * (uint32_t)(ngroups * 2), sb + (int64_t)rowbase * ngroups * 2);
+    };
+    int tile = blockIdx.x;
+    const int stride = gridDim.x, last = ntiles - 1;
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; ++d) issue(w[d], sv[d], min(tile + d * stride, last));
+    // the activations were requested before (DEPTH - 1) * LPT ring loads
+    ring_wait16<(DEPTH - 1) * LPT>(a);
+    {
+        // one slab (16 rows x 256 bytes) at a time through the wave's LDS area; rows of 256 + 16 bytes, so that
+        // the 16 rows of a fragment read fall into 16 different bank groups
+        constexpr int AROW = 256 + 16;
+        uint8_t* stage = (uint8_t*)red + 2 * NW * 256 * sizeof(float) + wave * (16 * AROW);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *(v4i*)(stage + (4 * q + (lane >> 4)) * AROW + 16 * (lane & 15)) = a[4 * u + q];
+            // fragment (u, j) of lane (r, g): elements 128 u + 32 g + 8 j .. + 7 of row r.  The k order of a
+            // dequantised word is [0,4,1,5,2,6,3,7]: bring the activation fragment into the same order.
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v4i x = *(const v4i*)(stage + r * AROW + 64 * g + 16 * j);
+                v4i y;
+                y[0] = (int)__builtin_amdgcn_perm((unsigned)x[2], (unsigned)x[0], 0x05040100u);
+                y[1] = (int)__builtin_amdgcn_perm((unsigned)x[2], (unsigned)x[0], 0x07060302u);
+                y[2] = (int)__builtin_amdgcn_perm((unsigned)x[3], (unsigned)x[1], 0x05040100u);
+                y[3] = (int)__builtin_amdgcn_perm((unsigned)x[3], (unsigned)x[1], 0x07060302u);
+                a[4 * u + j] = y;
+            }
+        }
+    }
+
+    int parity = 0;
+    auto tile_done = [&](const v4i (&tw)[4], const v2i& ts, int tl) __attribute__((always_inline)) {
+        v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const unsigned sraw = ((unsigned)(u < 2 ? ts[0] : ts[1]) >> (16 * (u & 1))) & 0xffffu;
+            const float sc = wvalid ? f16_to_f32((unsigned short)sraw) : 0.f;
+            v4f t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const unsigned x = (unsigned)tw[u][j], x8 = x >> 8;
+                const v8h bf = make8(deq_lo(x), deq_hi(x), deq_lo(x8), deq_hi(x8));
+                v8h af;
+                __builtin_memcpy(&af, &a[4 * u + j], 16);
+                t = mfma_f16_16x16x32(af, bf, t);
+            }
+            acc += t * sc;
+        }
+        // cross-wave reduction of the K split, two alternating buffers: one barrier per tile
+        float* rbuf = red + parity * NW * 256;
+        parity ^= 1;
+        *(v4f*)(rbuf + (wave * 64 + lane) * 4) = acc;
+        __syncthreads();
+        const int o = threadIdx.x;
+        if (o < 256) {
+            const int row16 = o >> 4, col = o & 15;
+            const int src = ((row16 >> 2) * 16 + col) * 4 + (row16 & 3);
+            const int m = m0 + row16, n = tl * 16 + col;
+            float v = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) v += rbuf[ww * 256 + src];
+            if (m < M && n < N) {
+                if (partial) partial[((int64_t)blockIdx.z * M + m) * N + n] = v;
+                else C[(int64_t)m * N + n] = (_Float16)v;
+            }
+        }
+    };
+    // (the loop is left behind a full wait: no path of the flow graph may lead from a request back to the loop
+    // head without passing a wait that covers it, and the clamped requests of the last tiles are drained)
+    // Whole rounds of DEPTH tiles run in a loop whose body has no branch (every request and every wait is
+    // executed on every path, so what the static check of the assembly sees is what runs); the last
+    // my_tiles % DEPTH tiles, all requested by then, follow as straight-line code.  Requests past the last tile
+    // of the workgroup are clamped to the last tile of the matrix (cache hits) and never consumed.
+    const int my_tiles = (ntiles - (int)blockIdx.x + stride - 1) / stride;
+    auto slot = [&](auto dc) __attribute__((always_inline)) {
+        constexpr int d = decltype(dc)::value, NEXT = DEPTH - 1;
+        issue(w[(d + NEXT) % DEPTH], sv[(d + NEXT) % DEPTH], min(tile + NEXT * stride, last));
+        ring_wait<(DEPTH - 1) * LPT>(w[d][0], w[d][1], w[d][2], w[d][3], sv[d]);
+        tile_done(w[d], sv[d], tile);
+        tile += stride;
+    };
+    auto tail = [&](auto dc) __attribute__((always_inline)) {
+        constexpr int d = decltype(dc)::value;
+        ring_wait<(DEPTH - 2 - d) * LPT>(w[d][0], w[d][1], w[d][2], w[d][3], sv[d]);
+        tile_done(w[d], sv[d], tile);
+        tile += stride;
+    };
+    static_assert(DEPTH >= 2 && DEPTH <= 4, "ring slots are spelled out below");
+    for (int rd = my_tiles / DEPTH; rd > 0; --rd) {
+        slot(std::integral_constant<int, 0>{});
+        if constexpr (DEPTH > 1) slot(std::integral_constant<int, 1>{});
+        if constexpr (DEPTH > 2) slot(std::integral_constant<int, 2>{});
+        if constexpr (DEPTH > 3) slot(std::integral_constant<int, 3>{});
+    }
+    const int rem = my_tiles % DEPTH;
+    if constexpr (DEPTH > 1) { if (rem > 0) tail(std::integral_constant<int, 0>{}); }
+    if constexpr (DEPTH > 2) { if (rem > 1) tail(std::integral_constant<int, 1>{}); }
+    if constexpr (DEPTH > 3) { if (rem > 2) tail(std::integral_constant<int, 2>{}); }
+    ring_drain<0>();
+}
+
 template <int MT, int NT>
 int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Float16* C, int M, int N, int K, int groupsize,
                      int nz, float* partial, hipStream_t st) {
@@ -554,9 +721,27 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
     dim3 grid((unsigned)gx, (unsigned)mtiles, (unsigned)nz);
     float* part = nz > 1 ? partial : nullptr;
     bool launched = false;
+    if constexpr (MT == 1 && NT == 1) {
+        // 128-wide groups, resident activations, whole four-step shares: the ring kernel
+        if (groupsize == 128 && resident && steps_all % 4 == 0 && steps % 4 == 0 && !(((uintptr_t)S) & 7) &&
+            (int64_t)N * (K / 2) < (1ll << 32) && (int64_t)M * K * 2 < (1ll << 32)) {
+            // One workgroup per CU and row tile, ring depth = tiles per workgroup (two to four).  Two workgroups
+            // per CU with rings of two measured slower (20.4 vs 18.2 us at N = 28672): every workgroup reads all
+            // the activations of its row tile, and that traffic doubles.
+            const int wg = min(ntiles, max(1, 256 / min(rows, 256)));
+            const int per_wg = (ntiles + wg - 1) / wg;
+            dim3 rgrid((unsigned)((ntiles + per_wg - 1) / per_wg), (unsigned)mtiles, (unsigned)nz);
+            // reduction buffers + the wave-private staging area of the activations
+            const size_t rsmem = 2 * 8 * 256 * sizeof(float) + 8 * 16 * (256 + 16);
+            if (per_wg >= 4) w4a16_nk_ring_kernel<4><<<rgrid, 512, rsmem, st>>>(A, B, S, C, M, N, K, Kc, part);
+            else if (per_wg == 3) w4a16_nk_ring_kernel<3><<<rgrid, 512, rsmem, st>>>(A, B, S, C, M, N, K, Kc, part);
+            else w4a16_nk_ring_kernel<2><<<rgrid, 512, rsmem, st>>>(A, B, S, C, M, N, K, Kc, part);
+            launched = true;
+        }
+    }
     if constexpr (U == 4) {
         // consecutive steps per wave and one load for their four scales
-        if (groupsize == 128 && steps_all % 4 == 0 && steps % 4 == 0 && !(((uintptr_t)S) & 7)) {
+        if (!launched && groupsize == 128 && steps_all % 4 == 0 && steps % 4 == 0 && !(((uintptr_t)S) & 7)) {
             if (resident) w4a16_nk_stream_kernel<MT, NT, true, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize, Kc, part);
             else w4a16_nk_stream_kernel<MT, NT, false, true><<<grid, 512, smem, st>>>(A, B, S, C, M, N, K, groupsize, Kc, part);
             launched = true;
