@@ -160,7 +160,8 @@ int llmk_gemm_w4a16_marlin(const void* a_f16, const int32_t* b, void* c_f16, con
                            int64_t M, int64_t N, int64_t K, int groupsize,
                            void* workspace, int64_t workspace_bytes, void* stream);
 /* Same product for W stored [N, K/8] int32 by pack_weights_over_cols (nibble i of a word = k*8+i)
- * with s fp16 [N, K/g]; a/c fp16 or bf16 (dtype code).  fp16 only at present.  workspace is optional:
+ * with s fp16 [N, K/g]; a/c fp16 or bf16 (ac_dtype; bf16: M <= 64 with 128-wide groups streams the weights,
+ * every other bf16 call multiplies a bf16 copy of W and needs the N*K*2-byte workspace).  workspace is optional for fp16:
  * M > 512 with N*K*2 bytes (16-byte aligned) runs as dequantise + tiled MFMA GEMM; 64 < M <= 512 (and
  * 32 < M <= 64 with large weights) runs on tile kernels that expand the packed words themselves and use
  * up to 8*M*N*4 bytes for split-K partial sums; M <= 64, K > 4096 with ceil(K/4096)*M*N*4 bytes runs as

@@ -330,6 +330,24 @@ __global__ void nk_dequant_kernel(const int32_t* __restrict__ B, const _Float16*
     *(v4i*)(W + n * K + k) = o;
 }
 
+// The same for bf16 operands: (q - 8) * s formed in fp32 and rounded once to bf16, natural k order.
+__global__ void nk_dequant_bf16_kernel(const int32_t* __restrict__ B, const _Float16* __restrict__ S,
+                                       unsigned short* __restrict__ W, int64_t N, int64_t K, int groupsize) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t kw = K >> 3;
+    if (idx >= N * kw) return;
+    const int64_t n = idx / kw, k = (idx - n * kw) * 8;
+    const unsigned w = (unsigned)B[idx];
+    const float sc = (float)S[n * (K / groupsize) + k / groupsize];
+    v4i o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float lo = (float)((int)((w >> (8 * i)) & 15u) - 8) * sc, hi = (float)((int)((w >> (8 * i + 4)) & 15u) - 8) * sc;
+        o[i] = (int)pack_bf16x2(lo, hi);
+    }
+    *(v4i*)(W + n * K + k) = o;
+}
+
 // Weight-streaming variant of the [N, K/8] kernel for groupsize % 128 == 0 (every 128-K step lies in one
 // scale group): persistent workgroups of 8 waves walk 16-column tiles; the waves split K by interleaved
 // 128-K steps in batches of U, all loads of a batch issued before its first use and the weights of the next
@@ -543,10 +561,14 @@ __global__ __launch_bounds__(512) void w4a16_nk_stream_kernel(
 // 16-column tile, its activation fragments stay in registers, and the packed words and group scales of the
 // next DEPTH - 1 tiles are in flight in a ring of registers filled by hand-issued loads (see stream_ring.hpp:
 // one s_waitcnt per tile that leaves exactly the younger tiles outstanding).
-template <int DEPTH>
+// BF: bf16 activations and outputs.  A nibble becomes the bf16 number 128 + q by OR-ing it into 0x4300 (exact:
+// seven mantissa bits, q < 16), and the missing "- 136" of every product is the accumulator the MFMA chain of a
+// step starts from: -136 * sum_k a[m][k] over the step, computed once per wave with the same MFMA and a weight
+// fragment of constant 136 (the same for every tile).
+template <int DEPTH, bool BF = false>
 __global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
-    const _Float16* __restrict__ A, const int32_t* __restrict__ B, const _Float16* __restrict__ S,
-    _Float16* __restrict__ C, int M, int N, int Kfull, int Kc, float* __restrict__ partial) {
+    const unsigned short* __restrict__ A, const int32_t* __restrict__ B, const _Float16* __restrict__ S,
+    unsigned short* __restrict__ C, int M, int N, int Kfull, int Kc, float* __restrict__ partial) {
     using namespace llmk;
     constexpr int NW = 8, LPT = 5;                       // loads per tile and lane: four word vectors + the scales
     extern __shared__ float red[];                       // [2][NW][64][4]
@@ -622,6 +644,24 @@ __global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
         }
     }
 
+    // bf16: the bias of step u, -136 * sum_k a[row][k] in every column of the MFMA result
+    v4f bias[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) bias[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+    if constexpr (BF) {
+        const v4i c136 = {(int)0xc308c308u, (int)0xc308c308u, (int)0xc308c308u, (int)0xc308c308u};   // bf16 -136
+        v8bf neg136;
+        __builtin_memcpy(&neg136, &c136, 16);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v8bf af;
+                __builtin_memcpy(&af, &a[4 * u + j], 16);
+                bias[u] = mfma_bf16_16x16x32(af, neg136, bias[u]);
+            }
+    }
+
     int parity = 0;
     auto tile_done = [&](const v4i (&tw)[4], const v2i& ts, int tl) __attribute__((always_inline)) {
         v4f acc = {0.f, 0.f, 0.f, 0.f};
@@ -629,14 +669,28 @@ __global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
         for (int u = 0; u < 4; ++u) {
             const unsigned sraw = ((unsigned)(u < 2 ? ts[0] : ts[1]) >> (16 * (u & 1))) & 0xffffu;
             const float sc = wvalid ? f16_to_f32((unsigned short)sraw) : 0.f;
-            v4f t = {0.f, 0.f, 0.f, 0.f};
+            v4f t = bias[u];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const unsigned x = (unsigned)tw[u][j], x8 = x >> 8;
-                const v8h bf = make8(deq_lo(x), deq_hi(x), deq_lo(x8), deq_hi(x8));
-                v8h af;
-                __builtin_memcpy(&af, &a[4 * u + j], 16);
-                t = mfma_f16_16x16x32(af, bf, t);
+                const unsigned x = (unsigned)tw[u][j];
+                if constexpr (BF) {
+                    // element pairs (k0,k4) (k1,k5) (k2,k6) (k3,k7) of the word, as for fp16
+                    v4i bw;
+                    bw[0] = (int)((x & 0x000f000fu) | 0x43004300u);
+                    bw[1] = (int)(((x >> 4) & 0x000f000fu) | 0x43004300u);
+                    bw[2] = (int)(((x >> 8) & 0x000f000fu) | 0x43004300u);
+                    bw[3] = (int)(((x >> 12) & 0x000f000fu) | 0x43004300u);
+                    v8bf bf, af;
+                    __builtin_memcpy(&bf, &bw, 16);
+                    __builtin_memcpy(&af, &a[4 * u + j], 16);
+                    t = mfma_bf16_16x16x32(af, bf, t);
+                } else {
+                    const unsigned x8 = x >> 8;
+                    const v8h bf = make8(deq_lo(x), deq_hi(x), deq_lo(x8), deq_hi(x8));
+                    v8h af;
+                    __builtin_memcpy(&af, &a[4 * u + j], 16);
+                    t = mfma_f16_16x16x32(af, bf, t);
+                }
             }
             acc += t * sc;
         }
@@ -655,7 +709,7 @@ __global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
             for (int ww = 0; ww < NW; ++ww) v += rbuf[ww * 256 + src];
             if (m < M && n < N) {
                 if (partial) partial[((int64_t)blockIdx.z * M + m) * N + n] = v;
-                else C[(int64_t)m * N + n] = (_Float16)v;
+                else C[(int64_t)m * N + n] = BF ? f32_to_bf16(v) : f32_to_f16(v);
             }
         }
     };
@@ -693,9 +747,55 @@ __global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
     ring_drain<0>();
 }
 
+// The ring kernel takes 128-wide groups, K ranges of at most 32 steps in whole four-step shares, 8-byte aligned
+// scale rows and operands below 4 GiB (32-bit lane offsets); nz = number of K ranges.
+bool nk_ring_ok(int64_t M, int64_t N, int64_t K, int groupsize, int nz, const void* S) {
+    const int64_t steps_all = K >> 7, steps = (steps_all + nz - 1) / nz;
+    return groupsize == 128 && steps <= 32 && steps_all % 4 == 0 && steps % 4 == 0 && !(((uintptr_t)S) & 7) &&
+           N * (K / 2) < (1ll << 32) && M * K * 2 < (1ll << 32);
+}
+
+// fp16 or bf16 (bf) activations / outputs; partial: fp32 planes for nz > 1 (a summing pass follows)
+int launch_nk_ring(const void* A, const int32_t* B, const _Float16* S, void* C, int M, int N, int K, int nz, float* partial,
+                   bool bf, hipStream_t st) {
+    const int steps_all = K >> 7, steps = (steps_all + nz - 1) / nz, Kc = steps * 128;
+    const int ntiles = (N + 15) / 16, mtiles = (M + 15) / 16, rows = mtiles * nz;
+    // One workgroup per CU and row tile, ring depth = tiles per workgroup (two to four).  Two workgroups per CU
+    // with rings of two measured slower (20.4 vs 18.2 us at N = 28672): every workgroup reads all the activations
+    // of its row tile, and that traffic doubles.
+    const int wg = min(ntiles, max(1, 256 / min(rows, 256)));
+    const int per_wg = (ntiles + wg - 1) / wg;
+    dim3 rgrid((unsigned)((ntiles + per_wg - 1) / per_wg), (unsigned)mtiles, (unsigned)nz);
+    // reduction buffers + the wave-private staging area of the activations
+    const size_t rsmem = 2 * 8 * 256 * sizeof(float) + 8 * 16 * (256 + 16);
+    const unsigned short* a16 = (const unsigned short*)A;
+    unsigned short* c16 = (unsigned short*)C;
+    float* part = nz > 1 ? partial : nullptr;
+#define LLMK_RING(D)                                                                                             \
+    do {                                                                                                         \
+        if (bf) w4a16_nk_ring_kernel<D, true><<<rgrid, 512, rsmem, st>>>(a16, B, S, c16, M, N, K, Kc, part);      \
+        else w4a16_nk_ring_kernel<D, false><<<rgrid, 512, rsmem, st>>>(a16, B, S, c16, M, N, K, Kc, part);        \
+    } while (0)
+    if (per_wg >= 4) LLMK_RING(4);
+    else if (per_wg == 3) LLMK_RING(3);
+    else LLMK_RING(2);
+#undef LLMK_RING
+    LLMK_CHECK_LAUNCH("gemm_w4a16_nk(ring)");
+    if (nz > 1) {
+        const int64_t mn = (int64_t)M * N;
+        if (bf) llmk::splitk_sum_kernel<LLMK_BF16><<<(unsigned)cdiv64(cdiv64(mn, 4), 256), 256, 0, st>>>(partial, C, mn, nz);
+        else splitk_reduce_f16_kernel<<<(unsigned)cdiv64(mn, 4 * 256), 256, 0, st>>>(partial, (_Float16*)C, mn, nz);
+        LLMK_CHECK_LAUNCH("gemm_w4a16_nk(reduce)");
+    }
+    return LLMK_OK;
+}
+
 template <int MT, int NT>
 int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Float16* C, int M, int N, int K, int groupsize,
                      int nz, float* partial, hipStream_t st) {
+    if constexpr (MT == 1 && NT == 1) {
+        if (nk_ring_ok(M, N, K, groupsize, nz, S)) return launch_nk_ring(A, B, S, C, M, N, K, nz, partial, false, st);
+    }
     constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
     // nz K ranges, equally long up to one step
     const int steps_all = K >> 7, steps = (steps_all + nz - 1) / nz, Kc = steps * 128;
@@ -721,24 +821,6 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
     dim3 grid((unsigned)gx, (unsigned)mtiles, (unsigned)nz);
     float* part = nz > 1 ? partial : nullptr;
     bool launched = false;
-    if constexpr (MT == 1 && NT == 1) {
-        // 128-wide groups, resident activations, whole four-step shares: the ring kernel
-        if (groupsize == 128 && resident && steps_all % 4 == 0 && steps % 4 == 0 && !(((uintptr_t)S) & 7) &&
-            (int64_t)N * (K / 2) < (1ll << 32) && (int64_t)M * K * 2 < (1ll << 32)) {
-            // One workgroup per CU and row tile, ring depth = tiles per workgroup (two to four).  Two workgroups
-            // per CU with rings of two measured slower (20.4 vs 18.2 us at N = 28672): every workgroup reads all
-            // the activations of its row tile, and that traffic doubles.
-            const int wg = min(ntiles, max(1, 256 / min(rows, 256)));
-            const int per_wg = (ntiles + wg - 1) / wg;
-            dim3 rgrid((unsigned)((ntiles + per_wg - 1) / per_wg), (unsigned)mtiles, (unsigned)nz);
-            // reduction buffers + the wave-private staging area of the activations
-            const size_t rsmem = 2 * 8 * 256 * sizeof(float) + 8 * 16 * (256 + 16);
-            if (per_wg >= 4) w4a16_nk_ring_kernel<4><<<rgrid, 512, rsmem, st>>>(A, B, S, C, M, N, K, Kc, part);
-            else if (per_wg == 3) w4a16_nk_ring_kernel<3><<<rgrid, 512, rsmem, st>>>(A, B, S, C, M, N, K, Kc, part);
-            else w4a16_nk_ring_kernel<2><<<rgrid, 512, rsmem, st>>>(A, B, S, C, M, N, K, Kc, part);
-            launched = true;
-        }
-    }
     if constexpr (U == 4) {
         // consecutive steps per wave and one load for their four scales
         if (!launched && groupsize == 128 && steps_all % 4 == 0 && steps % 4 == 0 && !(((uintptr_t)S) & 7)) {
@@ -889,7 +971,8 @@ extern "C" int llmk_gemm_w4a16_marlin(const void* a, const int32_t* b, void* c, 
 extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* c, const void* s, int ac_dtype,
                                   int64_t M, int64_t N, int64_t K, int groupsize, void* workspace,
                                   int64_t workspace_bytes, void* stream) {
-    if (ac_dtype != LLMK_F16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a16_nk: only fp16 activations/outputs are supported (dtype code %d)", ac_dtype);
+    if (ac_dtype != LLMK_F16 && ac_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a16_nk: activations / outputs must be fp16 or bf16 (dtype code %d)", ac_dtype);
+    const bool bf = ac_dtype == LLMK_BF16;
     if (M < 0 || N < 0 || K < 0 || K % 128) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_nk: K=%lld must be a multiple of 128", (long long)K);
     if (M == 0 || N == 0) return LLMK_OK;
     if (K == 0) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a16_nk: K == 0");
@@ -903,7 +986,13 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
     const _Float16* A = (const _Float16*)a;
     const _Float16* S = (const _Float16*)s;
     _Float16* C = (_Float16*)c;
-    if (w4_tiles_expand(M, N, K, workspace, workspace_bytes) && K % 64 == 0 && groupsize % 64 == 0) {
+    // bf16: the weight-streaming ring kernel for decode sizes, everything else through the bf16 copy of W
+    const int nz_bf = (int)((K / 128 + 31) / 32);
+    const bool bf_ring = bf && M <= 64 && nk_ring_ok(M, N, K, groupsize, nz_bf, s) && !((uintptr_t)c & 7) &&
+                         (nz_bf == 1 || ((M * N) % 4 == 0 && workspace && workspace_bytes >= (int64_t)nz_bf * M * N * 4 &&
+                                         !((uintptr_t)workspace & 15)));
+    if (bf_ring) return launch_nk_ring(a, b_packed, S, c, (int)M, (int)N, (int)K, nz_bf, (float*)workspace, true, st);
+    if (!bf && w4_tiles_expand(M, N, K, workspace, workspace_bytes) && K % 64 == 0 && groupsize % 64 == 0) {
         // mid-size M: the 128-column tile kernels expand the packed words themselves (every weight byte is
         // read once; the separate expansion pass would write and re-read four times as much).  Measured
         // against the two-pass path: 1.3-2.8x faster up to M = 256, even to 1.4x at 512, slower from 2048
@@ -914,19 +1003,25 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
         if (llmk::dma_eligible(p, 2))
             return llmk::launch_big_half<llmk::K_W4NK, false>(p, st, "gemm_w4a16_nk(fused tiles)", workspace, workspace_bytes);
     }
-    if (M > 64 && K % 64 == 0 && workspace && workspace_bytes >= N * K * 2 && !((uintptr_t)workspace & 15)) {
-        // compute-bound: expand W once to fp16 [N, K], then run the tiled MFMA GEMM on it
+    if ((M > 64 || bf) && K % 64 == 0 && workspace && workspace_bytes >= N * K * 2 && !((uintptr_t)workspace & 15)) {
+        // compute-bound: expand W once to fp16 / bf16 [N, K], then run the tiled MFMA GEMM on it
         llmk::DirectArgs p{};
-        p.a = (const uint8_t*)a; p.b = (const uint8_t*)workspace; p.c = c; p.c_dtype = LLMK_F16;
+        p.a = (const uint8_t*)a; p.b = (const uint8_t*)workspace; p.c = c; p.c_dtype = ac_dtype;
         p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
         if (llmk::dma_eligible(p, 2)) {
-            nk_dequant_kernel<<<(unsigned)cdiv64(N * (K / 8), 256), 256, 0, st>>>(b_packed, S, (_Float16*)workspace, N, K, groupsize);
+            const unsigned blocks = (unsigned)cdiv64(N * (K / 8), 256);
+            if (bf) nk_dequant_bf16_kernel<<<blocks, 256, 0, st>>>(b_packed, S, (unsigned short*)workspace, N, K, groupsize);
+            else nk_dequant_kernel<<<blocks, 256, 0, st>>>(b_packed, S, (_Float16*)workspace, N, K, groupsize);
             LLMK_CHECK_LAUNCH("gemm_w4a16_nk(dequant)");
             const int64_t used = (N * K * 2 + 255) & ~(int64_t)255;
-            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_nk(tiled)", (uint8_t*)workspace + used,
-                                                             workspace_bytes > used ? workspace_bytes - used : 0);
+            void* rest = (uint8_t*)workspace + used;
+            const int64_t rest_bytes = workspace_bytes > used ? workspace_bytes - used : 0;
+            if (bf) return llmk::launch_big_half<llmk::K_BF16, false>(p, st, "gemm_w4a16_nk(tiled, bf16)", rest, rest_bytes);
+            return llmk::launch_big_half<llmk::K_F16, false>(p, st, "gemm_w4a16_nk(tiled)", rest, rest_bytes);
         }
     }
+    if (bf) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a16_nk: this bf16 call needs a 16-byte aligned workspace of N*K*2 = %lld bytes (bf16 copy of W)",
+                      (long long)(N * K * 2));
     if (groupsize % 128 == 0 && M <= 64) {
         // one 16-column block per tile: two blocks per tile (NT = 2) measured slower at every shape tried.
         // While the activations of a 16-row workgroup stay resident (K <= 4096), such workgroups side by side

@@ -27,7 +27,8 @@ def quantize_nk(w: torch.Tensor, group_size: int = 128):
 
 
 def w4a16_gemm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, group_size: int = 128):
-    """y[..., n] = sum_k x[..., k] * (nibble(n, k) - 8) * scales[n, k // group_size]; fp16 in / out."""
+    """y[..., n] = sum_k x[..., k] * (nibble(n, k) - 8) * scales[n, k // group_size]; fp16 or bf16 in / out
+    (the dtype of x), fp16 scales."""
     assert x.is_contiguous() and w_packed.is_contiguous() and scales.is_contiguous(), 'Input tensors must be contiguous'
     assert w_packed.dtype == torch.int32 and scales.dtype == torch.float16
     _lib.require_gpu(x, w_packed, scales)
@@ -36,8 +37,13 @@ def w4a16_gemm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, gr
     N = w_packed.size(0)
     assert w_packed.size(1) * 8 == K, 'packed weight must be [N, K/8]'
     y = x.new_empty(*x.size()[:-1], N)
-    if M > 64:
-        # fp16 copy of W for the compute-bound path, split-K partials behind it for mid-size M
+    assert x.dtype in (torch.float16, torch.bfloat16), 'activations must be fp16 or bf16'
+    steps, nz = K // 128, -(-(K // 128) // 32)
+    # bf16 at decode size runs on the weight-streaming kernel when its K ranges come in whole four-step shares
+    bf_decode = (x.dtype == torch.bfloat16 and M <= 64 and group_size == 128 and steps % 4 == 0
+                 and (-(-steps // nz)) % 4 == 0 and scales.data_ptr() % 8 == 0)
+    if M > 64 or (x.dtype == torch.bfloat16 and not bf_decode):
+        # fp16 / bf16 copy of W for the compute-bound path, split-K partials behind it for mid-size M
         ws = _lib.workspace(x.device, ((N * K * 2 + 255) // 256) * 256 + (8 * M * N * 4 if M <= 512 else 0))
     elif K > 4096 or M > 16:
         ws = _lib.workspace(x.device, max(8, -(-K // 4096)) * M * N * 4)   # fp32 partial sums of K ranges / K slices

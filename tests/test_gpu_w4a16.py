@@ -233,3 +233,37 @@ def test_w4a16_without_scratch(dev, M, N, K):
         _lib.call("llmk_gemm_w4a16_marlin", _lib.ptr(Ad), _lib.ptr(Bd), _lib.ptr(C), _lib.ptr(spd),
                   M, N, K, 128, None, 0, _lib.stream(Ad))
         assert_close_scaled(C, g.w4a16_gemm(A, q4, sm, 128), what="marlin without scratch")
+
+
+@pytest.mark.parametrize("M,N,K,gs", [(16, 4096, 4096, 128), (1, 256, 512, 128), (7, 1000, 1024, 128), (40, 520, 2048, 128),
+                                      (16, 28672, 4096, 128), (16, 1032, 14336, 128), (64, 264, 8192, 128),
+                                      (16, 256, 384, 128), (33, 300, 4608, 128), (16, 512, 1024, 64), (20, 129, 512, 256),
+                                      (300, 1000, 512, 128), (2048, 4096, 1024, 128)])
+def test_w4a16_nk_bf16(dev, M, N, K, gs):
+    """bf16 activations / outputs for the [N, K/8] layout: the weight-streaming kernel at decode sizes (128-wide
+    groups, whole four-step K shares), the bf16 copy of W plus the bf16 tile GEMM everywhere else."""
+    announce("w4a16 nk bf16", M, N, K, gs)
+    torch.manual_seed(2)
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    qn, s = q.w4a16_quant_nk(w, gs)
+    packed, _ = bp.pack_cols(qn.numpy(), 4, 32)
+    y = w4a16.w4a16_gemm(x.to(dev), torch.from_numpy(packed).to(dev), s.to(dev), gs)
+    assert y.dtype == torch.bfloat16 and y.shape == (M, N)
+    deq = (qn.double() - 8) * s.double().repeat_interleave(gs, 1)            # [N, K], exact
+    assert_close_scaled(y, x.double() @ deq.T, what="w4a16 nk bf16")
+
+
+def test_w4a16_nk_bf16_decode_is_exact_for_small_integers(dev):
+    """Integer activations, unit scales: the bf16 decode kernel (nibbles as 128 + q, the -136 * sum(a) bias in the
+    accumulator) returns the exact integer product wherever it is representable in bf16."""
+    announce("w4a16 nk bf16 exact")
+    torch.manual_seed(3)
+    M, N, K = 16, 512, 1024
+    x = torch.randint(-2, 3, (M, K)).float()
+    qn = torch.randint(0, 16, (N, K), dtype=torch.uint8)
+    s = torch.ones(N, K // 128, dtype=torch.float16)
+    packed, _ = bp.pack_cols(qn.numpy(), 4, 32)
+    y = w4a16.w4a16_gemm(x.bfloat16().to(dev), torch.from_numpy(packed).to(dev), s.to(dev), 128)
+    ref = x.double() @ (qn.double() - 8).T
+    assert torch.equal(y.cpu().double(), ref.bfloat16().double())
