@@ -12,7 +12,21 @@ property on the generated assembly, for every path of the control-flow graph:
   among themselves, so the load has then landed; stores are not counted, they may complete at any time).
 
 It also refuses kernels with register spills or a private (scratch) segment among those that contain such
-loads.  build.py runs it on every source and fails the build when it does not hold.
+loads.
+
+A second property concerns the scalar registers such an instruction reads (its base address).  A vector-memory
+instruction needs five wait states after a VALU instruction (v_readfirstlane_b32, v_readlane_b32, a compare or a
+carry-out) wrote a scalar register it reads; the hardware does not interlock.  The compiler inserts the wait
+states for the instructions it emits and cannot see into an asm statement, so:
+
+  for every VALU instruction that writes scalar registers, on every path of fewer than five wait states from it
+  (an instruction is one wait state, `s_nop n` is n + 1): no vector-memory instruction between `;;#ASMSTART` /
+  `;;#ASMEND` reads one of those registers.
+
+Likewise a direct-to-LDS load reads M0 (its LDS base) and needs one wait state after a scalar write to M0: an
+asm `..._lds_...` load must not come right after the instruction that writes m0.
+
+build.py runs these checks on every source and fails the build when one does not hold.
 """
 import re
 import sys
@@ -87,11 +101,93 @@ def _is_vm(op):
     return op.startswith(_VM_PREFIX)
 
 
+_SREG1 = re.compile(r"\bs(\d+)\b")
+_SREGR = re.compile(r"\bs\[(\d+):(\d+)\]")
+_VM_ANY = ("global_", "buffer_", "flat_", "scratch_")
+_VALU_SGPR_WAIT_STATES = 5
+# VALU instructions whose SECOND operand is a scalar destination (carry-out / scale flag)
+_SDST_SECOND = ("v_mad_u64_u32", "v_mad_i64_i32", "v_add_co_u32", "v_sub_co_u32", "v_subrev_co_u32", "v_addc_co_u32",
+                "v_subb_co_u32", "v_subbrev_co_u32", "v_div_scale_f32", "v_div_scale_f64")
+
+
+def _sregs(text):
+    out = set("s%d" % int(m) for m in _SREG1.findall(text))
+    for a, b in _SREGR.findall(text):
+        out.update("s%d" % i for i in range(int(a), int(b) + 1))
+    if re.search(r"\bvcc\b", text):
+        out.update(("vcc_lo", "vcc_hi"))
+    out.update(re.findall(r"\bvcc_(?:lo|hi)\b", text))
+    return out
+
+
+def _valu_sgpr_writes(op, args):
+    """Scalar registers a VALU instruction writes (empty for everything else)."""
+    if not op.startswith("v_"):
+        return set()
+    ops = [a.strip() for a in args.split(",")]
+    out = set()
+    if ops and not ops[0].startswith(("v", "a")):
+        out |= _sregs(ops[0])
+    if op.startswith(_SDST_SECOND) and len(ops) > 1:
+        out |= _sregs(ops[1])
+    return out
+
+
+def _check_scalar_settle(f, problems):
+    """No asm vector-memory instruction reads a scalar register within five wait states of a VALU write to it."""
+    checked = 0
+    for i in range(1, len(f.ins)):
+        op, args, in_asm = f.ins[i]
+        pop, pargs, _ = f.ins[i - 1]
+        if in_asm and op.startswith(_VM_ANY) and "_lds_" in op and pop.startswith("s_") and \
+                pargs.split(",")[0].strip() == "m0":
+            problems.append("%s: asm `%s %s` reads M0 with no wait state after `%s %s`" % (f.name, op, args, pop, pargs))
+    for wi, (op, args, _) in enumerate(f.ins):
+        written = _valu_sgpr_writes(op, args)
+        if not written:
+            continue
+        seen = {}
+        stack = [(wi + 1, _VALU_SGPR_WAIT_STATES, frozenset(written))]
+        while stack:
+            i, left, live = stack.pop()
+            while left > 0 and live and i < len(f.ins):
+                if seen.get((i, live), 0) >= left:
+                    break
+                seen[(i, live)] = left
+                op2, args2, in_asm = f.ins[i]
+                if in_asm and op2.startswith(_VM_ANY):
+                    checked += 1
+                    hit = live & _sregs(args2)
+                    if hit:
+                        problems.append("%s: asm `%s %s` reads %s only %d wait states after `%s %s` wrote it (needs %d)"
+                                        % (f.name, op2, args2, sorted(hit), _VALU_SGPR_WAIT_STATES - left, op, args,
+                                           _VALU_SGPR_WAIT_STATES))
+                        break
+                if op2 == "s_endpgm":
+                    break
+                if op2.startswith("s_") and not op2.startswith(("s_cbranch", "s_branch", "s_nop", "s_waitcnt", "s_cmp",
+                                                                 "s_bitcmp", "s_barrier")):
+                    # a scalar-ALU or scalar-memory write replaces the VALU's value: interlocked from here on
+                    live = live - _sregs(args2.split(",")[0])
+                left -= (int(args2.strip() or 0) + 1) if op2 == "s_nop" else 1
+                if op2 == "s_branch":
+                    i = f.labels.get(args2.strip(), len(f.ins))
+                    continue
+                if op2.startswith("s_cbranch"):
+                    tgt = f.labels.get(args2.strip())
+                    if tgt is not None:
+                        stack.append((tgt, left, live))
+                i += 1
+    return checked
+
+
 def check_file(path):
     """Returns (number of hand-issued register loads checked, list of violation strings)."""
     funcs, meta = _parse(path)
     problems, checked = [], 0
     for f in funcs:
+        if any(in_asm and op.startswith(_VM_ANY) for op, _, in_asm in f.ins):
+            _check_scalar_settle(f, problems)
         loads = [i for i, (op, args, in_asm) in enumerate(f.ins)
                  if in_asm and op.startswith(("global_load", "buffer_load", "flat_load")) and "_lds_" not in op]
         if not loads:

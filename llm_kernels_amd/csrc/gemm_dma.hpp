@@ -29,11 +29,13 @@ constexpr int d_a(int mi) { return 64 * mi * 128; }
 constexpr int d_stage(int mi) { return d_a(mi) + D_B + D_S; }
 constexpr int d_lds(int mi) { return D_NSTAGE * d_stage(mi) + D_MAX_KT * 4; }
 
+// Direct-to-LDS loads: M0 holds the LDS base.  A load that reads M0 needs one wait state after the scalar write
+// to it, which the compiler inserts for its own instructions and not inside an asm statement: hence the s_nop.
 __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* sbase) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 __device__ __forceinline__ void dma4(uint32_t lds_addr, uint32_t voff, const void* sbase) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 // s_waitcnt immediates for gfx9: vmcnt = imm[3:0] | imm[15:14] << 4, expcnt = imm[6:4] (7 = no wait),
 // lgkmcnt = imm[11:8] (15 = no wait)

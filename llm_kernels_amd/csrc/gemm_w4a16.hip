@@ -589,7 +589,7 @@ __global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
     v4i a[16];
     {
         // load 4 u + q: rows 4 q .. 4 q + 3 of the 256-byte slab of step u (a 16-lane group reads 256 contiguous bytes)
-        const char* ab = (const char*)A + ((int64_t)k0 + s0 * 128) * 2;
+        const RingBase ab = ring_base((const char*)A + ((int64_t)k0 + s0 * 128) * 2);
         const uint32_t rowb = (uint32_t)(Kfull * 2), lrow = (uint32_t)(lane >> 4), lcol = 16u * (uint32_t)(lane & 15);
 #define LLMK_LDA(u, q) a[4 * u + q] = ring_load_b128<u * 256>((uint32_t)min(m0 + 4 * q + (int)lrow, M - 1) * rowb + lcol, ab)
         LLMK_LDA(0, 0); LLMK_LDA(0, 1); LLMK_LDA(0, 2); LLMK_LDA(0, 3);
@@ -607,12 +607,12 @@ __global__ __launch_bounds__(512) void w4a16_nk_ring_kernel(
         const int rowbase = tile * 16;
         const uint32_t row = (uint32_t)min(r, N - 1 - rowbase);             // rows past N repeat the last row
         const uint32_t vo = row * (uint32_t)(kwords * 4) + 16u * (uint32_t)g;
-        const char* tb = bb + (int64_t)rowbase * kwords * 4;
+        const RingBase tb = ring_base(bb + (int64_t)rowbase * kwords * 4);
         tw[0] = ring_load_b128<0>(vo, tb);
         tw[1] = ring_load_b128<64>(vo, tb);
         tw[2] = ring_load_b128<128>(vo, tb);
         tw[3] = ring_load_b128<192>(vo, tb);
-        ts = ring_load_b64<0>(row * (uint32_t)(ngroups * 2), sb + (int64_t)rowbase * ngroups * 2);
+        ts = ring_load_b64<0>(row * (uint32_t)(ngroups * 2), ring_base(sb + (int64_t)rowbase * ngroups * 2));
     };
     int tile = blockIdx.x;
     const int stride = gridDim.x, last = ntiles - 1;

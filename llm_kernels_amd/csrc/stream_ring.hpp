@@ -16,25 +16,47 @@
 
 namespace llmk {
 
+// The base pointer of hand-issued loads: the same in every lane, held in scalar registers, and settled.
+//
+// The compiler may carry a wave-uniform pointer in vector registers (64-bit multiplies have no scalar form, and
+// behind divergent control flow anything can end up there) and move it to scalar registers with
+// v_readfirstlane_b32 right in front of the use.  A vector-memory instruction that reads a scalar register
+// needs five wait states after a VALU instruction wrote it; the hardware does not interlock, the compiler
+// inserts them for the loads it emits itself and knows nothing about the ones inside an asm statement, which
+// would then take their base from whatever the register held before: a wild address.  ring_base() therefore
+// ends in "s_nop 4" that names both halves as read-write operands, so every load that uses the base is at
+// least five wait states behind the last VALU write to it.  The loads take nothing but a RingBase, and
+// check_asm.py proves the distance on the assembly of every build.
+struct RingBase {
+    const void* p;
+};
+__device__ __forceinline__ RingBase ring_base(const void* p) {
+    const uint64_t u = (uint64_t)(uintptr_t)p;
+    uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)u);
+    uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
+    asm volatile("s_nop 4 ; scalar base settled" : "+s"(lo), "+s"(hi));
+    return RingBase{(const void*)(uintptr_t)(((uint64_t)hi << 32) | lo)};
+}
+
 template <int IMM>
-__device__ __forceinline__ v4i ring_load_b128(uint32_t voff, const void* sbase) {
+__device__ __forceinline__ v4i ring_load_b128(uint32_t voff, RingBase base) {
     static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
     v4i v;
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(base.p), "n"(IMM) : "memory");
     return v;
 }
 template <int IMM>
-__device__ __forceinline__ v2i ring_load_b64(uint32_t voff, const void* sbase) {
+__device__ __forceinline__ v2i ring_load_b64(uint32_t voff, RingBase base) {
     static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
     v2i v;
-    asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+    asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(base.p), "n"(IMM) : "memory");
     return v;
 }
 template <int IMM>
-__device__ __forceinline__ int ring_load_b32(uint32_t voff, const void* sbase) {
+__device__ __forceinline__ int ring_load_b32(uint32_t voff, RingBase base) {
     static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
     int v;
-    asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+    asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(base.p), "n"(IMM) : "memory");
     return v;
 }
 
@@ -42,6 +64,14 @@ __device__ __forceinline__ int ring_load_b32(uint32_t voff, const void* sbase) {
 // up in the statement's text, which keeps the compiler from merging several such sites into one block.
 template <int ID>
 __device__ __forceinline__ void ring_drain() { asm volatile("s_waitcnt vmcnt(0) ; ring exit %0" ::"n"(ID) : "memory"); }
+
+template <int IMM>
+__device__ __forceinline__ int ring_load_u16(uint32_t voff, RingBase base) {
+    static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate");
+    int v;
+    asm volatile("global_load_ushort %0, %1, %2 offset:%3" : "=v"(v) : "v"(voff), "s"(base.p), "n"(IMM) : "memory");
+    return v;
+}
 
 // s_waitcnt vmcnt(N) that names the registers it releases
 template <int N>
@@ -66,6 +96,10 @@ __device__ __forceinline__ void ring_wait16(v4i (&a)[16]) {
                  : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
                    "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15])
                  : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void ring_wait(int& a) {
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void ring_wait(int& a, int& b, int& c, int& d) {

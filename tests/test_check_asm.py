@@ -1,12 +1,14 @@
 """check_asm proves, on device assembly, that nothing touches the destination of a hand-issued register load
-before a covering s_waitcnt.  Synthetic listings: the accepted pattern and each way it can go wrong."""
+before a covering s_waitcnt, and that the scalar registers such an instruction reads have settled (five wait
+states after a VALU write, one after a write to M0).  Synthetic listings: the accepted patterns and each way
+they can go wrong."""
 import os
 
 from llm_kernels_amd import check_asm
 
 HEAD = "kern:\n"
 LOAD = "\t;;#ASMSTART\n\tglobal_load_dwordx2 v[10:11], v20, s[2:3]\n\t;;#ASMEND\n"
-DMA = "\t;;#ASMSTART\n\ts_mov_b32 m0, s5\n\tglobal_load_lds_dwordx4 v21, s[6:7]\n\t;;#ASMEND\n"
+DMA = "\t;;#ASMSTART\n\ts_mov_b32 m0, s5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 v21, s[6:7]\n\t;;#ASMEND\n"
 
 
 def _check(tmp_path, body):
@@ -54,3 +56,38 @@ def test_rejects_spills_in_kernels_with_such_loads(tmp_path):
                 "amdhsa.kernels:\n  - .name:           kern\n    .private_segment_fixed_size: 64\n    .vgpr_spill_count: 3\n")
     n, bad = check_asm.check_file(p)
     assert n == 1 and len(bad) == 1 and "spilled" in bad[0]
+
+
+WAIT = "\ts_waitcnt vmcnt(0)\n"
+
+
+def test_rejects_base_read_too_soon_after_a_valu_write(tmp_path):
+    # v_readfirstlane_b32 writes s3; the load that reads s[2:3] follows with two wait states in between
+    body = "\tv_readfirstlane_b32 s3, v7\n\tv_add_u32_e32 v1, v2, v3\n\ts_mul_i32 s9, s8, s8\n" + LOAD + WAIT
+    _, bad = _check(tmp_path, body)
+    assert len(bad) == 1 and "wait states" in bad[0] and "s3" in bad[0]
+    # a carry-out is a VALU write of scalar registers as well
+    body = "\tv_mad_u64_u32 v[30:31], s[2:3], v5, s10, v[32:33]\n" + LOAD + WAIT
+    assert len(_check(tmp_path, body)[1]) == 1
+    # ... also across a branch
+    body = "\tv_readfirstlane_b32 s2, v7\n\ts_cbranch_scc1 .LBB0_2\n\ts_nop 7\n.LBB0_2:\n" + LOAD + WAIT
+    assert len(_check(tmp_path, body)[1]) == 1
+
+
+def test_accepts_settled_base(tmp_path):
+    body = "\tv_readfirstlane_b32 s2, v6\n\tv_readfirstlane_b32 s3, v7\n\t;;#ASMSTART\n\ts_nop 4 ; settled\n\t;;#ASMEND\n" + LOAD + WAIT
+    assert _check(tmp_path, body)[1] == []
+    # five ordinary instructions are five wait states
+    body = "\tv_readfirstlane_b32 s3, v7\n" + "\tv_add_u32_e32 v1, v2, v3\n" * 5 + LOAD + WAIT
+    assert _check(tmp_path, body)[1] == []
+    # a scalar-ALU write replaces the VALU's value (interlocked), and a source operand is not a write
+    body = "\tv_mad_u64_u32 v[30:31], s[2:3], v5, s10, v[32:33]\n\ts_add_u32 s2, s12, s14\n\ts_addc_u32 s3, s13, s15\n" + LOAD + WAIT
+    assert _check(tmp_path, body)[1] == []
+    body = "\tv_mul_f32_e32 v71, s2, v73\n" + LOAD + WAIT
+    assert _check(tmp_path, body)[1] == []
+
+
+def test_rejects_lds_load_right_after_the_write_to_m0(tmp_path):
+    body = "\t;;#ASMSTART\n\ts_mov_b32 m0, s5\n\tglobal_load_lds_dwordx4 v21, s[6:7]\n\t;;#ASMEND\n" + WAIT
+    _, bad = _check(tmp_path, body)
+    assert len(bad) == 1 and "M0" in bad[0]
