@@ -845,8 +845,13 @@ int launch_nk_stream(const _Float16* A, const int32_t* B, const _Float16* S, _Fl
 // 1.3-2.8x faster than the separate expansion pass up to 256 rows, even to 1.4x at 512); 33 to 64 when the
 // weight matrix is large, where the tile kernel with split-K beats the weight-streaming kernels (which read
 // the activations once per 16 columns), provided the scratch for its partial sums is there.
-bool w4_tiles_expand(int64_t M, int64_t N, int64_t K, const void* workspace, int64_t workspace_bytes) {
-    if (M > 64) return M <= 512;
+// `wide`: the layout also has the expansion inside the 256-column tile kernel (row-packed layout only).  Up to 512
+// rows the fused tile kernels win everywhere (1.3-2.8x); beyond that the fused 256 x 256 kernel wins over the
+// dequantisation pass + fp16 GEMM only when the problem takes two or more rounds of 256 tiles (4096 x 28672 x 4096:
+// 741 vs 758 us, 2048 x 14336 x 4096: 198 vs 201 us), and loses on one round (4096^3: 109 vs 105 us).
+bool w4_tiles_expand(int64_t M, int64_t N, int64_t K, const void* workspace, int64_t workspace_bytes, bool wide = false) {
+    if (M > 512) return wide && ((M + 255) / 256) * ((N + 255) / 256) >= 512;
+    if (M > 64) return true;
     if (M <= 32 || K % 64) return false;
     const int64_t nk = N * K;
     if (!(K > 4096 ? nk >= ((int64_t)32 << 20) : nk >= ((int64_t)96 << 20))) return false;
@@ -992,11 +997,9 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
                          (nz_bf == 1 || ((M * N) % 4 == 0 && workspace && workspace_bytes >= (int64_t)nz_bf * M * N * 4 &&
                                          !((uintptr_t)workspace & 15)));
     if (bf_ring) return launch_nk_ring(a, b_packed, S, c, (int)M, (int)N, (int)K, nz_bf, (float*)workspace, true, st);
-    if (!bf && w4_tiles_expand(M, N, K, workspace, workspace_bytes) && K % 64 == 0 && groupsize % 64 == 0) {
+    if (!bf && w4_tiles_expand(M, N, K, workspace, workspace_bytes, true) && K % 64 == 0 && groupsize % 64 == 0) {
         // mid-size M: the 128-column tile kernels expand the packed words themselves (every weight byte is
-        // read once; the separate expansion pass would write and re-read four times as much).  Measured
-        // against the two-pass path: 1.3-2.8x faster up to M = 256, even to 1.4x at 512, slower from 2048
-        // (no 256 x 256 tile variant).
+        // read once; the separate expansion pass would write and re-read four times as much).
         llmk::DirectArgs p{};
         p.a = (const uint8_t*)a; p.b = (const uint8_t*)b_packed; p.b_s = s; p.c = c; p.c_dtype = LLMK_F16;
         p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1; p.group = groupsize;

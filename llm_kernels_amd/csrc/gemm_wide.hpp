@@ -41,7 +41,11 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     const int r = lane & 15, g = lane >> 4;
     const int wm = wave >> 2, wn = wave & 3;
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    // 4-bit weights (fp16 activations): the weight rows of a stage are not loaded into LDS but expanded there by
+    // the threads themselves from packed words that travel HBM -> registers, see w4_request / w4_expand
+    constexpr bool W4NK = (KIND == K_W4NK), W4 = W4NK;
+    static_assert(KIND != K_W4MARLIN && !(W4 && GROUPED), "4-bit weights: row-packed layout, dense launches only");
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
     const int KT = K >> 7;
@@ -142,15 +146,81 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     }
     const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT * 4u;
 
+    // ---- 4-bit weights: a thread owns the same piece of the 128-column half h = 0, 1 of the tile as in the
+    // 128-column tile kernel (gemm_dma.hpp): per K step and half one 8-byte load of packed weights and one load
+    // of group scales, i.e. four loads per thread and stage like the four weight loads of the other kinds, so
+    // that the wait counts of the loop are the same.
+    uint32_t w4_off[2] = {0, 0}, w4_soff[2] = {0, 0}, w4_lds[2] = {0, 0};
+    if constexpr (W4NK) {
+        // thread t: quarter q = t & 3 (16 weights of the 64-element K step) of LDS row (t >> 2) + 128 h
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int Rr = (tid >> 2) + 128 * h, q = tid & 3, rho = Rr & 63;
+            const int col = (Rr & 192) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
+            const uint32_t n = (uint32_t)min(n0 + col, N - 1);
+            w4_off[h] = n * (uint32_t)(p.K >> 1) + (uint32_t)q * 8u;               // bytes into the packed matrix
+            w4_soff[h] = n * (uint32_t)(p.K / p.group) * 2u;                        // bytes into the scale matrix
+            w4_lds[h] = (uint32_t)Rr * 128u + (uint32_t)((2 * q) ^ ((Rr >> 1) & 7)) * 16u;   // chunk 2q; chunk 2q+1 is at ^16
+        }
+    }
+    // (variables of the exact register width, so that no widening move is ever placed between load and wait)
+    uint64_t w4_words[2] = {0, 0};
+    unsigned w4_scale16[2] = {0, 0};
+    auto w4_request = [&](int kt) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if constexpr (W4NK) {
+                w4_words[h] = asm_load_b64(w4_off[h], (const uint8_t*)p.b + (int64_t)kt * 32);
+                w4_scale16[h] = asm_load_u16(w4_soff[h], (const uint8_t*)p.b_s + (int64_t)((kt * 64) / p.group) * 2);
+            }
+        }
+    };
+    // the four loads of w4_request(kt) have landed when at most the AL activation loads issued after them are in
+    // flight ...
+    auto w4_wait = [&]() {
+        if constexpr (W4NK)
+            asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w4_words[0]), "+v"(w4_scale16[0]), "+v"(w4_words[1]), "+v"(w4_scale16[1]) : "n"(AL) : "memory");
+    };
+    // ... and, expanded, become the weight rows of stage kt: four pieces (half h = piece >> 1, word piece & 1),
+    // which the loop spreads over four MFMA tiles
+    auto w4_expand_piece = [&](int kt, int piece) {
+        uint8_t* bst = lds + (kt & 1) * W_STAGE + W_A;
+        const int h = piece >> 1, jj = piece & 1;
+        if constexpr (W4NK) {
+            const unsigned s16 = w4_scale16[h];
+            const v2h sc = w4_as_h2(s16 | (s16 << 16));
+            uint8_t* dst = bst + w4_lds[h];
+            if (jj == 0) *(v4i*)dst = w4_word_to_f16x8((unsigned)w4_words[h], sc);
+            else *(v4i*)(dst + ((w4_lds[h] & 16u) ? -16 : 16)) = w4_word_to_f16x8((unsigned)(w4_words[h] >> 32), sc);
+        }
+    };
+    auto w4_expand = [&](int kt) {
+        w4_wait();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int piece = 0; piece < 4; ++piece) w4_expand_piece(kt, piece);
+    };
+
+    // Nothing is in flight when the last K step begins (the step before it ended with vmcnt(0)); this wait costs
+    // nothing and puts a covering wait on every static path into that step, also on those that the trip counts
+    // rule out (a request in the loop followed by a skipped middle step), which the check of the assembly walks.
+    auto w4_drain = [&]() {
+        if constexpr (W4NK)
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(w4_words[0]), "+v"(w4_scale16[0]), "+v"(w4_words[1]), "+v"(w4_scale16[1]) : : "memory");
+    };
+
     auto issue = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
         const uint8_t* ga = p.a + (int64_t)kt * 128;
         const uint8_t* gb = bbase + (int64_t)kt * 128;
         const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
+        if constexpr (W4) w4_request(kt);          // in front of the activation loads: see w4_expand
 #pragma unroll
         for (int i = 0; i < AL; ++i) dma16(st + (uint32_t)(wave * AL + i) * 1024u, aoff[i], ga);
+        if constexpr (!W4) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(st + W_A + (uint32_t)(wave * 4 + i) * 1024u, boff[i], gb);
+            for (int i = 0; i < 4; ++i) dma16(st + W_A + (uint32_t)(wave * 4 + i) * 1024u, boff[i], gb);
+        }
         if constexpr (SCALED) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
     };
 
@@ -176,6 +246,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     if (KT > 0) issue(0);
+    if constexpr (W4) if (KT > 0) w4_expand(0);
     if constexpr (SCALED) {
         for (int i = tid; i < 2 * KT; i += W_THREADS) {
             const int c = i >= KT ? 1 : 0, kk = i - c * KT;
@@ -243,6 +314,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     auto step = [&](int kt, auto sync_c, auto issue_c, auto nr_c) {
         constexpr bool SYNC = decltype(sync_c)::value, ISSUE = decltype(issue_c)::value;
         constexpr int NR = decltype(nr_c)::value;
+        if constexpr (W4 && !SYNC) w4_drain();
         const uint8_t* As = stage_a(kt);
         float sa[R];
         if constexpr (SCALED && NR > 0) {
@@ -254,7 +326,16 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 #pragma unroll
         for (int i = 0; i < R; ++i) {
             if (i + 1 < NR) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
-            if (i == W_EARLY_ROW && ISSUE) {
+            if constexpr (W4) {
+                // 4-bit weights: the packed words of step kt + 1, requested a step ago, become the weight rows of
+                // the other stage (nobody has read those since the barrier of step kt - 1, so no barrier here),
+                // and the words of step kt + 2 are requested into the registers just freed.
+                if (i == W_EARLY_ROW && SYNC) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    w4_wait();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else if (i == W_EARLY_ROW && ISSUE) {
                 // Every wave has had its weight fragments of this step in registers since the step began, so
                 // behind this barrier the weight half of the stage may be overwritten: the weight loads of
                 // step kt + 2 go out here, the activation loads behind the barrier of row 7.  Two bursts of
@@ -280,7 +361,12 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
                 } else {
                     if (i < NR) acc[i][j] = mma_plain<KIND>(bf[j], af[i & 1], acc[i][j]);
                 }
-                if (i == W_EARLY_ROW && ISSUE) issue_b_part(kt + 2, j);
+                if constexpr (W4) {
+                    if (i == W_EARLY_ROW && SYNC) {
+                        w4_expand_piece(kt + 1, j);
+                        if (j == 3 && ISSUE) w4_request(kt + 2);
+                    }
+                } else if (i == W_EARLY_ROW && ISSUE) issue_b_part(kt + 2, j);
                 if (i == R - 1 && SYNC) {
                     if (ISSUE) issue_part(kt + 2, j);      // a quarter behind each tile (0.5-1 % faster than all at once)
                     if (NR > 0) {
@@ -374,7 +460,9 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
 template <int KIND, bool GROUPED>
 int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
     if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
-    constexpr bool HAS_WIDE = KIND != K_W4NK && KIND != K_W4MARLIN;             // the 4-bit expansion exists in the 128-column kernels only
+    // 4-bit weights: the row-packed layout, dense launches (the Marlin scatter of 2-byte pieces measured 4-9 % slower
+    // inside the 256-column kernel than the dequantisation pass at every M > 512)
+    constexpr bool HAS_WIDE = KIND != K_W4MARLIN && !(GROUPED && KIND == K_W4NK);
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
     // a segment of a grouped GEMM rarely ends on a tile boundary: count one ragged tile per segment on top of

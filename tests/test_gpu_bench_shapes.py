@@ -195,9 +195,11 @@ def test_mul_bench_shapes(dev, M, N, K):
     assert (C[rows.to(dev)].cpu().double() - ref).abs().max() <= 0.05
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 4096, 4096), (128, 28672, 4096), (16, 128256, 4096)])
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 4096), (128, 28672, 4096), (16, 128256, 4096), (4096, 14336, 4096),
+                                   (2048, 28672, 4096)])
 def test_w4a16_nk_bench_shapes(dev, M, N, K):
-    """Configuration 1 layout ([N, K/8] bit-packed, s = absmax / 7) at M = 4096 and the widest weights."""
+    """Configuration 1 layout ([N, K/8] bit-packed, s = absmax / 7) at M = 4096 and the widest weights; the last two
+    take two or more rounds of 256 x 256 tiles and run on the tile kernel that expands the packed words itself."""
     announce("w4a16 nk bench shape", M, N, K)
     torch.manual_seed(1)
     x = torch.randn(M, K, device=dev).half()

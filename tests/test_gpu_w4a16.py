@@ -196,6 +196,24 @@ def test_w4a16_nk_mid_m_fused_tiles(dev, M, N, K, gs):
     assert_close_scaled(y, ref, what="w4a16 nk fused tiles")
 
 
+@pytest.mark.parametrize("M,N,K,gs", [(2300, 14400, 384, 128), (4100, 8200, 128, 64), (2560, 14336, 256, 128),
+                                      (600, 61000, 640, 64)])
+def test_w4a16_nk_fused_256_column_tiles(dev, M, N, K, gs):
+    """More than 512 rows and two or more rounds of 256 x 256 tiles: the packed words are expanded inside the
+    256-column tile kernel (two, four, six and ten K steps of 64: from no steady-state step to eight; ragged rows
+    and columns; groups of one K step and of two)."""
+    announce("w4a16 nk fused 256-column tiles", M, N, K, gs)
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).half()
+    w = torch.randn(N, K) * 0.02
+    qn, s = q.w4a16_quant_nk(w, gs)
+    packed, _ = bp.pack_cols(qn.numpy(), 4, 32)
+    y = w4a16.w4a16_gemm(x.to(dev), torch.from_numpy(packed).to(dev), s.to(dev), gs)
+    assert y.dtype == torch.half and y.shape == (M, N)
+    ref = g.w4a16_gemm(x, qn.t().int().contiguous(), s.t().contiguous(), gs)
+    assert_close_scaled(y, ref, what="w4a16 nk fused 256-column tiles")
+
+
 @pytest.mark.parametrize("M,N,K,gs", [(4096, 4096, 256, 128), (3990, 4100, 384, 64), (4096, 3848, 128, 32)])
 def test_w4a16_nk_large_tile_shapes(dev, M, N, K, gs):
     announce("w4a16 nk large tiles", M, N, K, gs)
