@@ -144,3 +144,10 @@ def workspace(device, nbytes):
         buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
         _ws[key] = buf
     return buf
+
+
+def release_workspaces(device=None):
+    """Drops the cached scratch buffers (of one device, or of all): the next call that needs scratch allocates
+    again.  The memory goes back to torch's allocator once the launches that use it have run (stream-ordered)."""
+    for key in [k for k in _ws if device is None or k[0] == torch.device(device).index]:
+        del _ws[key]

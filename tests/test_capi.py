@@ -57,3 +57,19 @@ def test_product_refuses_cpu_tensors():
         fp8_kernel.act_quant(torch.randn(4, 128))
     with pytest.raises(_lib.LlmkError):
         bitpack.pack_weights_over_rows(torch.zeros(8, 8, dtype=torch.uint8), 4, 32, False)
+
+
+def test_release_workspaces_drops_the_cached_scratch():
+    saved = dict(_lib._ws)
+    try:
+        _lib._ws.clear()
+        _lib._ws[(0, 11)] = object()
+        _lib._ws[(0, 12)] = object()
+        _lib._ws[(1, 11)] = object()
+        _lib.release_workspaces("cuda:1")
+        assert sorted(_lib._ws) == [(0, 11), (0, 12)]
+        _lib.release_workspaces()
+        assert not _lib._ws
+    finally:
+        _lib._ws.clear()
+        _lib._ws.update(saved)
