@@ -166,11 +166,11 @@ class Case:
         self.flops = 2.0 * M * N * K
         self.bytes = {"fp8": _bytes_fp8, "int8": _bytes_i8, "int8_pt": _bytes_i8_pt, "w4a8": _bytes_w4a8}.get(op, None)
         self.bytes = self.bytes(M, N, K) if self.bytes else _bytes_w4a16(M, N, K)
-        self.mfma_dtype = {"fp8": "fp8", "int8": "int8", "int8_pt": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
+        self.mfma_dtype = {"fp8": "fp8", "int8": "int8", "int8_pt": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16", "w4a16_nk_bf16": "bf16"}[op]
         intensity = self.flops / self.bytes
         ridge = PEAK_TFLOPS[self.mfma_dtype] * 1e12 / (PEAK_HBM_GBS * 1e9)
         self.bound = "hbm" if intensity < ridge else "mfma"
-        self.dtype = {"fp8": "fp8_e4m3", "int8": "int8", "int8_pt": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16"}[op]
+        self.dtype = {"fp8": "fp8_e4m3", "int8": "int8", "int8_pt": "int8", "w4a8": "int8", "w4a16": "fp16", "w4a16_nk": "fp16", "w4a16_nk_bf16": "bf16"}[op]
 
     # ---- device side
     def setup(self, dev):
@@ -214,8 +214,8 @@ class Case:
             C = torch.empty(M, N, dtype=torch.half, device=dev)
             ws = torch.zeros(max(16, N // 128 * 16), dtype=torch.int32, device=dev)
             self.launch = lambda i: mul(A, Bs[i % nbuf], C, sp, ws)
-        elif op == "w4a16_nk":
-            A = x.half()
+        elif op in ("w4a16_nk", "w4a16_nk_bf16"):
+            A = x.half() if op == "w4a16_nk" else x.bfloat16()
             packed, s, _ = w4a16.quantize_nk(w, 128)
             Ps = [packed.clone() for _ in range(nbuf)]
             self.launch = lambda i: w4a16.w4a16_gemm(A, Ps[i % nbuf], s, 128)
@@ -441,7 +441,7 @@ def main():
     else:
         if args.workload not in WORKLOADS:
             # any other shape of a known operator, spelt like the registered names: <op>_m<M>_n<N>_k<K>
-            m = re.fullmatch(r"(fp8|int8|int8_pt|w4a8|w4a16|w4a16_nk)_m(\d+)_n(\d+)_k(\d+)", args.workload)
+            m = re.fullmatch(r"(fp8|int8|int8_pt|w4a8|w4a16|w4a16_nk|w4a16_nk_bf16)_m(\d+)_n(\d+)_k(\d+)", args.workload)
             if not m:
                 raise SystemExit("unknown workload %r" % args.workload)
             WORKLOADS[args.workload] = (m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4)))

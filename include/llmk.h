@@ -40,7 +40,9 @@ extern "C" {
 int         llmk_version(void);
 const char* llmk_last_error(void);
 /* Bytes of scratch llmk_gemm_fp8_block / _i8_block / _w4a8 / llmk_grouped_gemm can use for this shape
- * (0 = none).  The scratch is optional: without it a slower kernel variant runs. */
+ * (0 = none; M = all rows of a grouped launch).  The scratch is optional: without it, or with less of it, a
+ * slower kernel variant runs.  For M > 512 it ends with 64 MiB for the partial sums of a split last round of
+ * tiles. */
 int64_t     llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* ------------------------------------------------------------------ bit packing

@@ -47,7 +47,8 @@ int launch_stream(DirectArgs& p, void* workspace, int64_t workspace_bytes, hipSt
 
 }  // namespace
 
-extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+// scratch without the (fixed-size) part for a split last round of 256-column tiles
+static int64_t workspace_core_bytes(int64_t M, int64_t N, int64_t K) {
     // large-M kernels stream fp32 activation scales; 16-bit scales are widened into the workspace first;
     // mid-size M with few tiles adds the fp32 split-K partials behind them
     if (K <= 0) return 0;
@@ -58,6 +59,11 @@ extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const int64_t scales = (M * (K / 128) * 4 + 255) & ~(int64_t)255;
     const int z = splitk_factor(M, N, K);
     return scales + (z > 1 ? (int64_t)z * M * N * 4 : 0);
+}
+
+extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    // more than 512 rows: room for the partial sums of a split last round of 256-column tiles behind the rest
+    return workspace_core_bytes(M, N, K) + (K > 0 && M > 512 ? w_tail_bytes() : 0);
 }
 
 extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
@@ -143,7 +149,9 @@ extern "C" int llmk_gemm_fp8_block_static(const void* a, const float* a_s, const
                                           int c_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
     int rc = check_common("gemm_fp8_block_static", a, b, M, N, K, c_dtype);
     if (rc) return rc;
-    const int64_t need = llmk_gemm_workspace_bytes(M, N, K);
+    // (the built-in array serves the scratch a shape cannot do without efficiently; the optional partial sums of a
+    // split last round of tiles, 64 MiB, are left out: large shapes run unsplit here)
+    const int64_t need = workspace_core_bytes(M, N, K);
     if (need > (int64_t)LLMK_STATIC_SCRATCH_BYTES)
         LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_fp8_block_static: M=%lld N=%lld K=%lld needs %lld bytes of scratch, the built-in "
                   "buffer holds %lld; use llmk_gemm_fp8_block with a caller-provided workspace",

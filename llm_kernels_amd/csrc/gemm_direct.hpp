@@ -98,6 +98,7 @@ struct DirectArgs {
     int ksplit;            // 0 / 1 = no split
     int kc_steps;          // weight-streaming kernel with K ranges: 128-byte steps per range (gridDim.z ranges)
     int group;             // K_W4NK / K_W4MARLIN: K elements per fp16 group scale
+    int tail_split;        // 256-column tile kernel: the tiles of a short last round are split along K (partial = scratch)
 };
 
 // Upper bound of the row tiles of a grouped GEMM (segment ends are only known on the device): every segment

@@ -28,6 +28,129 @@ constexpr int w_bm(int r) { return 32 * r; }
 constexpr int w_stage(int r) { return w_bm(r) * 128 + W_B + W_S; }        // 66560 / 50176
 constexpr int w_lds(int r) { return 2 * w_stage(r) + 2 * D_MAX_KT * 4; }  // 135168 / 102400 bytes
 
+// ---- which tile a workgroup works on.  `lin` = linear workgroup id (blockIdx.y * gridDim.x + blockIdx.x), gx = column
+// tiles.  Workgroups go to the eight XCDs round robin by linear id, each XCD with its own L2, and 256 of them (one
+// per CU) run at a time.
+struct WideTile {
+    int bx, m_start, m_end, e;
+    bool found;
+};
+
+template <bool GROUPED, int R>
+__device__ __forceinline__ WideTile wide_tile_of(const DirectArgs& p, int lin, int gx) {
+    constexpr int W_BM = w_bm(R);
+    WideTile t;
+    t.e = 0;
+    t.found = false;
+    if constexpr (!GROUPED) {
+        // Within every round of 256 workgroups give each XCD a compact block of 8 x 4 tiles of one strip of four
+        // tile rows instead of every eighth tile of the grid, so that its L2 holds few operand rows and all XCDs of
+        // a round share the four activation row tiles.
+        const int gy = (p.M + W_BM - 1) / W_BM, total = gx * gy;
+        if (lin >= total) return t;
+        int bx = lin % gx, by = lin / gx;
+        constexpr int H = 4;      // strips of 8 or 16 tile rows measured 1-13 % slower
+        if (gy % H == 0) {
+            int lp = lin;
+            if (lin < (total & ~255)) {
+                const int w = lin & 255;
+                lp = (lin & ~255) + (w & 7) * 32 + (w >> 3);
+            }
+            const int strip = lp / (H * gx), rr = lp % (H * gx);
+            bx = rr / H;
+            by = strip * H + rr % H;
+        }
+        t.bx = bx;
+        t.m_start = by * W_BM;
+        t.m_end = min(p.M, t.m_start + W_BM);
+        t.found = true;
+    } else {
+        int e = 0;
+        int64_t s0 = p.seg_indptr[0];
+        if (gx % 8 == 0) {
+            // XCD x (workgroup id mod 8) owns the column tiles x, x + 8, ...; it walks them segment by
+            // segment, and for every column tile all row tiles of the segment back to back, so the workgroups
+            // that share a weight tile run at the same time on the L2 that holds it.
+            const int x = lin & 7, cx = gx >> 3;
+            int s = lin >> 3;
+            for (; e < p.E; ++e) {
+                const int64_t s1 = p.seg_indptr[e + 1];
+                const int tl = (int)((s1 - s0 + W_BM - 1) / W_BM);
+                if (s < tl * cx) {
+                    const int bl = s / tl, rt = s - bl * tl;
+                    t.found = true;
+                    t.bx = bl * 8 + x;
+                    t.m_start = (int)s0 + rt * W_BM;
+                    t.m_end = min((int)s1, t.m_start + W_BM);
+                    break;
+                }
+                s -= tl * cx;
+                s0 = s1;
+            }
+        } else {
+            int tile = lin / gx, cum = 0;
+            t.bx = lin % gx;
+            for (; e < p.E; ++e) {
+                const int64_t s1 = p.seg_indptr[e + 1];
+                const int tl = (int)((s1 - s0 + W_BM - 1) / W_BM);
+                if (tile < cum + tl) { t.found = true; t.m_start = (int)s0 + (tile - cum) * W_BM; t.m_end = min((int)s1, t.m_start + W_BM); break; }
+                cum += tl;
+                s0 = s1;
+            }
+        }
+        t.e = e;
+    }
+    return t;
+}
+
+// number of tiles of the launch (the valid linear ids are 0 .. total - 1 under both orders above)
+template <bool GROUPED, int R>
+__device__ __forceinline__ int wide_total_tiles(const DirectArgs& p, int gx) {
+    constexpr int W_BM = w_bm(R);
+    if constexpr (!GROUPED) return gx * ((p.M + W_BM - 1) / W_BM);
+    int rows = 0;
+    int64_t s0 = p.seg_indptr[0];
+    for (int e = 0; e < p.E; ++e) {
+        const int64_t s1 = p.seg_indptr[e + 1];
+        rows += (int)((s1 - s0 + W_BM - 1) / W_BM);
+        s0 = s1;
+    }
+    return rows * gx;
+}
+
+// A launch of `total` tiles runs in rounds of 256 (one workgroup per CU).  When the last round holds at most 128
+// tiles, each of them is split along K into z = 256 / ntail (at most 8) work items of ktz K steps (even, at least
+// eight), which write fp32 partial sums that wide_tail_sum_kernel adds: the round then takes 1 / z of a tile's
+// time instead of all of it with most of the chip idle.  The split is taken when the time it saves (a K step
+// costs about 1.6 us) is at least 1.5 times what the partial sums cost (0.5 MB written and read per work item at
+// 5 TB/s, plus 6 us for the second kernel) and K has at least 64 steps (8192 bytes; with fewer steps a tile is too
+// short for the split to pay: measured on the Mixtral gate/up projection, 955 -> 985 us).  z == 1: no split.
+struct WideTail {
+    int full, ntail, z, ktz;
+};
+constexpr int W_TAIL_MIN_KT = 64;
+__host__ __device__ inline WideTail wide_tail_plan(int total, int KT) {
+    WideTail w;
+    w.full = total & ~255;
+    w.ntail = total - w.full;
+    w.z = 1;
+    w.ktz = KT;
+    if (w.ntail > 0 && w.ntail <= 128 && KT >= W_TAIL_MIN_KT) {
+        int z = 256 / w.ntail;
+        if (z > 8) z = 8;
+        int ktz = ((KT + z - 1) / z + 1) & ~1;
+        if (ktz < 8) ktz = 8;
+        z = (KT + ktz - 1) / ktz;
+        const int saved_x10 = KT * 16 * (z - 1) / z, cost_x10 = w.ntail * z + 60;      // tenths of a microsecond
+        if (z > 1 && 2 * saved_x10 >= 3 * cost_x10) {
+            w.ktz = ktz;
+            w.z = z;
+        }
+    }
+    return w;
+}
+constexpr int W_TAIL_ITEMS = 256;               // upper bound of ntail * z
+
 template <int KIND, bool GROUPED, int R = 8>
 __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     static_assert(R == 8 || R == 4, "tile rows per wave");
@@ -48,72 +171,36 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
-    const int KT = K >> 7;
-    int bx = blockIdx.x, by = blockIdx.y;
-    if constexpr (!GROUPED) {
-        // Workgroups go to the eight XCDs round robin by linear id, each XCD with its own L2, and 256 of them
-        // (one per CU) run at a time.  Within every such round give each XCD a compact block of 8 x 4 tiles of
-        // one strip of four tile rows instead of every eighth tile of the grid, so that its L2 holds few
-        // operand rows and all XCDs of a round share the four activation row tiles.
-        const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
-        const int lin = by * gx + bx;
-        constexpr int H = 4;      // strips of 8 or 16 tile rows measured 1-13 % slower
-        if (gy % H == 0) {
-            int lp = lin;
-            if (lin < (total & ~255)) {
-                const int w = lin & 255;
-                lp = (lin & ~255) + (w & 7) * 32 + (w >> 3);
-            }
-            const int strip = lp / (H * gx), rr = lp % (H * gx);
-            bx = rr / H;
-            by = strip * H + rr % H;
+    const int KT_all = K >> 7;
+    // K steps [kt0, kt0 + KT) of the tile; a work item of a split last round writes fp32 sums to `part`
+    int kt0 = 0, KT = KT_all;
+    float* part = nullptr;
+    const int gx = gridDim.x;
+    int lin = blockIdx.y * gx + blockIdx.x;
+    WideTile wt = wide_tile_of<GROUPED, R>(p, lin, gx);
+    if (p.tail_split) {
+        // (the tiles of all but the last round need nothing of this: for them the plan only confirms lin < full;
+        // the segment pointers it reads are the ones the lookup above has just read)
+        const int total = wide_total_tiles<GROUPED, R>(p, gx);
+        const WideTail tp = wide_tail_plan(total, KT_all);
+        if (lin >= tp.full && tp.z > 1) {
+            const int j = lin - tp.full, kpart = j / tp.ntail, idx = j - kpart * tp.ntail;
+            if (kpart >= tp.z) return;
+            lin = tp.full + idx;
+            kt0 = kpart * tp.ktz;
+            KT = min(tp.ktz, KT_all - kt0);
+            part = p.partial + (int64_t)(kpart * tp.ntail + idx) * (W_BM * W_BN);
+            wt = wide_tile_of<GROUPED, R>(p, lin, gx);
         }
     }
-    int m_start, m_end;
+    if (!wt.found) return;
+    const int bx = wt.bx, m_start = wt.m_start, m_end = wt.m_end;
     const uint8_t* bbase = p.b;
     int64_t bs_off = 0;
     if constexpr (GROUPED) {
-        int e = 0;
-        int64_t s0 = p.seg_indptr[0];
-        bool found = false;
-        const int gx = gridDim.x;
-        if (gx % 8 == 0) {
-            // XCD x (workgroup id mod 8) owns the column tiles x, x + 8, ...; it walks them segment by
-            // segment, and for every column tile all row tiles of the segment back to back, so the workgroups
-            // that share a weight tile run at the same time on the L2 that holds it.
-            const int lin = blockIdx.y * gx + blockIdx.x, x = lin & 7, cx = gx >> 3;
-            int s = lin >> 3;
-            for (; e < p.E; ++e) {
-                const int64_t s1 = p.seg_indptr[e + 1];
-                const int t = (int)((s1 - s0 + W_BM - 1) / W_BM);
-                if (s < t * cx) {
-                    const int bl = s / t, rt = s - bl * t;
-                    found = true;
-                    bx = bl * 8 + x;
-                    m_start = (int)s0 + rt * W_BM;
-                    m_end = min((int)s1, m_start + W_BM);
-                    break;
-                }
-                s -= t * cx;
-                s0 = s1;
-            }
-        } else {
-            int tile = blockIdx.y, cum = 0;
-            for (; e < p.E; ++e) {
-                const int64_t s1 = p.seg_indptr[e + 1];
-                const int t = (int)((s1 - s0 + W_BM - 1) / W_BM);
-                if (tile < cum + t) { found = true; m_start = (int)s0 + (tile - cum) * W_BM; m_end = min((int)s1, m_start + W_BM); break; }
-                cum += t;
-                s0 = s1;
-            }
-        }
-        if (!found) return;
-        const int64_t widx = p.weight_indices ? p.weight_indices[e] : e;
+        const int64_t widx = p.weight_indices ? p.weight_indices[wt.e] : wt.e;
         bbase += widx * (int64_t)N * K;
-        bs_off = widx * (int64_t)((N + 127) / 128) * KT;
-    } else {
-        m_start = by * W_BM;
-        m_end = min(p.M, m_start + W_BM);
+        bs_off = widx * (int64_t)((N + 127) / 128) * KT_all;
     }
     const int n0 = bx * W_BN;
 
@@ -144,7 +231,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const int col = (row & 192) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
-    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT * 4u;
+    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
 
     // ---- 4-bit weights: a thread owns the same piece of the 128-column half h = 0, 1 of the tile as in the
     // 128-column tile kernel (gemm_dma.hpp): per K step and half one 8-byte load of packed weights and one load
@@ -170,8 +257,8 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             if constexpr (W4NK) {
-                w4_words[h] = asm_load_b64(w4_off[h], (const uint8_t*)p.b + (int64_t)kt * 32);
-                w4_scale16[h] = asm_load_u16(w4_soff[h], (const uint8_t*)p.b_s + (int64_t)((kt * 64) / p.group) * 2);
+                w4_words[h] = asm_load_b64(w4_off[h], (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 32);
+                w4_scale16[h] = asm_load_u16(w4_soff[h], (const uint8_t*)p.b_s + (int64_t)(((kt0 + kt) * 64) / p.group) * 2);
             }
         }
     };
@@ -211,9 +298,9 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 
     auto issue = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
-        const uint8_t* ga = p.a + (int64_t)kt * 128;
-        const uint8_t* gb = bbase + (int64_t)kt * 128;
-        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
+        const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
+        const uint8_t* gb = bbase + (int64_t)(kt0 + kt) * 128;
+        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
         if constexpr (W4) w4_request(kt);          // in front of the activation loads: see w4_expand
 #pragma unroll
         for (int i = 0; i < AL; ++i) dma16(st + (uint32_t)(wave * AL + i) * 1024u, aoff[i], ga);
@@ -228,14 +315,14 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     // mid-step barrier, the activation rows and the scale column behind the barrier of the step.
     auto issue_part = [&](int kt, int part) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
-        const uint8_t* ga = p.a + (int64_t)kt * 128;
-        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)kt * 4;
+        const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
+        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
         if (part < AL) dma16(st + (uint32_t)(wave * AL + part) * 1024u, aoff[part < AL ? part : 0], ga);
         if constexpr (SCALED) if (part == 3) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
     };
     auto issue_b_part = [&](int kt, int part) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
-        dma16(st + W_A + (uint32_t)(wave * 4 + part) * 1024u, boff[part], bbase + (int64_t)kt * 128);
+        dma16(st + W_A + (uint32_t)(wave * 4 + part) * 1024u, boff[part], bbase + (int64_t)(kt0 + kt) * 128);
     };
 
     // acc[i][j][q] = C[row 16i + r][col 32*(j >> 1) + 8g + 4*(j & 1) + q] of the wave's 16 R x 64 tile
@@ -251,7 +338,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         for (int i = tid; i < 2 * KT; i += W_THREADS) {
             const int c = i >= KT ? 1 : 0, kk = i - c * KT;
             const int64_t blk = min(bx * 2 + c, nblk - 1);
-            bsl[c * D_MAX_KT + kk] = ld_scale(p.b_s, bs_off + blk * KT + kk, p.s_dtype);
+            bsl[c * D_MAX_KT + kk] = ld_scale(p.b_s, bs_off + blk * KT_all + kt0 + kk, p.s_dtype);
         }
     }
     __builtin_amdgcn_s_waitcnt(LLMK_WAIT_VMCNT_0);
@@ -286,6 +373,16 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     auto store_row = [&](int i) {
         const int m = m_start + wm * 16 * R + 16 * i + r;
         if (m >= m_end) return;
+        if constexpr (KIND != K_I8_ROWCOL) {
+            if (part) {          // work item of a split last round: the fp32 sums of its K range, [tile row][tile column]
+                float* dst = part + (wm * 16 * R + 16 * i + r) * W_BN + wn * 64 + 8 * g;
+                *(v4f*)dst = acc[i][0];
+                *(v4f*)(dst + 4) = acc[i][1];
+                *(v4f*)(dst + 32) = acc[i][2];
+                *(v4f*)(dst + 36) = acc[i][3];
+                return;
+            }
+        }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int nbh = n0 + wn * 64 + 32 * h + 8 * g;
@@ -421,17 +518,74 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     for (int i = 0; i < R; ++i) store_row(i);
 }
 
+// Adds the partial sums of the split last round (see wide_tail_plan) and writes the outputs of its tiles: grid
+// (tiles of that round, slices of 32 tile rows), the K ranges in ascending order (the result does not depend on
+// timing); a thread sums eight rows at a time so that eight loads are in flight per K range.
+template <bool GROUPED, int R>
+__global__ __launch_bounds__(256) void wide_tail_sum_kernel(DirectArgs p, int esz) {
+    constexpr int W_BM = w_bm(R);
+    const int gx = (p.N + W_BN - 1) / W_BN;
+    const WideTail tp = wide_tail_plan(wide_total_tiles<GROUPED, R>(p, gx), (p.K * esz) >> 7);
+    const int idx = blockIdx.x;
+    if (tp.z <= 1 || idx >= tp.ntail) return;
+    const WideTile wt = wide_tile_of<GROUPED, R>(p, tp.full + idx, gx);
+    if (!wt.found) return;
+    const int rows = wt.m_end - wt.m_start, c4 = (threadIdx.x & 63) * 4, n = wt.bx * W_BN + c4;
+    const int row0 = (int)blockIdx.y * 32 + (threadIdx.x >> 6);
+    if ((int)blockIdx.y * 32 >= rows) return;
+    v4f s[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) s[it] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < tp.z; ++k) {
+        const float* src = p.partial + ((int64_t)(k * tp.ntail + idx) * W_BM + row0) * W_BN + c4;
+#pragma unroll
+        for (int it = 0; it < 8; ++it) s[it] += *(const v4f*)(src + it * 4 * W_BN);      // rows past the tile end: stale scratch, not stored
+    }
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int row = row0 + 4 * it;
+        if (row >= rows) continue;
+        const int64_t off = (int64_t)(wt.m_start + row) * p.N + n;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (n + q < p.N) st_out(p.c, off + q, s[it][q], p.c_dtype);
+    }
+}
+
+// scratch of the split last round: W_TAIL_ITEMS partial tiles of the larger tile shape
+constexpr int64_t w_tail_bytes() { return (int64_t)W_TAIL_ITEMS * w_bm(8) * W_BN * 4; }
+
 template <int KIND, bool GROUPED, int R = 8>
-int launch_wide(const DirectArgs& p, hipStream_t stream, const char* name) {
+int launch_wide(const DirectArgs& p0, hipStream_t stream, const char* name, void* ws = nullptr, int64_t ws_bytes = 0) {
     static std::atomic<uint64_t> configured{0};
     auto kern = gemm_wide_kernel<KIND, GROUPED, R>;
     constexpr int W_BM = w_bm(R), W_LDS = w_lds(R);
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK) ? 2 : 1;
     if (int rc = llmk_reserve_lds((const void*)kern, W_LDS, configured, name)) return rc;
+    DirectArgs p = p0;
     const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, W_BM) : (p.M + W_BM - 1) / W_BM;
     dim3 grid((unsigned)((p.N + W_BN - 1) / W_BN), (unsigned)tiles_m);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
+    // a short last round of tiles is split along K when the scratch for its partial sums is there (dense: decided
+    // here; grouped: the segment ends are known on the device only, so the kernel decides, from 256 tiles on)
+    bool tail = false;
+    p.tail_split = 0;
+    if constexpr (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || KIND == K_F16 || KIND == K_BF16) {
+        const int KT = (p.K * ESZ) >> 7;
+        if (ws && ws_bytes >= w_tail_bytes() && !((uintptr_t)ws & 15) && KT >= W_TAIL_MIN_KT && p.c)
+            tail = GROUPED ? (int64_t)grid.x * grid.y >= 256 : wide_tail_plan((int)(grid.x * grid.y), KT).z > 1;
+    }
+    if (tail) {
+        p.tail_split = 1;
+        p.partial = (float*)ws;
+        grid.y += (W_TAIL_ITEMS + grid.x - 1) / grid.x;     // the work items of the split round
+    }
     kern<<<grid, W_THREADS, W_LDS, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
+    if (tail) {
+        wide_tail_sum_kernel<GROUPED, R><<<dim3(128, W_BM / 32), 256, 0, stream>>>(p, ESZ);
+        LLMK_CHECK_LAUNCH(name);
+    }
     return LLMK_OK;
 }
 
@@ -458,7 +612,7 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
 // shape (60 / 36 / 43 / 26 / 16 microseconds for 256 x 256, 128 x 256, 256 x 128, 128 x 128 and 64 x 128 at K = 4096
 // for fp8; the ratios hold for the other kinds and K).  Ties go to the larger tile (less operand re-reading).  Segments of a grouped GEMM are judged by their average length.
 template <int KIND, bool GROUPED>
-int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
+int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* ws = nullptr, int64_t ws_bytes = 0) {
     if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
     // 4-bit weights: the row-packed layout, dense launches (the Marlin scatter of 2-byte pieces measured 4-9 % slower
     // inside the 256-column kernel than the dequantisation pass at every M > 512)
@@ -477,11 +631,11 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name) {
             // (a tie goes to the 128-row tile for block-scaled int8, whose per-step conversions leave the tall
             // tile less of its advantage: grouped Mixtral down projection -3 %; +1 % for fp8)
             const double t_half = 36.0 * rounds(128, 256);
-            if (t_half < t_wide || (KIND == K_I8_BLOCK && GROUPED && t_half == t_wide)) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
-            return launch_wide<KIND, GROUPED>(p, stream, name);
+            if (t_half < t_wide || (KIND == K_I8_BLOCK && GROUPED && t_half == t_wide)) return launch_wide<KIND, GROUPED, 4>(p, stream, name, ws, ws_bytes);
+            return launch_wide<KIND, GROUPED>(p, stream, name, ws, ws_bytes);
         }
         const double t_half = 36.0 * rounds(128, 256);
-        if (t_half < t4 && t_half <= t2 && t_half <= t1) return launch_wide<KIND, GROUPED, 4>(p, stream, name);
+        if (t_half < t4 && t_half <= t2 && t_half <= t1) return launch_wide<KIND, GROUPED, 4>(p, stream, name, ws, ws_bytes);
     }
     if (t4 <= t2 && t4 <= t1) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
     if (t2 <= t1) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
@@ -514,7 +668,8 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
             p.ksplit = z;
         }
     }
-    return launch_dma<KIND, GROUPED>(p, stream, name);
+    if (p.ksplit > 1 || !workspace || workspace_bytes <= used) return launch_dma<KIND, GROUPED>(p, stream, name);
+    return launch_dma<KIND, GROUPED>(p, stream, name, (uint8_t*)workspace + used, workspace_bytes - used);   // split last round
 }
 
 // K slices for the half-precision tile kernel (a K step is 64 elements there): same rule as splitk_factor
@@ -531,7 +686,8 @@ int launch_big_half(DirectArgs p, hipStream_t stream, const char* name, void* wo
             p.ksplit = z;
         }
     }
-    return launch_dma<KIND, GROUPED>(p, stream, name);
+    if (p.ksplit > 1) return launch_dma<KIND, GROUPED>(p, stream, name);
+    return launch_dma<KIND, GROUPED>(p, stream, name, workspace, workspace_bytes);                             // split last round
 }
 
 }  // namespace llmk

@@ -314,3 +314,35 @@ def test_wide_tile_kernel_ragged_shapes(dev, kind, M, N, K):
         with default_dtype(out):
             c = fn(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
         assert_close_scaled(c, ref, what="wide %s" % kind)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
+@pytest.mark.parametrize("M,N,K,out", [(1100, 1300, 8192, torch.bfloat16), (600, 5000, 16384, torch.float32),
+                                       (2500, 3000, 8192, torch.float16), (4096, 6144, 8192, torch.bfloat16)])
+def test_large_tiles_split_last_round(dev, kind, M, N, K, out):
+    """Long K and a tile count that leaves a short last round of 256 workgroups (30, 60, 120 and 128 tiles of
+    256 x 256, or the corresponding 128-row tiles): the tiles of that round are split along K and a second kernel
+    adds the fp32 partial sums.  Ragged rows and columns, every output dtype."""
+    announce("split last round", kind, M, N, K, out)
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    with default_dtype(out):
+        if kind == "fp8":
+            a, a_s = q.act_quant_fp8(x)
+            b, b_s = q.weight_quant_fp8(w)
+            c = fp8_kernel.fp8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+        else:
+            a, a_s = q.act_quant_int8(x)
+            b, b_s = q.weight_quant_int8(w)
+            c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert c.dtype == out
+    rows = torch.randperm(M)[:96].sort().values                     # 96 random rows, all columns; every element finite
+    assert bool(torch.isfinite(c).all())
+    assert_close_scaled(c[rows.to(dev)], g.gemm_blockwise(a[rows], a_s[rows], b, b_s), what="split last round " + kind)
+    # all rows: column sums against a one-row oracle GEMM of the scale-weighted column sums of A
+    wsum = (a.float().double().reshape(M, K // 128, 128) * a_s.double()[:, :, None]).sum(0).reshape(1, K)
+    want = g.gemm_blockwise(wsum, torch.ones(1, K // 128, dtype=torch.float64), b.float(), b_s)[0]
+    got = c.double().sum(0).cpu()
+    ref_rms = g.gemm_blockwise(a[rows], a_s[rows], b, b_s).pow(2).mean().sqrt().item()
+    assert bool(((got - want).abs() <= 1e-2 * ref_rms * (M ** 0.5) + 1e-2 * want.abs()).all()), "column sums"

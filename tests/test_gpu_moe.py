@@ -212,6 +212,32 @@ def test_grouped_gemm_large_tiles_exact(dev, M, N, K):
     assert torch.all(out[used:] == 5.0)
 
 
+@pytest.mark.parametrize("M,N,K,E", [(9000, 2048, 8192, 6), (9000, 1280, 8192, 6), (4700, 4096, 14336, 3)])
+def test_grouped_gemm_split_last_round_exact(dev, M, N, K, E):
+    """Long K and a number of 256 x 256 tiles that leaves a short last round: the tiles of that round are split
+    along K (fp32 partial sums in the scratch, a second kernel adds them).  Same exact-integer check as above;
+    column-tile counts that are and are not a multiple of the XCD count, an empty and a one-row segment."""
+    announce("grouped split last round", M, N, K, E)
+    torch.manual_seed(M + N + K)
+    used = M - 5
+    cuts = sorted(int(x) for x in torch.randperm(used - 2)[:E - 3] + 2)
+    seg = torch.tensor([0, 0, 1] + cuts + [used])                             # an empty and a one-row segment first
+    assert len(seg) == E + 1 and bool((seg[1:] >= seg[:-1]).all())
+    widx = torch.randperm(E)
+    a = torch.randint(-7, 8, (M, K), dtype=torch.int8)
+    b = torch.randint(-7, 8, (E, N, K), dtype=torch.int8)
+    a_s = torch.ones(M, K // 128, dtype=torch.float32)
+    b_s = torch.ones(E, (N + 127) // 128, K // 128, dtype=torch.float32)
+    c = torch.full((M, N), 5.0, dtype=torch.float32, device=dev)
+    _lib_call_grouped_i8(dev, a, a_s, b, b_s, c, seg, widx)
+    out = c.cpu()
+    for e in range(E):
+        lo, hi = int(seg[e]), int(seg[e + 1])
+        ref = (a[lo:hi].float() @ b[widx[e]].float().T)                       # |sum| < 2^24: exact in fp32
+        assert torch.equal(out[lo:hi], ref), "segment %d" % e
+    assert torch.all(out[used:] == 5.0)
+
+
 def _lib_call_grouped_i8(dev, a, a_s, b, b_s, c, seg, widx):
     """grouped_gemm_triton on activations that are already int8 with their 1 x 128 scales."""
     d = [t.to(dev).contiguous() for t in (a, a_s, b, b_s, seg.long(), widx.long())]
