@@ -1,5 +1,6 @@
 // W4A8 GEMM: int8 activations x row-packed uint4 weights with two-level scales.
 #include "gemm_wide.hpp"
+#include "stream_ring.hpp"
 
 using namespace llmk;
 
@@ -43,7 +44,9 @@ __global__ void w4a8_expand_kernel(const int32_t* __restrict__ packed, const int
 //
 // Workgroup = 8 waves on 16 MT rows x 16 columns (two packed rows), persistent over column tiles; each wave
 // takes a run of consecutive 128-K steps; activation fragments, their per-group sums and scales stay resident.  The
-// loads of tiles i+1 and i+2 are in flight while tile i is multiplied; past the last tile the same number of
+// loads of tiles i+1 and i+2 are in flight while tile i is multiplied: a ring of three register sets filled by
+// hand-issued loads and released by one hand-counted wait per tile (stream_ring.hpp; with ordinary loads the
+// compiler ended every conditional request of the loop with a full wait).  Past the last tile the same number of
 // loads is still issued (all lanes on one hot line) so that the wait counts stay exact.
 struct W4A8Args {
     const int8_t* a; const void* a_s; const int32_t* packed; const void* b_s; const int8_t* s4; const int8_t* z4;
@@ -79,33 +82,45 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
 
     // z / s: the four zero points and second-level scales of this lane's column, one byte per step of the wave;
     // bs: the block scale of step (lane & 3)
-    struct TileRegs { unsigned z, s, bs; v4i w[2 * ROUNDS]; };
+    struct TileRegs { int z, s, bs; v4i w[2 * ROUNDS]; };
+    constexpr int LPT = 2 * ROUNDS + 3;                   // loads per tile and lane
+    const RingBase zbase = ring_base(p.z4), sbase = ring_base(p.s4), bsbase = ring_base(p.b_s);
     auto issue_tile = [&](TileRegs& t, int tile) __attribute__((always_inline)) {
         const bool live = tile < ntiles;
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
             const int prow = live ? min(tile * 2 + hh, np - 1) : 0;
-            const uint8_t* rowp = (const uint8_t*)p.packed + ((int64_t)prow * Kfull + k0) * 4;
+            const RingBase rowp = ring_base((const uint8_t*)p.packed + ((int64_t)prow * Kfull + k0) * 4);
 #pragma unroll
             for (int rd = 0; rd < ROUNDS; ++rd) {
                 const uint32_t off = (uint32_t)(rd * 8192 + wave * 1024 + lane * 16);
-                t.w[hh * ROUNDS + rd] = *(const v4i*)(rowp + (live ? min(off, (uint32_t)(K * 4 - 16)) : 0u));
+                t.w[hh * ROUNDS + rd] = ring_load_b128<0>(live ? min(off, (uint32_t)(K * 4 - 16)) : 0u, rowp);
             }
         }
         const int n = live ? min(tile * 16 + r, N - 1) : 0;
-        // dword at byte n * (K / 128) + first step of this wave, pulled back inside the table at its very end
+        // dword at byte n * (K / 128) + first step of this wave, pulled back inside the table at its very end (the
+        // shift that undoes the pull is applied where the bytes are used)
         const int64_t want = (int64_t)n * sfull + sk0 + ks0, last = (int64_t)N * sfull - 4;
-        const int64_t at = min(want, last);
-        const int sh = (int)(want - at) * 8;
-        unsigned zw, sw;
-        __builtin_memcpy(&zw, p.z4 + at, 4);
-        __builtin_memcpy(&sw, p.s4 + at, 4);
-        t.z = sh < 32 ? zw >> sh : 0u;
-        t.s = sh < 32 ? sw >> sh : 0u;
+        const uint32_t at = (uint32_t)min(want, last);
+        t.z = ring_load_b32<0>(at, zbase);
+        t.s = ring_load_b32<0>(at, sbase);
         const int64_t bsrow = (int64_t)((min(tile, ntiles - 1) * 16) >> 7) * sfull + sk0;
         const int kb = min(ks0 + (lane & 3), steps - 1);
-        if constexpr (SDT == LLMK_F32) t.bs = __float_as_uint(((const float*)p.b_s)[bsrow + kb]);
-        else t.bs = ((const unsigned short*)p.b_s)[bsrow + kb];
+        if constexpr (SDT == LLMK_F32) t.bs = ring_load_b32<0>((uint32_t)(bsrow + kb) * 4u, bsbase);
+        else t.bs = ring_load_u16<0>((uint32_t)(bsrow + kb) * 2u, bsbase);
+    };
+    // how far the dword of zero points / scales of a tile was pulled back (bits): the same for every tile of a lane
+    // except the last columns of the matrix
+    auto pulled = [&](int tile) {
+        const int n = tile < ntiles ? min(tile * 16 + r, N - 1) : 0;
+        const int64_t want = (int64_t)n * sfull + sk0 + ks0, last = (int64_t)N * sfull - 4;
+        return (int)(want - min(want, last)) * 8;
+    };
+    auto tile_wait = [&](auto nc, TileRegs& t) __attribute__((always_inline)) {
+        constexpr int NY = decltype(nc)::value;
+        if constexpr (ROUNDS == 1) ring_wait<NY>(t.w[0], t.w[1]);
+        else ring_wait<NY>(t.w[0], t.w[1], t.w[2], t.w[3]);
+        ring_wait<NY>(t.z, t.s, t.bs);
     };
     auto stage_tile = [&](const TileRegs& t, int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -115,25 +130,62 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
                 *(v4i*)(tbuf + buf * TB + hh * ROWSTRIDE + rd * 8192 + wave * 1024 + lane * 16) = t.w[hh * ROUNDS + rd];
     };
 
-    // resident activation fragments (chunks g and g + 4 of every 128-byte step) and their scales first, so that
-    // the per-step sums below are computed while the first weight tiles are still on their way
-    v8i afrag[U][MT];
-    float ascale[U][MT];
+    // resident activation fragments (chunks g and g + 4 of every 128-byte step) and their scales are requested
+    // first, hand-issued like the weights (an ordinary load in front of hand-issued ones would make the compiler
+    // wait for all of them): the per-step sums below are computed while the first weight tiles are on their way
+    v4i alo[U][MT], ahi[U][MT];
+    int araw[U][MT];
+    {
+        typedef typename ScaleIO<SDT>::Raw SRaw;
+        const RingBase abase = ring_base((const uint8_t*)p.a + k0), asbase = ring_base(p.a_s);
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+        for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int ks = min(ks0 + u, steps - 1);
-            const int arow = min(m0 + 16 * mt + r, M - 1);
-            afrag[u][mt] = ld_split((const uint8_t*)p.a + (int64_t)arow * Kfull + k0 + 16 * g + (int64_t)ks * 128);
-            ascale[u][mt] = ScaleIO<SDT>::cvt(((const typename ScaleIO<SDT>::Raw*)p.a_s)[(int64_t)arow * sfull + sk0 + ks]);
-        }
+            for (int mt = 0; mt < MT; ++mt) {
+                const int ks = min(ks0 + u, steps - 1);
+                const int arow = min(m0 + 16 * mt + r, M - 1);
+                const uint32_t off = (uint32_t)arow * (uint32_t)Kfull + (uint32_t)(16 * g + ks * 128);
+                alo[u][mt] = ring_load_b128<0>(off, abase);
+                ahi[u][mt] = ring_load_b128<64>(off, abase);
+                const uint32_t soff = (uint32_t)(arow * sfull + sk0 + ks) * (uint32_t)sizeof(SRaw);
+                if constexpr (sizeof(SRaw) == 4) araw[u][mt] = ring_load_b32<0>(soff, asbase);
+                else araw[u][mt] = ring_load_u16<0>(soff, asbase);
+            }
+    }
 
     int tile = blockIdx.x;
     const int stride = gridDim.x;
+    if (tile >= ntiles) return;
     TileRegs tr[D];
 #pragma unroll
     for (int j = 0; j < D - 1; ++j) issue_tile(tr[j], tile + j * stride);
+
+    // the activations have landed when only the loads of the two tiles just requested are in flight
+    v8i afrag[U][MT];
+    float ascale[U][MT];
+    {
+        constexpr int NY = (D - 1) * LPT;
+        static_assert(U == 4 && (MT == 1 || MT == 2), "the waits below are spelled out for these sizes");
+        if constexpr (MT == 1) {
+            ring_wait<NY>(alo[0][0], alo[1][0], alo[2][0], alo[3][0], ahi[0][0], ahi[1][0], ahi[2][0], ahi[3][0]);
+            ring_wait<NY>(araw[0][0], araw[1][0], araw[2][0], araw[3][0]);
+        } else {
+            ring_wait<NY>(alo[0][0], alo[1][0], alo[2][0], alo[3][0], ahi[0][0], ahi[1][0], ahi[2][0], ahi[3][0]);
+            ring_wait<NY>(alo[0][MT - 1], alo[1][MT - 1], alo[2][MT - 1], alo[3][MT - 1], ahi[0][MT - 1], ahi[1][MT - 1], ahi[2][MT - 1], ahi[3][MT - 1]);
+            ring_wait<NY>(araw[0][0], araw[1][0], araw[2][0], araw[3][0]);
+            ring_wait<NY>(araw[0][MT - 1], araw[1][MT - 1], araw[2][MT - 1], araw[3][MT - 1]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const v4i x = alo[u][mt], y = ahi[u][mt];
+                afrag[u][mt] = (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+                typedef typename ScaleIO<SDT>::Raw SRaw;
+                if constexpr (sizeof(SRaw) == 4) ascale[u][mt] = __int_as_float(araw[u][mt]);
+                else ascale[u][mt] = ScaleIO<SDT>::cvt((SRaw)(araw[u][mt] & 0xffff));
+            }
+    }
 
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -149,6 +201,7 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
             sum += __shfl_xor(sum, 32, 64);
             if (g == 0 && step_ok(u)) tab[(mt * 16 + r) * steps + ks0 + u] = make_float2(ascale[u][mt], (float)sum);
         }
+    tile_wait(std::integral_constant<int, LPT>{}, tr[0]);          // the first tile; the second may still be on its way
     stage_tile(tr[0], 0);
     __syncthreads();
     float2 rtab[TAB_REGS ? U : 1][4];
@@ -237,10 +290,12 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
         bool ok[U], all_ok = true;
         float bs[U];
         int ksc[U], zu[U], su[U];
+        const int sh = pulled(tile);
+        const unsigned tz = sh < 32 ? (unsigned)t.z >> sh : 0u, ts = sh < 32 ? (unsigned)t.s >> sh : 0u;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             ksc[u] = min(ks0 + u, steps - 1);
-            const int z = (int)(t.z << (24 - 8 * u)) >> 24, sc4 = (int)(t.s << (24 - 8 * u)) >> 24;
+            const int z = (int)(tz << (24 - 8 * u)) >> 24, sc4 = (int)(ts << (24 - 8 * u)) >> 24;
             zu[u] = z;
             su[u] = sc4;
             // (q - z) * s for q = 0 and q = 15 bound every product of the group (24-bit multiplies are exact here)
@@ -272,12 +327,12 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
         }
     };
     // cross-wave reduction and store of the finished tile; the same barrier publishes the next tile's bytes
-    auto finish = [&](int tl, const TileRegs& next, int next_buf) __attribute__((always_inline)) {
+    auto finish = [&](auto stage_c, int tl, const TileRegs& next, int next_buf) __attribute__((always_inline)) {
         float* rbuf = red + parity * NW * MT * 256;
         parity ^= 1;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) *(v4f*)(rbuf + ((wave * MT + mt) * 64 + lane) * 4) = acc[mt];
-        stage_tile(next, next_buf);
+        if constexpr (decltype(stage_c)::value) stage_tile(next, next_buf);
         __syncthreads();
         const int n0 = tl * 16;
         for (int o = tid; o < MT * 256; o += NW * 64) {
@@ -293,20 +348,42 @@ __global__ __launch_bounds__(512) void w4a8_stream_kernel(W4A8Args p) {
         }
         clear_acc();
     };
+    // Slot d of the ring: request tile i + 2 into the set that tile i - 1 has left, multiply tile i (its words are in
+    // LDS, staged by the slot before), wait for tile i + 1 (only the LPT loads just requested are younger), and
+    // finish: reduce and store tile i while the same barrier publishes the staged words of tile i + 1.  Whole rounds
+    // of the three slots run in a loop without a branch (requests past the last tile are clamped).  Behind the loop
+    // everything requested is waited for, consumed or not, and the remaining one or two tiles request nothing: a
+    // register whose load nobody consumes would be reused by the compiler while the load is still in flight.
     int lbuf = 0;
-    auto one = [&](const TileRegs& cur, const TileRegs& nxt, TileRegs& fill) __attribute__((always_inline)) {
-        issue_tile(fill, tile + (D - 1) * stride);
-        mul_tile(cur, lbuf);
-        finish(tile, nxt, lbuf ^ 1);
+    const std::true_type yes;
+    const std::false_type no;
+    auto slot = [&](auto dc) __attribute__((always_inline)) {
+        constexpr int d = decltype(dc)::value;
+        issue_tile(tr[(d + 2) % D], tile + (D - 1) * stride);
+        mul_tile(tr[d], lbuf);
+        tile_wait(std::integral_constant<int, LPT>{}, tr[(d + 1) % D]);
+        finish(yes, tile, tr[(d + 1) % D], lbuf ^ 1);
         lbuf ^= 1;
         tile += stride;
     };
-    while (tile < ntiles) {
-#pragma unroll
-        for (int j = 0; j < D; ++j) {
-            one(tr[j], tr[(j + 1) % D], tr[(j + D - 1) % D]);
-            if (tile >= ntiles) break;
+    static_assert(D == 3, "ring slots are spelled out below");
+    const int my_tiles = (ntiles - tile + stride - 1) / stride;
+    for (int rd = my_tiles / D; rd > 0; --rd) {
+        slot(std::integral_constant<int, 0>{});
+        slot(std::integral_constant<int, 1>{});
+        slot(std::integral_constant<int, 2>{});
+    }
+    tile_wait(std::integral_constant<int, 0>{}, tr[1]);
+    const int rem = my_tiles % D;
+    if (rem > 0) {
+        mul_tile(tr[0], lbuf);
+        if (rem > 1) {
+            finish(yes, tile, tr[1], lbuf ^ 1);
+            lbuf ^= 1;
+            tile += stride;
+            mul_tile(tr[1], lbuf);
         }
+        finish(no, tile, tr[1], lbuf);
     }
 }
 
@@ -373,7 +450,9 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
     // K > 4096 runs as ranges of at most 4096 with fp32 partial sums in the workspace (up to 64 rows)
     const int64_t nz = (K / 128 + 31) / 32;
     const bool long_k_ok = nz == 1 || (row_blocks <= 2 && workspace && workspace_bytes >= nz * M * N * 4 && !(((uintptr_t)workspace) & 15));
-    if (fused_wins && long_k_ok && group_int4 == 128 && !(((uintptr_t)a | (uintptr_t)b_packed) & 15)) {
+    // (the hand-issued loads of the fused kernel take 32-bit lane offsets into the activations and the tables)
+    const bool small_offsets = M * K < (1ll << 32) && N * (K / 128) < (1ll << 32);
+    if (fused_wins && long_k_ok && small_offsets && group_int4 == 128 && !(((uintptr_t)a | (uintptr_t)b_packed) & 15)) {
         W4A8Args p{a, a_s, b_packed, b_s, b_s4, b_z4, c, c_dtype, (int)M, (int)N, (int)K, 0, nullptr};
         if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: c_dtype %d", c_dtype);
         hipStream_t st = (hipStream_t)stream;

@@ -75,6 +75,14 @@ __device__ __forceinline__ int ring_load_u16(uint32_t voff, RingBase base) {
 
 // s_waitcnt vmcnt(N) that names the registers it releases
 template <int N>
+__device__ __forceinline__ void ring_wait(v4i& a, v4i& b) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void ring_wait(int& a, int& b, int& c) {
+    asm volatile("s_waitcnt vmcnt(%3)" : "+v"(a), "+v"(b), "+v"(c) : "n"(N) : "memory");
+}
+template <int N>
 __device__ __forceinline__ void ring_wait(v4i& a, v4i& b, v4i& c, v4i& d) {
     asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N) : "memory");
 }
