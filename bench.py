@@ -361,8 +361,22 @@ def run_case(case, dev, steps, warmup, eager=False):
         torch.cuda.synchronize()
         ev.append(e0.elapsed_time(e1))
     ev.sort()
+    # HBM-bound cases also without the flush (a replay queued right behind another): what a caller sees whose weights
+    # are still in the 256 MB memory-side cache; reported beside the cold figure, never instead of it
+    warm = None
+    if cold:
+        wv = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            replay()
+            e0.record()
+            replay()
+            e1.record()
+            torch.cuda.synchronize()
+            wv.append(e0.elapsed_time(e1))
+        warm = sorted(wv)[1]
     return {"wall": wall, "ev_ms": ev[len(ev) // 2], "ev_ms_min": ev[0], "ev_ms_max": ev[-1],
-            "preroll_ms": preroll_ms, "preroll_replays": n_pre, "cold": cold}
+            "preroll_ms": preroll_ms, "preroll_replays": n_pre, "cold": cold, "warm_ms": warm}
 
 
 def measured_traffic(workload):
@@ -389,6 +403,7 @@ def record(case, t, steps):
             "us_per_launch_min": round(t["ev_ms_min"] * 1e3 / steps, 2), "us_per_launch_max": round(t["ev_ms_max"] * 1e3 / steps, 2),
             "timed_replays": TIMED_REPLAYS, "preroll_ms": round(t["preroll_ms"], 1), "preroll_replays": t["preroll_replays"],
             "cache_flushed_before_each_replay": t["cold"],
+            "us_per_launch_without_flush": None if t.get("warm_ms") is None else round(t["warm_ms"] * 1e3 / steps, 2),
             "tflops": round(tflops, 2), "gbs": round(gbs, 1), "alg_bytes": case.bytes, "flops": case.flops,
             "weight_copies_rotated": case.nbuf, "wall_ms_per_step": round(t["wall"] * 1e3 / steps, 4), "roofline": roof}
 
