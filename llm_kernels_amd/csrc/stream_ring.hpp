@@ -95,19 +95,11 @@ __device__ __forceinline__ void ring_wait(v4i& a, v4i& b, v4i& c, v4i& d, v4i& e
     asm volatile("s_waitcnt vmcnt(%8)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h) : "n"(N) : "memory");
 }
 template <int N>
-__device__ __forceinline__ void ring_wait(v4i& a, v4i& b, v4i& c, v4i& d, v4i& e, v4i& f, v4i& g, v4i& h, v4i& s) {
-    asm volatile("s_waitcnt vmcnt(%9)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h), "+v"(s) : "n"(N) : "memory");
-}
-template <int N>
 __device__ __forceinline__ void ring_wait16(v4i (&a)[16]) {
     asm volatile("s_waitcnt vmcnt(%16)"
                  : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
                    "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15])
                  : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void ring_wait(int& a) {
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void ring_wait(int& a, int& b, int& c, int& d) {
