@@ -317,12 +317,13 @@ def test_wide_tile_kernel_ragged_shapes(dev, kind, M, N, K):
 
 
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
-@pytest.mark.parametrize("M,N,K,out", [(1100, 1300, 8192, torch.bfloat16), (600, 5000, 16384, torch.float32),
-                                       (2500, 3000, 8192, torch.float16), (4096, 6144, 8192, torch.bfloat16)])
+@pytest.mark.parametrize("M,N,K,out", [(5120, 10240, 8192, torch.bfloat16), (4096, 4608, 8192, torch.float32),
+                                       (5000, 10200, 8192, torch.float16), (1100, 1300, 8192, torch.bfloat16)])
 def test_large_tiles_split_last_round(dev, kind, M, N, K, out):
-    """Long K and a tile count that leaves a short last round of 256 workgroups (30, 60, 120 and 128 tiles of
-    256 x 256, or the corresponding 128-row tiles): the tiles of that round are split along K and a second kernel
-    adds the fp32 partial sums.  Ragged rows and columns, every output dtype."""
+    """Long K and a tile count that leaves a short last round of 256 workgroups: 800 tiles of 256 x 256 (three
+    rounds and 32 tiles, split eight ways), 576 tiles of 128 x 256 (two rounds and 64 tiles, split four ways), the
+    first again with ragged rows and columns, and a small problem on smaller tiles for contrast.  The tiles of the
+    short round are split along K and a second kernel adds the fp32 partial sums.  Every output dtype."""
     announce("split last round", kind, M, N, K, out)
     torch.manual_seed(M + N + K)
     x = torch.randn(M, K).bfloat16()
