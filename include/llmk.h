@@ -131,10 +131,12 @@ int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const 
 /* per-token x per-channel W8A8 with one full-K int32 accumulation (a scheme with
  * no counterpart function in the reference).  c may be NULL; c_i32 (raw accumulators) may be NULL.
  * M <= 64 streams the weights once; larger M runs on the MFMA tile kernels (int32 accumulation inside
- * the MFMA, c = float(acc) * a_s[m] * b_s[n] in the epilogue of either path). */
+ * the MFMA, c = float(acc) * a_s[m] * b_s[n] in the epilogue of either path).  With a workspace of
+ * llmk_gemm_workspace_bytes(M, N, K), shapes with few tiles and a long K are split along K; the slices' int32 sums
+ * are added as integers before the scaling, so c and c_i32 do not depend on the split. */
 int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, const float* b_s,
                         void* c, int c_dtype, int32_t* c_i32, int64_t M, int64_t N, int64_t K,
-                        void* stream);
+                        void* workspace, int64_t workspace_bytes, void* stream);
 /* b packed [N/8, K] int32, nibble (n % 8) of word [n/8, k]; b8 = int8((q - z4[n,kg]) * s4[n,kg]).
  * ref: quantization/w4a8_kernel.py:317-448 */
 /* workspace: at least N*K bytes (the expanded int8 weights); with round16(N*K) +

@@ -41,7 +41,7 @@ SIGNATURES = {
     "llmk_gemm_fp8_block": [_p, _p, _p, _p, _p, _i, _l, _l, _l, _p, _l, _p],
     "llmk_gemm_fp8_block_static": [_p, _p, _p, _p, _p, _i, _l, _l, _l, _p],
     "llmk_gemm_i8_block": [_p, _p, _p, _p, _i, _p, _i, _l, _l, _l, _p, _l, _p],
-    "llmk_gemm_i8_rowcol": [_p, _p, _p, _p, _p, _i, _p, _l, _l, _l, _p],
+    "llmk_gemm_i8_rowcol": [_p, _p, _p, _p, _p, _i, _p, _l, _l, _l, _p, _l, _p],
     "llmk_gemm_w4a8": [_p, _p, _p, _p, _i, _p, _p, _p, _i, _l, _l, _l, _i, _p, _l, _p],
     "llmk_gemm_w4a16_marlin_workspace_bytes": [_l, _l, _l],
     "llmk_gemm_w4a16_marlin": [_p, _p, _p, _p, _l, _l, _l, _i, _p, _l, _p],

@@ -98,7 +98,8 @@ extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t
 }
 
 extern "C" int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, const float* b_s, void* c,
-                                   int c_dtype, int32_t* c_i32, int64_t M, int64_t N, int64_t K, void* stream) {
+                                   int c_dtype, int32_t* c_i32, int64_t M, int64_t N, int64_t K, void* workspace,
+                                   int64_t workspace_bytes, void* stream) {
     int rc = check_common("gemm_i8_rowcol", a, b, M, N, K, c_dtype);
     if (rc) return rc;
     if (M == 0 || N == 0) return LLMK_OK;
@@ -108,7 +109,16 @@ extern "C" int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.c_i32 = c_i32; p.a_s = a_s; p.b_s = b_s;
     p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
     // large M: the tile kernels accumulate int32 over the whole K range inside the MFMA and scale in the epilogue
-    if (M > 64 && dma_eligible(p)) return launch_dma<K_I8_ROWCOL, false>(p, (hipStream_t)stream, "gemm_i8_rowcol(tiled)");
+    if (M > 64 && dma_eligible(p)) {
+        // few tiles and a long K: K slices over the CUs, int32 partial sums in the workspace, one pass that adds
+        // them as integers and scales (same bits as the unsplit kernel)
+        const int z = splitk_factor(M, N, K);
+        if (z > 1 && workspace && workspace_bytes >= (int64_t)z * M * N * 4 && !((uintptr_t)workspace & 15)) {
+            p.partial = (float*)workspace;
+            p.ksplit = z;
+        }
+        return launch_dma<K_I8_ROWCOL, false>(p, (hipStream_t)stream, "gemm_i8_rowcol(tiled)");
+    }
     return launch_direct<K_I8_ROWCOL, false>(p, (int)M, (hipStream_t)stream, "gemm_i8_rowcol");
 }
 

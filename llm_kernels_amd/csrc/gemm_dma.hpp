@@ -555,8 +555,12 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             if (nv <= 0) continue;
             const int64_t off = (int64_t)m * N + nbh;
             if constexpr (KIND == K_I8_ROWCOL) {
-                rowcol_epilogue8(p, acc[i][2 * h], acc[i][2 * h + 1], m, off, nbh, nv);
-                if (!p.c) continue;
+                // (a K slice leaves its int32 sums, bit for bit, in the fp32 partial buffer: the summing pass
+                // adds them as integers and scales once, so the result does not depend on the split)
+                if (!split) {
+                    rowcol_epilogue8(p, acc[i][2 * h], acc[i][2 * h + 1], m, off, nbh, nv);
+                    if (!p.c) continue;
+                }
             }
             if (cdt == LLMK_BF16) store_run8<LLMK_BF16>(cout, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
             else if (cdt == LLMK_F16) store_run8<LLMK_F16>(cout, off, acc[i][2 * h], acc[i][2 * h + 1], nv, vec_ok);
@@ -594,6 +598,49 @@ __global__ void splitk_sum_kernel(const float* __restrict__ partial, void* __res
     }
 }
 
+// The same for the per-token x per-channel int8 kind: the partials are int32 sums over K slices; they are
+// added as integers (exactly what one workgroup over all of K would have held), written out raw when the
+// caller asked for them, and scaled by a_s[m] * b_s[n] into the output dtype.
+template <int ODT>
+__global__ void splitk_sum_rowcol_kernel(const int32_t* __restrict__ partial, DirectArgs p, int64_t mn, int z) {
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= mn) return;
+    const float* as = (const float*)p.a_s;
+    const float* bs = (const float*)p.b_s;
+    if (p.N % 4 == 0) {                       // the four elements share a row, every slice is 16-byte aligned
+        v4i s = {0, 0, 0, 0};
+        int k = 0;
+        for (; k + 4 <= z; k += 4) {
+            v4i t[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) t[j] = *(const v4i*)(partial + (int64_t)(k + j) * mn + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s += t[j];
+        }
+        for (; k < z; ++k) s += *(const v4i*)(partial + (int64_t)k * mn + i);
+        if (p.c_i32) {
+            if ((((uintptr_t)p.c_i32) & 15) == 0) *(v4i*)(p.c_i32 + i) = s;
+            else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) p.c_i32[i + q] = s[q];
+            }
+        }
+        if (p.c) {
+            const int m = (int)(i / p.N), n = (int)(i % p.N);
+            const float am = as[m];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) FloatIO<ODT>::st(p.c, i + q, (float)s[q] * am * bs[n + q]);
+        }
+    } else {
+        for (int64_t j = i; j < min(i + 4, mn); ++j) {
+            int s = 0;
+            for (int k = 0; k < z; ++k) s += partial[(int64_t)k * mn + j];
+            if (p.c_i32) p.c_i32[j] = s;
+            if (p.c) FloatIO<ODT>::st(p.c, j, (float)s * as[j / p.N] * bs[j % p.N]);
+        }
+    }
+}
+
 // fp16 / bf16 activation scales -> fp32 (the pipeline above streams 4-byte scale elements)
 template <int SDT>
 __global__ void scales_to_f32_kernel(const void* __restrict__ src, float* __restrict__ dst, int64_t n) {
@@ -624,6 +671,14 @@ int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     if (split) {
         const int64_t mn = (int64_t)p.M * p.N;
         const unsigned blocks = (unsigned)cdiv64(cdiv64(mn, 4), 256);
+        if constexpr (KIND == K_I8_ROWCOL) {
+            const int32_t* part = (const int32_t*)p.partial;
+            if (p.c_dtype == LLMK_BF16) splitk_sum_rowcol_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(part, p, mn, p.ksplit);
+            else if (p.c_dtype == LLMK_F16) splitk_sum_rowcol_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(part, p, mn, p.ksplit);
+            else splitk_sum_rowcol_kernel<LLMK_F32><<<blocks, 256, 0, stream>>>(part, p, mn, p.ksplit);
+            LLMK_CHECK_LAUNCH(name);
+            return LLMK_OK;
+        }
         if (p.c_dtype == LLMK_BF16) splitk_sum_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
         else if (p.c_dtype == LLMK_F16) splitk_sum_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);
         else splitk_sum_kernel<LLMK_F32><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, p.ksplit);

@@ -103,6 +103,8 @@ def int8_gemm_per_token(a, a_s, b, b_s, return_int32: bool = False):
     assert a_s.numel() == M and b_s.numel() == N, 'need one scale per token and per output channel'
     c = a.new_empty(*a.size()[:-1], N, dtype=torch.get_default_dtype())
     acc = a.new_empty(*a.size()[:-1], N, dtype=torch.int32) if return_int32 else None
+    # (only the K split of mid-size M uses scratch here)
+    ws = _lib.gemm_workspace(a.device, M, N, K) if M <= 512 else (None, 0)
     _lib.call("llmk_gemm_i8_rowcol", _lib.ptr(a), _lib.ptr(a_s), _lib.ptr(b), _lib.ptr(b_s), _lib.ptr(c),
-              _lib.dt(c.dtype), _lib.ptr(acc), M, N, K, _lib.stream(a), exc=AssertionError)
+              _lib.dt(c.dtype), _lib.ptr(acc), M, N, K, *ws, _lib.stream(a), exc=AssertionError)
     return (c, acc) if return_int32 else c

@@ -108,7 +108,8 @@ def test_int8_block_accumulators_bit_exact(dev, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (16, 4096, 4096), (130, 200, 1024), (128, 4096, 14336),
                                    (65, 136, 128), (300, 264, 640), (1000, 521, 1152), (2048, 4096, 2048),
-                                   (4096, 4096, 1024), (3850, 4110, 640)])
+                                   (4096, 4096, 1024), (3850, 4110, 640),
+                                   (300, 1000, 8192), (70, 1001, 8192), (100, 2050, 4096)])   # K split into 7, 8, 4
 def test_int8_per_token_int32_bit_exact(dev, M, N, K):
     announce("int8 rowcol", M, N, K)
     torch.manual_seed(M + K)
@@ -118,6 +119,12 @@ def test_int8_per_token_int32_bit_exact(dev, M, N, K):
         c, acc = int8_kernel.int8_gemm_per_token(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev), return_int32=True)
     assert acc.dtype == torch.int32 and torch.equal(acc.cpu(), g.int8_gemm_int32(a, b))
     assert_close_scaled(c, g.int8_gemm_rowcol(a, a_s, b, b_s), what="int8 rowcol")
+    # without scratch the entry point cannot split K: the slices' integer sums must give the same bits
+    ad, bd, asd, bsd = a.to(dev), b.to(dev), a_s.to(dev).float().contiguous(), b_s.to(dev).float().contiguous()
+    c0 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    _lib.call("llmk_gemm_i8_rowcol", _lib.ptr(ad), _lib.ptr(asd), _lib.ptr(bd), _lib.ptr(bsd), _lib.ptr(c0),
+              _lib.dt(c0.dtype), None, M, N, K, None, 0, _lib.stream(ad))
+    assert torch.equal(c0, c), "int8 rowcol: split and unsplit K differ"
     with default_dtype(torch.float32):     # scaled output alone (no accumulator buffer), full-range operands
         a2 = torch.randint(-128, 128, (M, K), dtype=torch.int8)
         b2 = torch.randint(-128, 128, (N, K), dtype=torch.int8)
