@@ -177,10 +177,13 @@ def _w4a16_check(C, A, w_deq_kn, what, seed=0):
     return ref, rows
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 4096, 4096), (16, 28672, 4096), (128, 28672, 4096), (16, 4096, 14336)])
+CONFIG1_GRID = [(M, N, K) for (N, K) in [(4096, 4096), (14336, 4096), (28672, 4096), (4096, 14336)] for M in (16, 128, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", CONFIG1_GRID)
 def test_mul_bench_shapes(dev, M, N, K):
-    """simple-Marlin `mul` beyond the 2048 rows of the reference's own recipe (test.py:139-157), same inputs
-    recipe (randn * 0.1) and its 0.05 threshold on the sampled rows."""
+    """simple-Marlin `mul` on every shape of configuration 1, beyond the 2048 rows of the reference's own recipe
+    (test.py:139-157): same inputs recipe (randn * 0.1) and its 0.05 threshold on the sampled rows."""
     announce("marlin mul bench shape", M, N, K)
     torch.manual_seed(42)
     A = (torch.randn(M, K, device=dev) * 0.1).half()
@@ -195,11 +198,11 @@ def test_mul_bench_shapes(dev, M, N, K):
     assert (C[rows.to(dev)].cpu().double() - ref).abs().max() <= 0.05
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 4096, 4096), (128, 28672, 4096), (16, 128256, 4096), (4096, 14336, 4096),
-                                   (2048, 28672, 4096)])
+@pytest.mark.parametrize("M,N,K", CONFIG1_GRID + [(16, 128256, 4096), (2048, 28672, 4096)])
 def test_w4a16_nk_bench_shapes(dev, M, N, K):
-    """Configuration 1 layout ([N, K/8] bit-packed, s = absmax / 7) at M = 4096 and the widest weights; the last two
-    take two or more rounds of 256 x 256 tiles and run on the tile kernel that expands the packed words itself."""
+    """Configuration 1 layout ([N, K/8] bit-packed, s = absmax / 7) on every shape of the configuration and the
+    widest weights; M = 4096 with N >= 14336 and the last shape take two or more rounds of 256 x 256 tiles and run on
+    the tile kernel that expands the packed words itself."""
     announce("w4a16 nk bench shape", M, N, K)
     torch.manual_seed(1)
     x = torch.randn(M, K, device=dev).half()
