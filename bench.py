@@ -263,7 +263,32 @@ class Case:
             def run():
                 return x.half().float() @ gemm_ref.w4a16_dequant_kn(q, s, 128).float()
         dt, self.cpu_passes = _timed_passes(run, CPU_BUDGET_S)
+        # the matmul alone, on weights dequantised beforehand (what a CPU deployment that keeps an fp32 copy pays)
+        xd, wd = self._cpu_dense(op, x, w)
+        self.cpu_matmul_s, _ = _timed_passes(lambda: xd @ wd, min(CPU_BUDGET_S, 1.5))
         return dt, rows
+
+    def _cpu_dense(self, op, x, w):
+        """(activations, dequantised weights^T) in fp32 for the matmul-only CPU figure (same operands)."""
+        from oracle import quant_ref, marlin_ref, gemm_ref
+        if op == "fp8":
+            a, a_s = quant_ref.act_quant_fp8(x.bfloat16())
+            b, b_s = quant_ref.weight_quant_fp8(w)
+            return a.float() * a_s.repeat_interleave(128, 1), quant_ref.weight_dequant_block(b, b_s).T.contiguous()
+        if op == "int8_pt":
+            xf, wf = x.bfloat16().float(), w.float()
+            sa, sb = xf.abs().amax(1) / 127.0, wf.abs().amax(1) / 127.0
+            return torch.round(xf / sa[:, None]) * sa[:, None], (torch.round(wf / sb[:, None]) * sb[:, None]).T.contiguous()
+        if op in ("int8", "w4a8"):
+            a, a_s = quant_ref.act_quant_int8(x.bfloat16(), rounding="away" if op == "int8" else "up")
+            ad = a.float() * a_s.float().repeat_interleave(128, 1)
+            if op == "int8":
+                b, b_s = quant_ref.weight_quant_int8(w)
+                return ad, quant_ref.weight_dequant_block(b, b_s).T.contiguous()
+            qq, s, s4, z4 = quant_ref.w4a8_weight_quant_levels(w)
+            return ad, quant_ref.w4a8_weight_dequant(qq, s, s4, z4).float().T.contiguous()
+        _, q, s = marlin_ref.fake_quantize(w.t().contiguous().half(), 128)
+        return x.half().float(), gemm_ref.w4a16_dequant_kn(q, s, 128).float()
 
 
 WORKLOADS = {}
@@ -280,7 +305,12 @@ MOE_WORKLOADS = {"moe_mixtral_fp8_t4096": ("fp8", 4096), "moe_mixtral_int8_t4096
 DEFAULT_WORKLOAD = "fp8_m4096_n4096_k4096"
 HEADLINE_SET = ["w4a16_m16_n4096_k4096", "w4a16_nk_m16_n4096_k4096", "w4a16_nk_m16_n28672_k4096", "fp8_m16_n4096_k4096", "fp8_m16_n28672_k4096", "fp8_m16_n4096_k14336",
                 "fp8_m16_n128256_k4096", "w4a16_nk_m16_n128256_k4096",
-                "w4a16_m4096_n4096_k4096", "w4a16_nk_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "int8_m4096_n14336_k4096", "int8_pt_m4096_n14336_k4096", "w4a8_m16_n4096_k4096", "moe_mixtral_fp8_t4096", "moe_mixtral_fp8_t16"]
+                "w4a16_m4096_n4096_k4096", "w4a16_nk_m4096_n4096_k4096", "fp8_m4096_n4096_k4096", "fp8_m4096_n28672_k4096",
+                "int8_m4096_n14336_k4096", "int8_pt_m4096_n14336_k4096",
+                # the mid-size rows of the benchmark grids (few tiles, cold weights): the weakest points
+                "fp8_m256_n4096_k4096", "fp8_m256_n4096_k14336", "int8_pt_m128_n4096_k4096", "w4a16_nk_m128_n4096_k4096",
+                "w4a8_m16_n4096_k4096", "w4a8_m128_n4096_k4096", "w4a8_m4096_n4096_k4096",
+                "moe_mixtral_fp8_t4096", "moe_mixtral_fp8_t16"]
 
 
 PREROLL_MS = 150.0        # untimed replays of the captured steps before anything is timed (clock and cache state settle)
@@ -421,11 +451,76 @@ def cpu_baseline(case, budget):
         return {"value": round(case.bytes / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": "host memcpy of the same size"}
     cpu_flops = case.flops * rows / case.T if case.op == "moe" else 2.0 * rows * case.N * case.K
-    return {"value": round(cpu_flops / dt / 1e12, 4), "unit": "TFLOP/s",
-            "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
-                      "1 warm-up + %d timed passes of %.3f s each, weight dequantisation included in every pass"
-                      % (rows, case.T if case.op == "moe" else case.M, getattr(case, "cpu_passes", 1), dt)}
+    out = {"value": round(cpu_flops / dt / 1e12, 4), "unit": "TFLOP/s",
+           "cores": torch.get_num_threads(), "kind": "port", "cpu_model": _cpu_model(),
+           "sample": "torch-CPU dequantize-then-matmul (fp32) of the same operands, first %d of %d rows, "
+                     "1 warm-up + %d timed passes of %.3f s each, weight dequantisation included in every pass"
+                     % (rows, case.T if case.op == "moe" else case.M, getattr(case, "cpu_passes", 1), dt)}
+    mm = getattr(case, "cpu_matmul_s", None)
+    if mm:
+        out["matmul_only_value"] = round(cpu_flops / mm / 1e12, 4)      # same unit; weights dequantised beforehand
+    return out
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or platform.machine()
+
+
+def calibration(dev):
+    """What this box sustains on the two resources the roofline prices against, from the library's calibration
+    kernels (llmk_calib_mfma: nothing but matrix instructions on random register operands, eight waves per CU;
+    llmk_calib_read: a read without arithmetic, linear and with the decode kernels' addresses, of 1 GiB, four
+    times the memory-side cache).  Reported beside the published peaks, never instead of them."""
+    from llm_kernels_amd import _lib
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    st = _lib.stream(torch.empty(1, device=dev))
+    out = torch.empty(cus * 512, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    res = {"cus": cus}
+
+    def timed(launch, reps=5):
+        launch()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            launch()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e-3)
+        return sorted(ts)[len(ts) // 2]
+
+    torch.manual_seed(0)
+    iters = 2000
+    kinds = (("fp8", _lib.KIND_FP8, 2 * 16 * 16 * 128, (torch.randn(65536, device=dev) * 0.5).to(torch.float8_e4m3fn)),
+             ("int8", _lib.KIND_I8, 2 * 16 * 16 * 64, torch.randint(-127, 128, (65536,), dtype=torch.int8, device=dev)),
+             ("f16", _lib.KIND_F16, 2 * 16 * 16 * 32, torch.randn(32768, device=dev).half()),
+             ("bf16", _lib.KIND_BF16, 2 * 16 * 16 * 32, torch.randn(32768, device=dev).bfloat16()))
+    for name, kind, flops_per_mfma, ops in kinds:
+        dt_s = timed(lambda: _lib.call("llmk_calib_mfma", kind, iters, _lib.ptr(ops), _lib.ptr(out), cus, _lib.ptr(clocks), st))
+        res["mfma_%s_sustained_tflops" % name] = round(cus * 8 * iters * 32 * flops_per_mfma / dt_s / 1e12, 1)
+        ck = clocks.tolist()
+        if ck[1] > 0:
+            res["mfma_%s_loop_ticks_per_100mhz_tick" % name] = round(ck[0] / ck[1], 3)
+    global _flush_buf
+    if _flush_buf is None:
+        _flush_buf = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    for name, pattern, wgs in (("hbm_read_linear_gbs", 0, cus * 8), ("hbm_read_decode_tiles_gbs", 1, cus)):
+        dt_s = timed(lambda: _lib.call("llmk_calib_read", _lib.ptr(_flush_buf), _flush_buf.numel(), pattern, _lib.ptr(sink), wgs, st))
+        res[name] = round(_flush_buf.numel() / dt_s / 1e9, 1)
+    res["note"] = ("sustained rates of this box by the library's calibration kernels; roofline.peak stays the published "
+                   "figure (HBM 8000 GB/s; fp8 / int8 5000, fp16 / bf16 2500 TFLOP/s)")
+    return res
 
 
 def main():
@@ -436,6 +531,7 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
     ap.add_argument("--headline-only", action="store_true", help="skip the other headline shapes (reported under 'cases')")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-calibration", action="store_true", help="skip the sustained-MFMA / HBM-read calibration kernels")
     ap.add_argument("--eager", action="store_true", help="launch every step from Python instead of replaying a HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -479,6 +575,7 @@ def main():
             torch.cuda.empty_cache()
 
     cpu = None if args.no_cpu else cpu_baseline(case, CPU_BUDGET_HEADLINE_S)
+    calib = None if args.no_calibration else calibration(dev)
 
     out = {
         "metric": "w4a16/fp8 GEMM TFLOPS & % roofline (HBM at M=16, MFMA at M=4096)",
@@ -492,7 +589,7 @@ def main():
                    "cache_flushed_before_each_replay": rec["cache_flushed_before_each_replay"],
                    "wall_ms_per_step": rec["wall_ms_per_step"], "alg_bytes": rec["alg_bytes"],
                    "flops": rec["flops"], "launch": "eager" if args.eager else "hip_graph"},
-        "roofline": rec["roofline"], "cpu_baseline": cpu,
+        "roofline": rec["roofline"], "cpu_baseline": cpu, "calibration": calib,
     }
     if cases:
         out["cases"] = cases

@@ -41,8 +41,8 @@ int         llmk_version(void);
 const char* llmk_last_error(void);
 /* Bytes of scratch llmk_gemm_fp8_block / _i8_block / _w4a8 / llmk_grouped_gemm can use for this shape
  * (0 = none; M = all rows of a grouped launch).  The scratch is optional: without it, or with less of it, a
- * slower kernel variant runs.  For M > 512 it ends with 64 MiB for the partial sums of a split last round of
- * tiles. */
+ * slower kernel variant runs.  For M > 512 and K >= 8192 it ends with 64 MiB for the partial sums of a split
+ * last round of tiles (shorter K is never split there). */
 int64_t     llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* ------------------------------------------------------------------ bit packing
@@ -115,12 +115,15 @@ int llmk_gemm_fp8_block(const void* a_e4m3, const float* a_s, const void* b_e4m3
                         void* c, int c_dtype, int64_t M, int64_t N, int64_t K,
                         void* workspace, int64_t workspace_bytes, void* stream);
 /* llmk_gemm_fp8_block for callers that cannot allocate device memory (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and
- * results (bit for bit) as llmk_gemm_fp8_block called with a workspace of llmk_gemm_workspace_bytes(M, N, K)
- * bytes, but the scratch is a device array built into the library (LLMK_STATIC_SCRATCH_BYTES per GPU, held
- * until the process ends); the call itself allocates and frees nothing.  Shapes whose scratch exceeds the
- * array fail with LLMK_ERR_SHAPE.  All calls on one GPU share the array: calls that may overlap on
- * different streams of that GPU race, issue them on one stream. */
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands as
+ * llmk_gemm_fp8_block, but the scratch is a device array built into the library (LLMK_STATIC_SCRATCH_BYTES per
+ * GPU, held until the process ends); the call itself allocates and frees nothing.  The array serves the
+ * activation scales / split-K / K-range partial sums, not the optional 64 MiB of a split last round of tiles:
+ * results equal llmk_gemm_fp8_block with a workspace of llmk_gemm_workspace_bytes(M, N, K) bytes bit for bit
+ * whenever that size holds no such 64 MiB (M <= 512 or K < 8192); beyond that the workspace entry may split its
+ * last round of tiles along K and the two differ in the fp32 summation order only (same tolerance against the
+ * oracle).  Shapes whose scratch exceeds the array fail with LLMK_ERR_SHAPE.  All calls on one GPU share
+ * the array: calls that may overlap on different streams of that GPU race, issue them on one stream. */
 #define LLMK_STATIC_SCRATCH_BYTES (32 << 20)
 int llmk_gemm_fp8_block_static(const void* a_e4m3, const float* a_s, const void* b_e4m3, const float* b_s,
                                void* c, int c_dtype, int64_t M, int64_t N, int64_t K, void* stream);
@@ -139,11 +142,12 @@ int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8_t* b, cons
                         void* workspace, int64_t workspace_bytes, void* stream);
 /* b packed [N/8, K] int32, nibble (n % 8) of word [n/8, k]; b8 = int8((q - z4[n,kg]) * s4[n,kg]).
  * ref: quantization/w4a8_kernel.py:317-448 */
-/* workspace: at least N*K bytes (the expanded int8 weights); with round16(N*K) +
- * llmk_gemm_workspace_bytes(M,N,K) bytes large M runs on the fast tile kernels.
- * Decode-size calls (small M, group_int4 == 128, 16-byte aligned a and b_packed) run one fused
- * kernel that reads the packed words once; it touches the workspace only for K > 4096 (fp32
- * partial sums of the K ranges, ceil(K / 4096) * M * N * 4 bytes). */
+/* workspace: llmk_gemm_w4a8_workspace_bytes(M, N, K, group_int4) bytes, 16-byte aligned, is what the path
+ * chosen for the shape uses (0 for decode-size calls with K <= 4096: small M, group_int4 == 128, 16-byte aligned a
+ * and b_packed run one fused kernel that reads the packed words once; fp32 partial sums of its K ranges,
+ * ceil(K / 4096) * M * N * 4 bytes, for K > 4096; otherwise the expanded int8 weights, round16(N*K), and behind
+ * them llmk_gemm_workspace_bytes(M,N,K) for the int8 tile kernels). */
+int64_t llmk_gemm_w4a8_workspace_bytes(int64_t M, int64_t N, int64_t K, int group_int4);
 int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, const void* b_s,
                    int s_dtype, const int8_t* b_s4, const int8_t* b_z4, void* c, int c_dtype,
                    int64_t M, int64_t N, int64_t K, int group_int4,
@@ -254,6 +258,20 @@ int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind, int c_dty
                       int64_t M, int64_t N, int64_t K, const int64_t* seg_indptr,
                       const int64_t* weight_indices, const void* scale_a, const void* scale_b,
                       int s_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ calibration (benchmark harness only)
+ * No counterpart in the reference and not on the product path: what the chip sustains on the two resources the
+ * GEMMs are priced against, for the same process that times them.
+ * llmk_calib_mfma: `workgroups` workgroups of eight waves, each wave `iters` x 32 matrix instructions of `kind`
+ * (LLMK_KIND_FP8: 16x16x128, LLMK_KIND_I8: 16x16x64, LLMK_KIND_F16 / BF16: 16x16x32) on register operands
+ * taken from `operands` (64 KiB of finite values of the operand type) into 32 independent accumulator tiles;
+ * out: workgroups * 512 floats (keeps the loop alive); clocks (optional): two int64, the s_memtime and the
+ * s_memrealtime (100 MHz) ticks the loop of one wave took.
+ * llmk_calib_read: reads nbytes (whole 64 KiB tiles) with no arithmetic, pattern 0 = linear stream, 1 = the
+ * address pattern of the weight-streaming GEMM kernels (16-row tiles of 4096-byte rows). */
+int llmk_calib_mfma(int kind, int iters, const void* operands, float* out, int workgroups, long long* clocks,
+                    void* stream);
+int llmk_calib_read(const void* src, int64_t nbytes, int pattern, int* sink, int workgroups, void* stream);
 
 #ifdef __cplusplus
 }

@@ -43,6 +43,7 @@ SIGNATURES = {
     "llmk_gemm_i8_block": [_p, _p, _p, _p, _i, _p, _i, _l, _l, _l, _p, _l, _p],
     "llmk_gemm_i8_rowcol": [_p, _p, _p, _p, _p, _i, _p, _l, _l, _l, _p, _l, _p],
     "llmk_gemm_w4a8": [_p, _p, _p, _p, _i, _p, _p, _p, _i, _l, _l, _l, _i, _p, _l, _p],
+    "llmk_gemm_w4a8_workspace_bytes": [_l, _l, _l, _i],
     "llmk_gemm_w4a16_marlin_workspace_bytes": [_l, _l, _l],
     "llmk_gemm_w4a16_marlin": [_p, _p, _p, _p, _l, _l, _l, _i, _p, _l, _p],
     "llmk_gemm_w4a16_nk": [_p, _p, _p, _p, _i, _l, _l, _l, _i, _p, _l, _p],
@@ -61,9 +62,11 @@ SIGNATURES = {
     "llmk_moe_pre_reorder_quant": [_p, _i, _p, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _l, _l, _p],
     "llmk_moe_post_reorder": [_p, _p, _i, _p, _p, _i, _p, _i, _i, _i, _i, _l, _l, _p],
     "llmk_moe_expert_scales": [_p, _p, _p, _i, _i, _l, _l, _l, _p, _p, _i, _p],
+    "llmk_calib_mfma": [_i, _i, _p, _p, _i, _p, _p],
+    "llmk_calib_read": [_p, _l, _i, _p, _i, _p],
     "llmk_grouped_gemm": [_p, _p, _p, _i, _i, _i, _l, _l, _l, _p, _p, _p, _p, _i, _p, _l, _p],
 }
-_RESTYPE = {"llmk_last_error": _c.c_char_p, "llmk_gemm_workspace_bytes": _l,
+_RESTYPE = {"llmk_last_error": _c.c_char_p, "llmk_gemm_workspace_bytes": _l, "llmk_gemm_w4a8_workspace_bytes": _l,
             "llmk_gemm_w4a16_marlin_workspace_bytes": _l}
 
 _lib = None
@@ -129,7 +132,9 @@ def gemm_workspace(device, M, N, K):
     if n <= 0:
         return None, 0
     buf = workspace(device, n)
-    return ptr(buf), buf.numel()
+    # the size asked for, not the size of the cached buffer: what a kernel does with its scratch (K splits) then
+    # depends on the shape alone, never on what an earlier call left behind
+    return ptr(buf), int(n)
 
 
 _ws = {}
@@ -149,5 +154,10 @@ def workspace(device, nbytes):
 def release_workspaces(device=None):
     """Drops the cached scratch buffers (of one device, or of all): the next call that needs scratch allocates
     again.  The memory goes back to torch's allocator once the launches that use it have run (stream-ordered)."""
-    for key in [k for k in _ws if device is None or k[0] == torch.device(device).index]:
+    index = None
+    if device is not None:
+        index = torch.device(device).index
+        if index is None:                      # "cuda" without an ordinal: the current device
+            index = torch.cuda.current_device()
+    for key in [k for k in _ws if index is None or k[0] == index]:
         del _ws[key]

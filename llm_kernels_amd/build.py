@@ -49,22 +49,17 @@ def _assembly(src):
     return out
 
 
+# what tells that a source hand-issues loads into registers: the loaders themselves, the header of the ring
+# kernels, or a tile-kernel kind whose weight rows are expanded from hand-loaded packed words
+_ASM_LOAD_MARKS = ('asm volatile("global_load_dword', "ring_load_", "asm_load_", "stream_ring.hpp",
+                   "K_W4NK", "K_W4MARLIN", "K_W4A8")
+
+
 def _has_asm_register_loads(src):
-    """True when the source (or a header of csrc/ it includes) issues register loads from inline asm."""
-    seen, todo = set(), [src]
-    while todo:
-        p = todo.pop()
-        if p in seen or not os.path.exists(p):
-            continue
-        seen.add(p)
-        text = open(p).read()
-        if "asm_load_" in text:
-            return True
-        for line in text.splitlines():
-            line = line.strip()
-            if line.startswith('#include "'):
-                todo.append(os.path.join(CSRC, line.split('"')[1]))
-    return False
+    """True when this source itself names hand-issued register loads (directly, by including the ring header, or
+    by instantiating a tile-kernel kind that uses them): its assembly must then show at least one."""
+    text = open(src).read()
+    return any(m in text for m in _ASM_LOAD_MARKS)
 
 
 def build(jobs=None, verbose=True):
@@ -73,19 +68,21 @@ def build(jobs=None, verbose=True):
     srcs = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
     jobs = jobs or min(8, len(srcs))
     # Kernels that load registers from inline asm are only correct while the compiler never touches the
-    # destination before the hand-placed wait: prove it on the assembly of this very build, or fail.
-    asm_srcs = [s for s in srcs if _has_asm_register_loads(s)]
+    # destination before the hand-placed wait: prove it on the assembly of this very build, or fail.  EVERY
+    # source is checked (a source without such loads has nothing to flag); a source whose text, or a header it
+    # includes, contains hand-issued loads must show at least one in its assembly, otherwise the check has gone blind.
     with cf.ThreadPoolExecutor(jobs) as ex:
-        asm_jobs = [ex.submit(_assembly, s) for s in asm_srcs]
+        asm_jobs = [(s, ex.submit(_assembly, s)) for s in srcs]
         objs = list(ex.map(_compile, srcs))
         checked = 0
-        for j in asm_jobs:
+        for src, j in asm_jobs:
             n, problems = check_asm.check_file(j.result())
             checked += n
             if problems:
                 raise RuntimeError("hand-issued register loads are not safe in this build:\n  " + "\n  ".join(problems[:20]))
-    if asm_srcs and checked == 0:
-        raise RuntimeError("check_asm found no hand-issued loads in %s: the check no longer sees them" % asm_srcs)
+            if n == 0 and _has_asm_register_loads(src):
+                raise RuntimeError("check_asm found no hand-issued loads in %s although its text has them: the check "
+                                   "no longer sees them" % src)
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

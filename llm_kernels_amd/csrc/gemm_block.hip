@@ -62,8 +62,9 @@ static int64_t workspace_core_bytes(int64_t M, int64_t N, int64_t K) {
 }
 
 extern "C" int64_t llmk_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    // more than 512 rows: room for the partial sums of a split last round of 256-column tiles behind the rest
-    return workspace_core_bytes(M, N, K) + (K > 0 && M > 512 ? w_tail_bytes() : 0);
+    // more than 512 rows and at least W_TAIL_MIN_KT K steps of 128 bytes (shorter tiles are never split): room for
+    // the partial sums of a split last round of 256-column tiles behind the rest
+    return workspace_core_bytes(M, N, K) + (K >= W_TAIL_MIN_KT * 128 && M > 512 ? w_tail_bytes() : 0);
 }
 
 extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* b, const float* b_s, void* c,

@@ -434,6 +434,37 @@ int launch_w4a8_stream(W4A8Args p, void* workspace, int64_t workspace_bytes, hip
 
 }  // namespace
 
+// Which path a shape takes (pointer alignment aside) and the scratch that path uses.
+namespace {
+struct W4A8Plan {
+    bool stream;          // fused decode kernel
+    int64_t nz;           // its K ranges
+    int64_t bytes;        // scratch the chosen path uses
+};
+W4A8Plan w4a8_plan(int64_t M, int64_t N, int64_t K, int group_int4) {
+    W4A8Plan pl{false, 1, 0};
+    if (M <= 0 || N <= 0 || K <= 0) return pl;
+    // Measured on MI355X with x = N * K / 4096^2: the fused kernel takes about 5 + 3.4 x microseconds per 32 rows
+    // of M; expanding to int8 and running the int8 GEMM about 26 + 3.6 x for x <= 4 and more beyond.
+    const double x = (double)N * (double)K / (4096.0 * 4096.0);
+    const int64_t row_blocks = (M + 31) / 32;
+    const bool fused_wins = row_blocks <= 2 || (row_blocks == 3 && x <= 3.0) || (row_blocks == 4 && x <= 2.0);
+    // K > 4096 runs as ranges of at most 4096 with fp32 partial sums in the workspace (up to 64 rows)
+    pl.nz = (K / 128 + 31) / 32;
+    const bool long_k_ok = pl.nz == 1 || row_blocks <= 2;
+    // (the hand-issued loads of the fused kernel take 32-bit lane offsets into the activations and the tables)
+    const bool small_offsets = M * K < (1ll << 32) && N * (K / 128) < (1ll << 32);
+    pl.stream = fused_wins && long_k_ok && small_offsets && group_int4 == 128;
+    if (pl.stream) pl.bytes = pl.nz > 1 ? pl.nz * M * N * 4 : 0;
+    else pl.bytes = ((N * K + 15) & ~(int64_t)15) + llmk_gemm_workspace_bytes(M, N, K);
+    return pl;
+}
+}  // namespace
+
+extern "C" int64_t llmk_gemm_w4a8_workspace_bytes(int64_t M, int64_t N, int64_t K, int group_int4) {
+    return w4a8_plan(M, N, K, group_int4).bytes;
+}
+
 extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b_packed, const void* b_s, int s_dtype,
                               const int8_t* b_s4, const int8_t* b_z4, void* c, int c_dtype, int64_t M, int64_t N,
                               int64_t K, int group_int4, void* workspace, int64_t workspace_bytes, void* stream) {
@@ -442,17 +473,9 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
     if (group_int4 < 4 || group_int4 % 4 || K % group_int4) LLMK_FAIL(LLMK_ERR_SHAPE, "gemm_w4a8: group_int4=%d must divide K and be a multiple of 4", group_int4);
     if (M == 0 || N == 0) return LLMK_OK;
     if (!a || !a_s || !b_packed || !b_s || !b_s4 || !b_z4 || !c) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a8: null pointer");
-    // Measured on MI355X with x = N * K / 4096^2: the fused kernel takes about 5 + 3.4 x microseconds per 32 rows
-    // of M; expanding to int8 and running the int8 GEMM about 26 + 3.6 x for x <= 4 and more beyond.
-    const double x = (double)N * (double)K / (4096.0 * 4096.0);
-    const int64_t row_blocks = (M + 31) / 32;
-    const bool fused_wins = row_blocks <= 2 || (row_blocks == 3 && x <= 3.0) || (row_blocks == 4 && x <= 2.0);
-    // K > 4096 runs as ranges of at most 4096 with fp32 partial sums in the workspace (up to 64 rows)
-    const int64_t nz = (K / 128 + 31) / 32;
-    const bool long_k_ok = nz == 1 || (row_blocks <= 2 && workspace && workspace_bytes >= nz * M * N * 4 && !(((uintptr_t)workspace) & 15));
-    // (the hand-issued loads of the fused kernel take 32-bit lane offsets into the activations and the tables)
-    const bool small_offsets = M * K < (1ll << 32) && N * (K / 128) < (1ll << 32);
-    if (fused_wins && long_k_ok && small_offsets && group_int4 == 128 && !(((uintptr_t)a | (uintptr_t)b_packed) & 15)) {
+    const W4A8Plan pl = w4a8_plan(M, N, K, group_int4);
+    const bool ranges_ok = pl.nz == 1 || (workspace && workspace_bytes >= pl.nz * M * N * 4 && !(((uintptr_t)workspace) & 15));
+    if (pl.stream && ranges_ok && !(((uintptr_t)a | (uintptr_t)b_packed) & 15)) {
         W4A8Args p{a, a_s, b_packed, b_s, b_s4, b_z4, c, c_dtype, (int)M, (int)N, (int)K, 0, nullptr};
         if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: c_dtype %d", c_dtype);
         hipStream_t st = (hipStream_t)stream;

@@ -38,10 +38,17 @@ def w4a16_gemm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, gr
     assert w_packed.size(1) * 8 == K, 'packed weight must be [N, K/8]'
     y = x.new_empty(*x.size()[:-1], N)
     assert x.dtype in (torch.float16, torch.bfloat16), 'activations must be fp16 or bf16'
-    steps, nz = K // 128, -(-(K // 128) // 32)
-    # bf16 at decode size runs on the weight-streaming kernel when its K ranges come in whole four-step shares
-    bf_decode = (x.dtype == torch.bfloat16 and M <= 64 and group_size == 128 and steps % 4 == 0
-                 and (-(-steps // nz)) % 4 == 0 and scales.data_ptr() % 8 == 0)
+    # bf16 at decode size runs on the weight-streaming ring kernel under exactly the conditions the library
+    # checks (128-wide groups, K ranges of at most 32 steps in whole four-step shares, 8-byte aligned scale rows
+    # and outputs, 32-bit lane offsets, and with more than one K range M * N % 4 == 0 for the summing pass);
+    # every other bf16 call goes through the bf16 copy of W and needs room for it
+    steps = K // 128
+    nz = max(1, -(-steps // 32))
+    per = -(-steps // nz)
+    ring_ok = (group_size == 128 and per <= 32 and steps % 4 == 0 and per % 4 == 0 and scales.data_ptr() % 8 == 0
+               and N * (K // 2) < (1 << 32) and M * K * 2 < (1 << 32))
+    bf_decode = (x.dtype == torch.bfloat16 and M <= 64 and ring_ok and y.data_ptr() % 8 == 0
+                 and (nz == 1 or (M * N) % 4 == 0))
     if M > 64 or (x.dtype == torch.bfloat16 and not bf_decode):
         # fp16 / bf16 copy of W for the compute-bound path, split-K partials behind it for mid-size M
         ws = _lib.workspace(x.device, ((N * K * 2 + 255) // 256) * 256 + (8 * M * N * 4 if M <= 512 else 0))

@@ -69,8 +69,9 @@ def weight_dequant(y: torch.Tensor, s: torch.Tensor, s4: torch.Tensor, z4: torch
     Mp, K = y.size()
     N = Mp * (PACKING_BITS // W_BITS)
     out = torch.empty((N, K), dtype=torch.float16, device=y.device)
-    _lib.call("llmk_weight_dequant_w4a8", _lib.ptr(y), _lib.ptr(s.contiguous()), _lib.ptr(s4.contiguous()),
-              _lib.ptr(z4.contiguous()), _lib.ptr(out), N, K, block_size, group_size_int4, _lib.stream(y))
+    s, s4, z4 = s.contiguous(), s4.contiguous(), z4.contiguous()      # named: alive until the launch is queued
+    _lib.call("llmk_weight_dequant_w4a8", _lib.ptr(y), _lib.ptr(s), _lib.ptr(s4), _lib.ptr(z4), _lib.ptr(out),
+              N, K, block_size, group_size_int4, _lib.stream(y))
     return out
 
 
@@ -90,9 +91,11 @@ def w4a8_gemm(a: torch.Tensor, a_s: torch.Tensor, b: torch.Tensor,
     N = b.size(0) * elements_per_sample
     assert a_s.dtype == b_s.dtype, 'activation and weight scales must share a dtype'
     c = a.new_empty(*a.size()[:-1], N, dtype=torch.get_default_dtype())
-    # expanded int8 weights, then the scratch of the int8 GEMM behind them
-    ws = _lib.workspace(a.device, ((N * K + 15) // 16) * 16 + max(0, _lib.load().llmk_gemm_workspace_bytes(M, N, K)))
+    # what this shape's kernels use: nothing for the fused decode kernel with K <= 4096, fp32 partial sums for its
+    # K ranges or the K slices of the fused tile kernels, the expanded int8 weights + the int8 GEMM's scratch otherwise
+    need = _lib.load().llmk_gemm_w4a8_workspace_bytes(M, N, K, GROUP_SIZE_INT4)
+    ws = _lib.workspace(a.device, need) if need > 0 else None
     _lib.call("llmk_gemm_w4a8", _lib.ptr(a), _lib.ptr(a_s), _lib.ptr(b), _lib.ptr(b_s), _lib.dt(a_s.dtype),
               _lib.ptr(b_s4), _lib.ptr(b_z4), _lib.ptr(c), _lib.dt(c.dtype), M, N, K, GROUP_SIZE_INT4,
-              _lib.ptr(ws), ws.numel(), _lib.stream(a), exc=AssertionError)
+              _lib.ptr(ws), need if ws is not None else 0, _lib.stream(a), exc=AssertionError)
     return c

@@ -299,39 +299,102 @@ def test_router(dev):
     assert torch.equal(ids.cpu(), oids) and torch.allclose(w.cpu(), ow, atol=1e-6)
 
 
-def test_ep_moe_forward_mixtral_dims_full_size(dev):
-    """8 experts, hidden 4096, intermediate 14336, 4096 tokens, top-2, fp8 128x128 weights.
+def _oracle_rows(a_rows, s_rows, w, ws, chunk=8192):
+    """gemm_blockwise of a few activation rows against one expert's weights, over column chunks of the weights
+    (bounds the float64 temporaries at Mixtral sizes)."""
+    N = w.shape[0]
+    out = []
+    for n0 in range(0, N, chunk):
+        n1 = min(N, n0 + chunk)
+        out.append(g.gemm_blockwise(a_rows, s_rows, w[n0:n1], ws[n0 // 128:(n1 + 127) // 128]))
+    return torch.cat(out, dim=-1)
 
-    Size-independent checks: (1) the rows of a 32-token subset must match the same forward run on the
-    subset alone (decode-sized kernels vs the large-M tiled kernels), (2) the subset run must match the
-    CPU oracle with every rounding point reproduced, (3) per-expert segment lengths equal the router's
-    histogram, (4) every output is finite.
+
+def _check_grouped_gemm_per_segment(c, a, a_s, w, ws, seg, what, seed=0):
+    """c [M, N] on the device against moe_ref.grouped_gemm's formula, expert by expert: the first, the last and two
+    random rows of every segment (all columns) at rtol = atol = 1e-2, and the column sums of the WHOLE segment
+    against a one-row oracle GEMM of the scale-weighted column sums of its activation rows (a wrong tile
+    anywhere in the segment moves them)."""
+    assert bool(torch.isfinite(c.float()).all()), what + ": non-finite output"
+    gen = torch.Generator().manual_seed(seed)
+    ah, ash, segl = a.cpu(), a_s.cpu(), seg.cpu().tolist()
+    K = ah.shape[1]
+    for e in range(len(segl) - 1):
+        m0, m1 = segl[e], segl[e + 1]
+        if m1 <= m0:
+            continue
+        rows = sorted({m0, m1 - 1, *(m0 + torch.randint(0, m1 - m0, (2,), generator=gen)).tolist()})
+        rt = torch.tensor(rows)
+        we, wse = w[e].cpu(), ws[e].cpu()
+        ref = _oracle_rows(ah[rt], ash[rt], we, wse)
+        assert_close_scaled(c[rt.to(c.device)], ref, what="%s expert %d rows %s" % (what, e, rows))
+        n = m1 - m0
+        wsum = (ah[m0:m1].float().double().reshape(n, K // 128, 128) * ash[m0:m1].double()[:, :, None]).sum(0).reshape(1, K)
+        want = _oracle_rows(wsum, torch.ones(1, K // 128, dtype=torch.float64), we.float(), wse)[0]
+        got = c[m0:m1].double().sum(0).cpu()
+        bound = 1e-2 * ref.pow(2).mean().sqrt().item() * (n ** 0.5) + 1e-2 * want.abs()
+        bad = (got - want).abs() > bound
+        assert not bad.any(), "%s expert %d: column checksum off in %d columns (max %.3e)" % (
+            what, e, int(bad.sum()), (got - want).abs().max().item())
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
+def test_ep_moe_mixtral_dims_full_size(dev, kind):
+    """8 experts, hidden 4096, intermediate 14336, 4096 tokens, top-2, 128x128 block-scaled weights (the MoE
+    benchmark workloads, fp8 and int8).
+
+    (1) Each of the two grouped GEMMs alone, on the operands the forward feeds it, against the oracle at
+        rtol = atol = 1e-2: sampled rows of every segment plus a checksum over every row of every segment.
+    (2) The whole forward on 256 sampled tokens against the CPU oracle with every rounding point reproduced
+        (the forward is separable by token); two chained GEMMs with a requantisation in between, where one ulp of
+        the bf16 intermediate can flip an 8-bit code, hence the wider end-to-end bound.
+    (3) Per-expert segment lengths equal the router's histogram; every output is finite.
     """
-    announce("ep_moe_forward mixtral full size")
+    announce("ep_moe mixtral full size", kind)
     torch.manual_seed(11)
     T, H, I, E, topk = 4096, 4096, 14336, 8, 2
-    w13 = torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
-    w13s = torch.empty(E, 2 * I // 128, H // 128, dtype=torch.float32, device=dev)
-    w2 = torch.empty(E, H, I, dtype=torch.float8_e4m3fn, device=dev)
-    w2s = torch.empty(E, H // 128, I // 128, dtype=torch.float32, device=dev)
+    fp8 = kind == "fp8"
+    qdt = torch.float8_e4m3fn if fp8 else torch.int8
+    sdt = torch.float32 if fp8 else torch.float16
+    wq = fp8_kernel.weight_quant if fp8 else int8_kernel.weight_quant
+    w13 = torch.empty(E, 2 * I, H, dtype=qdt, device=dev)
+    w13s = torch.empty(E, 2 * I // 128, H // 128, dtype=sdt, device=dev)
+    w2 = torch.empty(E, H, I, dtype=qdt, device=dev)
+    w2s = torch.empty(E, H // 128, I // 128, dtype=sdt, device=dev)
     for e in range(E):
-        w13[e], w13s[e] = fp8_kernel.weight_quant(torch.randn(2 * I, H, device=dev) * 0.02)
-        w2[e], w2s[e] = fp8_kernel.weight_quant(torch.randn(H, I, device=dev) * 0.02)
+        w13[e], w13s[e] = wq(torch.randn(2 * I, H, device=dev) * 0.02)
+        w2[e], w2s[e] = wq(torch.randn(H, I, device=dev) * 0.02)
     x = torch.randn(T, H, device=dev).bfloat16()
     ids, wts = softmax_topk_router(torch.randn(T, E, device=dev), topk)
-    out = ep_moe_forward(x, ids, wts, w13, w2, w13s, w2s, block_shape=[128, 128])
-    assert out.shape == (T, H) and torch.isfinite(out.float()).all()
-    _, _, seg = gk.run_moe_ep_preproess(ids, E)
+    rids, src2dst, seg = gk.run_moe_ep_preproess(ids, E)
     assert (seg[1:] - seg[:-1]).tolist() == torch.bincount(ids.flatten(), minlength=E).tolist()
+    widx = torch.arange(E, device=dev)
 
-    sub = torch.arange(0, T, T // 32, device=dev)[:32]
-    out_sub = ep_moe_forward(x[sub].contiguous(), ids[sub].contiguous(), wts[sub].contiguous(), w13, w2, w13s, w2s,
-                             block_shape=[128, 128])
-    # both runs quantise the same rows identically; only the fp32 summation order inside the GEMMs differs
-    assert_close_scaled(out[sub], out_sub.float(), rtol=3e-2, atol=3e-2, what="full vs subset")
+    # (1) gate / up projection: 8192 x 28672 x 4096
+    a1, a1s = gk.pre_reorder_quant(x, src2dst, ids, None, 0, E - 1, topk, H, qdt)
+    gu = torch.empty(T * topk, 2 * I, dtype=torch.bfloat16, device=dev)
+    gk.grouped_gemm_triton(a1, w13, gu, E, True, seg, widx, False, a1s, w13s, [128, 128])
+    _check_grouped_gemm_per_segment(gu, a1, a1s, w13, w13s, seg, "mixtral %s gate/up" % kind, seed=1)
+    # down projection: 8192 x 4096 x 14336
+    a2, a2s = gk.act_and_mul_quant(gu, 2 * I, rids, None, 0, E - 1, qdt, "silu")
+    do = torch.empty(T * topk, H, dtype=torch.bfloat16, device=dev)
+    gk.grouped_gemm_triton(a2, w2, do, E, True, seg, widx, False, a2s, w2s, [128, 128])
+    _check_grouped_gemm_per_segment(do, a2, a2s, w2, w2s, seg, "mixtral %s down" % kind, seed=2)
+    del a1, a1s, a2, a2s, gu, do
+
+    # (2) whole forward, 256 sampled tokens against the oracle
+    out = ep_moe_forward(x, ids, wts, w13, w2, w13s, w2s, block_shape=[128, 128])
+    assert out.shape == (T, H) and bool(torch.isfinite(out.float()).all())
+    sub = torch.arange(0, T, T // 256, device=dev)[:256]
+    aq = q.act_quant_fp8 if fp8 else q.act_quant_int8
     ref = m.ep_moe_forward(x[sub].cpu(), ids[sub].cpu(), wts[sub].cpu(), w13.cpu(), w13s.cpu(), w2.cpu(), w2s.cpu(),
-                           q.act_quant_fp8, dtype=torch.bfloat16)
-    assert_close_scaled(out_sub, ref, rtol=5e-2, atol=5e-2, what="subset vs oracle")
+                           aq, dtype=torch.bfloat16)
+    assert_close_scaled(out[sub], ref, rtol=5e-2, atol=5e-2, what="mixtral %s forward, 256 tokens vs oracle" % kind)
+    # the same tokens through the decode-sized kernels (a 32-token forward) agree with the large-M run
+    sub32 = sub[::8]
+    out_sub = ep_moe_forward(x[sub32].contiguous(), ids[sub32].contiguous(), wts[sub32].contiguous(), w13, w2, w13s, w2s,
+                             block_shape=[128, 128])
+    assert_close_scaled(out[sub32], out_sub.float(), rtol=3e-2, atol=3e-2, what="full vs 32-token run")
 
 
 # ------------------------------------------------------------------ fused permute / activation + quantisation

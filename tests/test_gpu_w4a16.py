@@ -256,7 +256,9 @@ def test_w4a16_without_scratch(dev, M, N, K):
 @pytest.mark.parametrize("M,N,K,gs", [(16, 4096, 4096, 128), (1, 256, 512, 128), (7, 1000, 1024, 128), (40, 520, 2048, 128),
                                       (16, 28672, 4096, 128), (16, 1032, 14336, 128), (64, 264, 8192, 128),
                                       (16, 256, 384, 128), (33, 300, 4608, 128), (16, 512, 1024, 64), (20, 129, 512, 256),
-                                      (300, 1000, 512, 128), (2048, 4096, 1024, 128)])
+                                      (300, 1000, 512, 128), (2048, 4096, 1024, 128),
+                                      # K > 4096 with M * N not a multiple of 4: the ring kernel's summing pass does not take it
+                                      (1, 1001, 8192, 128), (3, 50257, 8192, 128)])
 def test_w4a16_nk_bf16(dev, M, N, K, gs):
     """bf16 activations / outputs for the [N, K/8] layout: the weight-streaming kernel at decode sizes (128-wide
     groups, whole four-step K shares), the bf16 copy of W plus the bf16 tile GEMM everywhere else."""

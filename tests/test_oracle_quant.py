@@ -134,6 +134,13 @@ def test_rowwise():
     x = torch.randn(9, 384)
     y, s = q.int8_quant_rowwise(x)
     assert (y.abs().amax(1) == 127).all() and s.dtype == torch.float32
+    # hand row with ties: absmax 127 -> s = 1.0 exactly, every .5 rounds away from zero
+    # (half-up would give -0.5 -> 0 and -1.5 -> -1, half-even 0.5 -> 0 and 2.5 -> 2)
+    y, s = q.int8_quant_rowwise(torch.tensor([[0.5, -0.5, 1.5, -1.5, 2.5, 127.0]]))
+    assert s.tolist() == [1.0] and y.tolist() == [[1, -1, 2, -2, 3, 127]] and y.dtype == torch.int8
+    # a second row with another scale: s = 63.5 / 127 = 0.5, ties at odd multiples of 0.25
+    y, s = q.int8_quant_rowwise(torch.tensor([[0.25, -0.25, 0.75, -1.25, 63.5, -63.5]]))
+    assert s.tolist() == [0.5] and y.tolist() == [[1, -1, 2, -3, 127, -127]]
 
 
 # ----------------------------------------------------------------- fp8 128x128 weight quantizer
