@@ -1,4 +1,5 @@
 // Dense block-scaled fp8 / int8 GEMM entry points.
+#include <algorithm>
 #include <mutex>
 
 #include "gemm_wide.hpp"
@@ -57,7 +58,8 @@ static int64_t workspace_core_bytes(int64_t M, int64_t N, int64_t K) {
         return nz > 1 ? (int64_t)nz * M * N * 4 : 0;
     }
     const int64_t scales = (M * (K / 128) * 4 + 255) & ~(int64_t)255;
-    const int z = splitk_factor(M, N, K);
+    int z = splitk_factor(M, N, K);
+    if (M <= 512) z = std::max(z, mid_plan(M, N, K).z);      // the mid-size kernel's K slices
     return scales + (z > 1 ? (int64_t)z * M * N * 4 : 0);
 }
 
@@ -113,6 +115,15 @@ extern "C" int llmk_gemm_i8_rowcol(const int8_t* a, const float* a_s, const int8
     if (M > 64 && dma_eligible(p)) {
         // few tiles and a long K: K slices over the CUs, int32 partial sums in the workspace, one pass that adds
         // them as integers and scales (same bits as the unsplit kernel)
+        if (mid_wanted(M, N, K)) {
+            MidPlan pl = mid_plan(M, N, K);
+            if (pl.z > 1 && !(workspace && workspace_bytes >= (int64_t)pl.z * M * N * 4 && !((uintptr_t)workspace & 15))) pl.z = 1;
+            if (mid_eligible<K_I8_ROWCOL>(p, pl.mt, pl.z)) {
+                if (pl.z > 1) { p.partial = (float*)workspace; p.ksplit = pl.z; }
+                return pl.mt == 4 ? launch_mid<K_I8_ROWCOL, 4>(p, (hipStream_t)stream, "gemm_i8_rowcol(mid)")
+                                  : launch_mid<K_I8_ROWCOL, 2>(p, (hipStream_t)stream, "gemm_i8_rowcol(mid)");
+            }
+        }
         const int z = splitk_factor(M, N, K);
         if (z > 1 && workspace && workspace_bytes >= (int64_t)z * M * N * 4 && !((uintptr_t)workspace & 15)) {
             p.partial = (float*)workspace;

@@ -15,7 +15,9 @@ namespace llmk {
 
 enum : int { K_FP8_BLOCK = 0, K_I8_BLOCK = 1, K_I8_ROWCOL = 2, K_F16 = 3, K_BF16 = 4,
              K_W4NK = 5,      // fp16 activations x 4-bit weights packed [N, K/8] (tile kernels only)
-             K_W4MARLIN = 6 };// the same with weights and scales in the Marlin layout
+             K_W4MARLIN = 6,  // the same with weights and scales in the Marlin layout
+             K_W4A8 = 7 };    // int8 activations x uint4 weights packed eight rows per word [N/8, K] with int8 zero
+                              // point and scale per (row, 128-K group) and 128 x 128 block scales (tile kernels only)
 
 __device__ __forceinline__ float ld_scale(const void* p, int64_t i, int dt) {
     if (dt == LLMK_F32) return ((const float*)p)[i];
@@ -70,7 +72,7 @@ __device__ __forceinline__ v4f step_dot(const v8i& a, const v8i& b) {
     const v4f z = {0.f, 0.f, 0.f, 0.f};
     if constexpr (KIND == K_FP8_BLOCK) {
         return mfma_fp8_16x16x128(a, b, z);
-    } else if constexpr (KIND == K_I8_BLOCK || KIND == K_I8_ROWCOL) {
+    } else if constexpr (KIND == K_I8_BLOCK || KIND == K_I8_ROWCOL || KIND == K_W4A8) {
         v4i zi = {0, 0, 0, 0};
         v4i a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]};
         v4i b0 = {b[0], b[1], b[2], b[3]}, b1 = {b[4], b[5], b[6], b[7]};
@@ -98,6 +100,8 @@ struct DirectArgs {
     int ksplit;            // 0 / 1 = no split
     int kc_steps;          // weight-streaming kernel with K ranges: 128-byte steps per range (gridDim.z ranges)
     int group;             // K_W4NK / K_W4MARLIN: K elements per fp16 group scale
+    const int8_t* w4_s4;   // K_W4A8: second-level scales [N, K/128]
+    const int8_t* w4_z4;   // K_W4A8: zero points [N, K/128]
     int tail_split;        // 256-column tile kernel: the tiles of a short last round are split along K (partial = scratch)
 };
 

@@ -94,6 +94,42 @@ __device__ __forceinline__ v4i w4_word_to_f16x8(unsigned w, v2h sc) {
     o[3] = (int)__builtin_amdgcn_perm(p37, p26, 0x07060302u);
     return o;
 }
+// ---- uint4 weights packed eight rows per word, dequantised to int8 (K_W4A8) ----
+// A word holds the nibbles of eight weight rows at one k.  b8 = int8(int8(q - z) * s) with two's-complement wrap is
+// the low byte of (q - z) * s in any wider arithmetic, i.e. of q * s + c with c = -(z * s): one packed 16-bit
+// multiply-add handles two rows of a word at once (row j in the low half, row j + 4 in the high half, each with
+// its own s and c), and byte permutes gather four consecutive k of a row into one dword.
+typedef unsigned short w4_us2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ w4_us2 w4_as_us2(unsigned u) { w4_us2 r; __builtin_memcpy(&r, &u, 4); return r; }
+__device__ __forceinline__ unsigned w4_us2_bits(w4_us2 v) { unsigned r; __builtin_memcpy(&r, &v, 4); return r; }
+// sp[j], cp[j]: (s, c) of rows j | j + 4 as 16-bit pairs, from the eight scale / zero-point bytes of a packed row
+__device__ __forceinline__ void w4a8_row_consts(uint2 sb, uint2 zb, unsigned (&sp)[4], unsigned (&cp)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const unsigned sel = 0x0c000c00u | (unsigned)j | ((unsigned)(4 + j) << 16);      // [byte j of .x, 0, byte j of .y, 0]
+        sp[j] = __builtin_amdgcn_perm(sb.y, sb.x, sel);
+        const unsigned zp = __builtin_amdgcn_perm(zb.y, zb.x, sel);
+        cp[j] = w4_us2_bits((w4_us2){0, 0} - w4_as_us2(zp) * w4_as_us2(sp[j]));
+    }
+}
+// four consecutive words (k, k + 1, k + 2, k + 3) of a packed row -> out[i] = the four int8 weights of row i at
+// those k (byte order = k order)
+__device__ __forceinline__ void w4a8_words_to_i8(const v4i& w, const unsigned (&sp)[4], const unsigned (&cp)[4], unsigned (&out)[8]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        unsigned r[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned x = (((unsigned)w[i]) >> (4 * j)) & 0x000f000fu;
+            r[i] = w4_us2_bits(w4_as_us2(x) * w4_as_us2(sp[j]) + w4_as_us2(cp[j]));
+        }
+        const unsigned t01 = __builtin_amdgcn_perm(r[1], r[0], 0x06020400u);
+        const unsigned t23 = __builtin_amdgcn_perm(r[3], r[2], 0x06020400u);
+        out[j] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+        out[j + 4] = __builtin_amdgcn_perm(t23, t01, 0x07060302u);
+    }
+}
+
 // Register loads issued from inline asm like the direct-to-LDS loads, so that they take part in the same
 // hand-counted vmcnt scheme (a compiler-tracked load would make the compiler wait for every load in flight).
 // The destination is only read behind an explicit s_waitcnt that names it as a read-write operand.  The
@@ -103,6 +139,11 @@ __device__ __forceinline__ v4i w4_word_to_f16x8(unsigned w, v2h sc) {
 __device__ __forceinline__ uint64_t asm_load_b64(uint32_t voff, const void* sbase) {
     uint64_t v;
     asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+__device__ __forceinline__ v4i asm_load_b128(uint32_t voff, const void* sbase) {
+    v4i v;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
     return v;
 }
 __device__ __forceinline__ unsigned asm_load_u16(uint32_t voff, const void* sbase) {
@@ -182,11 +223,16 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // K_W4NK: fp16 activations by direct-to-LDS loads as for K_F16; the weight rows of a stage are expanded
     // from the packed words by the threads themselves (one 8-byte load, 16 weights, two 16-byte LDS writes per
     // thread and K step), one K step behind the loads and one ahead of the multiplication.
-    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
+    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || KIND == K_W4A8);
     // K_W4MARLIN: the same for the Marlin layout (16-byte units of 32 values: 4 k x 8 columns): a thread takes
     // half a unit and scatters its eight fp16 pairs over the weight rows.
-    constexpr bool W4NK = (KIND == K_W4NK), W4M = (KIND == K_W4MARLIN), W4 = W4NK || W4M;
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4) ? 2 : 1;
+    // K_W4A8: int8 activations and block scales as for K_I8_BLOCK; the int8 weight rows of a stage are expanded
+    // from words that pack eight rows each: a thread loads four consecutive words of one packed row (16 bytes)
+    // and writes four int8 weights of each of the eight rows; the zero points and second-level scales of the
+    // tile's 128 rows for every K step sit in an LDS table filled before the pipeline starts.
+    constexpr bool W4NK = (KIND == K_W4NK), W4M = (KIND == K_W4MARLIN), W4A8 = (KIND == K_W4A8);
+    constexpr bool W4H = W4NK || W4M, W4 = W4H || W4A8;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4H) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
     const int KT_all = K >> 7;
@@ -270,6 +316,18 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         w4_soff = n * (uint32_t)(p.K / p.group) * 2u;                          // bytes into the scale matrix
         w4_lds = (uint32_t)R * 128u + (uint32_t)((2 * q) ^ ((R >> 1) & 7)) * 16u;   // chunk 2q; chunk 2q+1 is at ^16
     }
+    // K_W4A8: zero points and second-level scales of the tile, raw bytes [K step][row] behind the weight-scale table
+    uint8_t* w4tab = lds + D_NSTAGE * D_STAGE + D_MAX_KT * 4;
+    if constexpr (W4A8) {
+        // thread t: packed row pr = t >> 5 of the tile's sixteen, words 4 kc .. 4 kc + 3 (kc = t & 31) of the K step
+        const int pr = tid >> 5, kc = tid & 31, np = N >> 3;
+        w4_off = (uint32_t)min((n0 >> 3) + pr, np - 1) * (uint32_t)(p.K * 4) + (uint32_t)kc * 16u;
+        // the eight rows of a packed row are tile columns 8 pr + i; column c of a 64-column half sits in LDS row
+        // 32 (c >> 5) + 16 ((c >> 2) & 1) + 4 ((c >> 3) & 3) + (c & 3): rows i = 0..3 are consecutive LDS rows from
+        // `base`, rows 4..7 the same 16 LDS rows further on; every pair of rows shares the swizzle of `base`
+        const int ph = pr & 7, base = 64 * (pr >> 3) + 32 * (ph >> 2) + 4 * (ph & 3);
+        w4_lds = (uint32_t)base | ((uint32_t)kc << 16) | ((uint32_t)pr << 24);
+    }
 
     // the same loads in two bursts for the block-scaled kinds on the taller tiles: activation rows before the
     // step is multiplied, weight rows and scale column between its two phases (the buffer they go to was
@@ -309,7 +367,9 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // variables of the exact register width, so that no widening move is ever placed between load and wait)
     uint64_t w4_words = 0, w4_scale = 0;
     unsigned w4_scale16 = 0;
+    v4i w4_words4 = {0, 0, 0, 0};
     auto w4_request = [&](int kt) {
+        if constexpr (W4A8) w4_words4 = asm_load_b128(w4_off, (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 512);
         if constexpr (W4NK) {
             w4_words = asm_load_b64(w4_off, (const uint8_t*)p.b + (int64_t)(kt0 + kt) * 32);
             w4_scale16 = asm_load_u16(w4_soff, (const uint8_t*)p.b_s + (int64_t)(((kt0 + kt) * 64) / p.group) * 2);
@@ -322,12 +382,28 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     // ... and from there, expanded, into the weight rows of stage kt
     auto w4_expand = [&](int kt) {
         if constexpr (W4) {
-            // everything but the MI youngest (activation) loads.  The two registers pass through the wait as
-            // read-write operands: the compiler must have them in VGPRs here and takes every later use from
-            // this statement, so no use can be scheduled above the wait.
+            // everything but the MI youngest (activation) loads (and the scale column behind them for the
+            // block-scaled kind).  The registers pass through the wait as read-write operands: the compiler must
+            // have them in VGPRs here and takes every later use from this statement, so no use can be scheduled
+            // above the wait.
             if constexpr (W4NK) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(w4_words), "+v"(w4_scale16) : "n"(MI) : "memory");
-            else asm volatile("s_waitcnt vmcnt(%2)" : "+v"(w4_words), "+v"(w4_scale) : "n"(MI) : "memory");
+            else if constexpr (W4M) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(w4_words), "+v"(w4_scale) : "n"(MI) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%1)" : "+v"(w4_words4) : "n"(MI + 1) : "memory");
             __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (W4A8) {
+            const int base = (int)(w4_lds & 0xffffu), kc = (int)((w4_lds >> 16) & 0xffu), pr = (int)(w4_lds >> 24);
+            const uint8_t* tabk = w4tab + kt * 128 + 8 * pr;
+            unsigned sp[4], cp[4], rows[8];
+            w4a8_row_consts(*(const uint2*)tabk, *(const uint2*)(tabk + 128 * KT), sp, cp);
+            w4a8_words_to_i8(w4_words4, sp, cp, rows);
+            uint8_t* dst = lds + (kt % D_NSTAGE) * D_STAGE + D_A + (kc & 3) * 4;
+            const int chunk = kc >> 2;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int R = base + (i & 3) + 16 * (i >> 2);
+                *(unsigned*)(dst + R * 128 + ((chunk ^ ((R >> 1) & 7)) * 16)) = rows[i];
+            }
         }
         if constexpr (W4NK) {
             const unsigned s16 = w4_scale16;
@@ -359,9 +435,15 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
                 }
         }
     };
-    // loads per stage per thread: MI (A) + 2 (B, or words + scale for K_W4NK) + 1 (scale column);
+    // Nothing is in flight when the last K step begins (the step before it ended with vmcnt(0)); this wait costs
+    // nothing and puts a covering wait on every static path into that step, also on those that the trip counts
+    // rule out (a request in the loop followed by a skipped middle step), which the check of the assembly walks.
+    auto w4_drain = [&]() {
+        if constexpr (W4A8) asm volatile("s_waitcnt vmcnt(0)" : "+v"(w4_words4) : : "memory");
+    };
+    // loads per stage per thread: MI (A) + 2 (B, or words + scale for K_W4NK; one load of words for K_W4A8) + 1 (scale column);
     // imm = vmcnt | no expcnt/lgkmcnt wait
-    constexpr int WAIT_ONE_STAGE = 0x0F70 | (MI + 2 + (SCALED ? 1 : 0));
+    constexpr int WAIT_ONE_STAGE = 0x0F70 | (MI + (W4A8 ? 1 : 2) + (SCALED ? 1 : 0));
 
     // acc[i][j][q] = C[row 16i + r][col 32*(j >> 1) + 8g + 4*(j & 1) + q] of the wave's 64 x 64 tile
     v4f acc[MI][4];
@@ -370,7 +452,22 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-    if (KT > 0) { w4_request(0); issue(0); w4_expand(0); }
+    if constexpr (W4A8) {
+        // the table first (ordinary loads; the wait for them also drains stage 0, whose words are expanded next).
+        // KT is the same for every thread of the workgroup, so the barrier is reached by all or by none.
+        if (KT > 0) {
+            w4_request(0);
+            issue(0);
+            for (int i = tid; i < 128 * KT; i += D_THREADS) {
+                const int row = i / KT, kk = i - row * KT;
+                const int64_t at = (int64_t)min(n0 + row, N - 1) * KT_all + kt0 + kk;
+                w4tab[kk * 128 + row] = (uint8_t)p.w4_s4[at];
+                w4tab[(KT + kk) * 128 + row] = (uint8_t)p.w4_z4[at];
+            }
+            __syncthreads();
+            w4_expand(0);
+        }
+    } else if (KT > 0) { w4_request(0); issue(0); w4_expand(0); }
     if (KT > 1) { w4_request(1); issue(1); }
     // weight scales of this tile for every K step -> LDS.  These are the only compiler-tracked vector
     // loads; they sit behind the first two stages in the memory queue, so waiting for them also waits
@@ -496,6 +593,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             __syncthreads();
             ++kt;
         }
+        w4_drain();
         if (kt < KT) {
             load_frags(kt);
             compute();
@@ -520,6 +618,7 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
             __syncthreads();
             ++kt;
         }
+        w4_drain();
         if (kt < KT) {
             compute();
             __builtin_amdgcn_sched_barrier(0);
@@ -655,18 +754,34 @@ inline bool dma_eligible(const DirectArgs& p, int esz = 1) {
            (int64_t)p.M * (kb >> 7) * 4 < (1ll << 32) && (kb >> 7) <= D_MAX_KT && p.K > 0;
 }
 
+// K steps one workgroup of the K_W4A8 kind walks (its share of a split K range): sizes its LDS table
+constexpr int D_LDS_MAX = 160 * 1024;
+inline int w4a8_table_steps(const DirectArgs& p) {
+    const int KT = p.K >> 7;
+    return p.ksplit > 1 ? (KT + p.ksplit - 1) / p.ksplit : KT;
+}
+// tallest tile (MI) whose stages leave room for that table
+inline int w4a8_max_mi(const DirectArgs& p) {
+    const int tab = 256 * w4a8_table_steps(p);
+    // (the 256-row tile has no registers to spare for the expansion: the kind runs on the 128- and 64-row tiles)
+    return d_lds(2) + tab <= D_LDS_MAX ? 2 : (d_lds(1) + tab <= D_LDS_MAX ? 1 : 0);
+}
+
 // a_s must be fp32 here (p.a_s); p.s_dtype describes b_s only.
 template <int KIND, bool GROUPED, int MI>
 int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     static std::atomic<uint64_t> configured{0};
     auto kern = gemm_dma_kernel<KIND, GROUPED, MI>;
-    if (int rc = llmk_reserve_lds((const void*)kern, d_lds(MI), configured, name)) return rc;
     constexpr int BM = 64 * MI;
     const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, BM) : (p.M + BM - 1) / BM;
     const bool split = !GROUPED && p.ksplit > 1 && p.partial;
+    // K_W4A8: the table of zero points and second-level scales (256 bytes per K step of the workgroup) behind the stages
+    const int lds_bytes = d_lds(MI) + (KIND == K_W4A8 ? 256 * w4a8_table_steps(p) : 0);
+    if (lds_bytes > D_LDS_MAX) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: %d bytes of LDS needed", name, lds_bytes);
+    if (int rc = llmk_reserve_lds((const void*)kern, KIND == K_W4A8 ? D_LDS_MAX : d_lds(MI), configured, name)) return rc;
     dim3 grid((unsigned)((p.N + D_BN - 1) / D_BN), (unsigned)tiles_m, split ? (unsigned)p.ksplit : 1u);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
-    kern<<<grid, D_THREADS, d_lds(MI), stream>>>(p);
+    kern<<<grid, D_THREADS, lds_bytes, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     if (split) {
         const int64_t mn = (int64_t)p.M * p.N;

@@ -1,0 +1,459 @@
+// Tile kernel for mid-size M (about 65 to 512 rows) on few column tiles: problems that neither fill the chip with
+// 128- or 256-column tiles nor fit the weight-streaming kernels, and whose weights mostly come cold from HBM.
+//
+// What bounds the 64 x 128 tile of gemm_dma.hpp there is the per-step overhead: one barrier, twelve fragment reads
+// and a dependent wait per wave for four matrix instructions on 128 bytes of K.  Here a K step is 512 bytes and
+// the eight waves of a workgroup split it four ways:
+//
+//   tile 16 MT x 64 (MT = 4 or 2), wave (wn, kq): all 16 MT rows x 32 columns (wn = wave & 1) of the 128-byte
+//   sub-block kq = wave >> 1 of the step: 2 MT matrix-instruction tiles for 2 MT + 4 fragment reads, one barrier
+//   per 512 bytes of K; the four partial sums of an output meet in LDS once, at the end of the tile.
+//
+// Activations (hot in L2: every workgroup of a row tile reads the same rows) go global -> LDS by direct-to-LDS
+// loads, one step ahead, two stages.  Weights (cold: each byte is needed by M / (16 MT) workgroups only) go
+// global -> registers three steps ahead, coalesced (eight lanes per 128-byte line), by hand-issued loads into a
+// ring of four register sets, and from there into one of two LDS stages one step before they are multiplied:
+// 1.5 KB per weight row in flight without spending LDS on it, and a natural place to unpack 4-bit weights
+// (K_W4A8: packed words in the ring, int8 rows in LDS).  The row tiles that share a column tile land on one XCD
+// (same workgroup id modulo 8 when the column tiles are a multiple of 8) and walk K in step, so that a weight line
+// comes from HBM once.
+//
+// What bounds it (measured): a CU takes about 110 GB/s from its L2, and a 64 x 64 tile needs 128 bytes per byte of
+// K (0.6 us per step); three activation stages with the weights through a single stage between two barriers, and
+// row tiles that start their K walk at different steps, were both slower.
+//
+// All loads of a step are issued unconditionally (steps past the end repeat the last one) so that one
+// hand-counted s_waitcnt per step is exact; check_asm.py proves the register loads on every build.
+#pragma once
+#include "gemm_dma.hpp"
+
+namespace llmk {
+
+constexpr int MD_BN = 64, MD_THREADS = 512;
+constexpr int MD_B = 4 * MD_BN * 128;                       // weight stage: [sub-block][column][128 B] = 32 KB
+constexpr int MD_S = 4 * 64 * 4;                            // activation-scale columns of a step: [sub-block][row] fp32
+constexpr int MD_RED_ROW = 68;                              // floats per row of the final reduction (64 + 4: bank spread)
+constexpr int md_a(int mt) { return 4 * 16 * mt * 128; }    // activation stage: [sub-block][row][128 B]
+constexpr int MD_NA = 2;                                    // activation stages
+constexpr int MD_NBS = 2;                                   // weight stages
+constexpr int md_stages(int mt) { return MD_NA * (md_a(mt) + MD_S) + MD_NBS * MD_B; }
+constexpr int md_red(int mt) { return 4 * 16 * mt * MD_RED_ROW * 4; }
+// stages (reused by the reduction), weight-scale table, K_W4A8 table of zero points and second-level scales
+constexpr int md_lds(int mt, int kt_tab) { return md_stages(mt) + D_MAX_KT * 4 + 128 * kt_tab; }
+
+template <int KIND, int MT>
+__global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
+    static_assert(MT == 4 || MT == 2, "tile rows");
+    constexpr int BM = 16 * MT;
+    constexpr bool W4A8 = (KIND == K_W4A8);
+    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || W4A8);
+    constexpr bool ROWCOL = (KIND == K_I8_ROWCOL);
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    constexpr int MD_A = md_a(MT);
+    constexpr int NB = W4A8 ? 2 : 4;                        // ring loads per thread and step
+    // ring slots: weights are requested MD_RING - 1 steps ahead.  The block-scaled 8-bit kinds on the 64-row tile keep
+    // products and accumulators apart and have no registers for a fourth slot (the build refuses spills in a
+    // kernel with hand-issued loads); three slots measured the same.
+    constexpr int MD_RING = (SCALED && !W4A8 && MT == 4) ? 3 : 4;
+    constexpr int NA = MT + (SCALED ? 1 : 0);               // direct-to-LDS loads per thread and step
+    static_assert(md_red(MT) <= md_stages(MT), "the reduction reuses the stages");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4, wn = wave & 1, kq = wave >> 1;
+    const int N = p.N;
+    const int K = p.K * ESZ;                                // row length in bytes
+    const int KT_all = K >> 7;                              // 128-byte sub-blocks per row
+    int kt0 = 0, KT = KT_all;                               // sub-blocks [kt0, kt0 + KT) of this workgroup
+    if (p.ksplit > 1) {
+        // slices in whole steps of four sub-blocks (one weight-scale block each for the scaled kinds)
+        const int per = (((KT_all + p.ksplit - 1) / p.ksplit) + 3) & ~3;
+        kt0 = (int)blockIdx.z * per;
+        KT = max(0, min(per, KT_all - kt0));
+    }
+    const int nsteps = (KT + 3) >> 2;
+    const int n0 = blockIdx.x * MD_BN, m_start = blockIdx.y * BM, m_end = min(p.M, m_start + BM);
+
+    // LDS map
+    uint8_t* const a_st = lds;                              // [3][MD_A]
+    uint8_t* const b_st = lds + MD_NA * MD_A;               // [MD_B]
+    uint8_t* const s_st = lds + MD_NA * MD_A + MD_NBS * MD_B;        // [3][MD_S]
+    float* const bsl = (float*)(lds + md_stages(MT));       // weight scale of the tile's column block per sub-block
+    uint8_t* const w4tab = lds + md_stages(MT) + D_MAX_KT * 4;   // K_W4A8: [s4 | z4][sub-block][64 rows] bytes
+
+    // ---- per-thread source offsets.  A piece = 8 rows x 128 bytes = what one load instruction of a wave covers
+    // (lane: row lane >> 3, 16-byte chunk lane & 7, XOR-swizzled with (row >> 1) & 7 on the global side so that
+    // the fragment reads are conflict-free).  Wave w moves pieces MT w .. MT w + MT - 1 of the 4 x 2 MT activation
+    // pieces and pieces 4 w .. 4 w + 3 of the 4 x 8 weight pieces of a step: piece = (sub-block, row group).
+    const int row8 = lane >> 3;
+    uint32_t aoff[MT], alds[MT];
+    int asub[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int pq = MT * wave + i, sub = pq / (2 * MT), row = 8 * (pq % (2 * MT)) + row8;
+        const uint32_t chunk = (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
+        aoff[i] = (uint32_t)min(m_start + row, m_end - 1) * (uint32_t)K + chunk;
+        alds[i] = (uint32_t)(sub * (BM * 128) + 8 * (pq % (2 * MT)) * 128);     // + lane * 16 by the hardware
+        asub[i] = sub;
+    }
+    uint32_t boff[4], blds[4];
+    int bsub[4];
+    if constexpr (!W4A8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int pq = 4 * wave + i, sub = pq >> 3, row = 8 * (pq & 7) + row8;
+            boff[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (uint32_t)(lane & 7) * 16u;
+            blds[i] = (uint32_t)(sub * (MD_BN * 128) + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16));
+            bsub[i] = sub;
+        }
+    } else {
+        // one wave per packed row (eight weight rows): lane l takes words 4 l .. 4 l + 3 of sub-blocks l >> 5 (load 0)
+        // and 2 + (l >> 5) (load 1) of the step's 512 words
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            boff[i] = (uint32_t)min((n0 >> 3) + wave, (N >> 3) - 1) * (uint32_t)(p.K * 4) + (uint32_t)(lane & 31) * 16u;
+            bsub[i] = 2 * i + (lane >> 5);
+            blds[i] = 0;
+        }
+        boff[2] = boff[3] = blds[2] = blds[3] = 0;
+        bsub[2] = bsub[3] = 0;
+    }
+    const uint32_t soff = (uint32_t)min(m_start + min(lane, BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
+
+    // sub-block `sub` of step s, clamped to the last one of the range (loads past the end repeat it)
+    // requests past the end repeat the last step
+    auto phys = [&](int s) { return min(s, nsteps - 1); };
+    auto kblock = [&](int s, int sub) { return kt0 + min(4 * phys(s) + sub, KT - 1); };
+
+    auto issue_a = [&](int s) {
+        const uint32_t st = lds_base + (uint32_t)(s % MD_NA) * MD_A;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) dma16(st + alds[i], aoff[i], p.a + (int64_t)kblock(s, asub[i]) * 128);
+        if constexpr (SCALED) {
+            const uint32_t ss = lds_base + MD_NA * MD_A + MD_NBS * MD_B + (uint32_t)(s % MD_NA) * MD_S + (uint32_t)(wave & 3) * 256u;
+            dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 4);
+        }
+    };
+    // ring of weight registers: slot = step % 4
+    v4i ring[MD_RING][NB];
+    auto issue_b = [&](v4i (&rs)[NB], int s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            if constexpr (W4A8) {
+                // lane-dependent sub-block: the two halves of the wave read different 128-word runs of the row
+                const int kb0 = kblock(s, 2 * i), kb1 = kblock(s, 2 * i + 1);
+                const uint32_t off = boff[i] + (uint32_t)((lane >> 5) ? kb1 - kb0 : 0) * 512u;
+                rs[i] = asm_load_b128(off, (const uint8_t*)p.b + (int64_t)kb0 * 512);
+            } else {
+                rs[i] = asm_load_b128(boff[i], p.b + (int64_t)kblock(s, bsub[i]) * 128);
+            }
+        }
+    };
+    // the loads of slot `slot` have landed when at most `younger` loads issued after them are in flight
+    auto ring_ready = [&](v4i (&rs)[NB], auto younger_c) __attribute__((always_inline)) {
+        constexpr int Y = decltype(younger_c)::value;
+        if constexpr (NB == 4)
+            asm volatile("s_waitcnt vmcnt(%4)" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]) : "n"(Y) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(rs[0]), "+v"(rs[1]) : "n"(Y) : "memory");
+    };
+    // ring slot -> weight stage s & 1 (nobody has read that stage since the barrier of step s - 1)
+    auto produce = [&](const v4i (&rs)[NB], int s) __attribute__((always_inline)) {
+        uint8_t* st = b_st + (s % MD_NBS) * MD_B;
+        if constexpr (!W4A8) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *(v4i*)(st + blds[i]) = rs[i];
+        } else {
+            // lane: words 4 kc .. 4 kc + 3 (kc = lane & 31) of sub-block 2 i + (lane >> 5); packed row = wave.  Row j of
+            // the packed row is tile column 8 wave + j.
+            const int kc = lane & 31;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int sub = 2 * i + (lane >> 5);
+                const int kb = min(4 * phys(s) + sub, KT - 1);
+                const uint8_t* tabk = w4tab + kb * 64 + 8 * wave;
+                unsigned sp[4], cp[4], rows[8];
+                w4a8_row_consts(*(const uint2*)tabk, *(const uint2*)(tabk + 64 * KT), sp, cp);
+                w4a8_words_to_i8(rs[i], sp, cp, rows);
+                uint8_t* dst = st + sub * (MD_BN * 128) + (kc & 3) * 4;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int R = 8 * wave + j;
+                    *(unsigned*)(dst + R * 128 + (((kc >> 2) ^ ((R >> 1) & 7)) * 16)) = rows[j];
+                }
+            }
+        }
+    };
+
+    // acc[i][j][q] = C[row 16 i + r][column 32 wn + 16 j + 4 g + q] summed over this wave's sub-blocks
+    v4f acc[MT][2];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i][0] = acc[i][1] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // fragment read offsets inside a 16-row slab: chunks g and g + 4 of row r, swizzled
+    const int lo = r * 128 + ((g ^ ((r >> 1) & 7)) * 16);
+    const int hi = r * 128 + (((g + 4) ^ ((r >> 1) & 7)) * 16);
+    auto ldfrag = [&](const uint8_t* base) {
+        const v4i x = *(const v4i*)(base + lo), y = *(const v4i*)(base + hi);
+        return (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+    };
+    auto compute = [&](int s) {
+        const uint8_t* As = a_st + (s % MD_NA) * MD_A + kq * (BM * 128);
+        const uint8_t* Bs = b_st + (s % MD_NBS) * MD_B + kq * (MD_BN * 128) + (wn * 32) * 128;
+        const int kb = 4 * phys(s) + kq;
+        const bool live = kb < KT;                         // wave-uniform: sub-blocks past the range add nothing
+        // activation fragments one tile row ahead of their use
+        v8i bf[2], af[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) bf[j] = ldfrag(Bs + j * 2048);
+        af[0] = ldfrag(As);
+        const v8i zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (SCALED) {
+            const float* Ss = (const float*)(s_st + (s % MD_NA) * MD_S) + kq * 64 + r;
+            const float bs = live ? bsl[min(kb, KT - 1)] : 0.f;
+            float sa[MT];
+#pragma unroll
+            for (int i = 0; i < MT; ++i) sa[i] = Ss[16 * i] * bs;
+            // the products of tile row i are scaled and accumulated while the matrix instructions of row i + 1 run
+            v4f t[2][2];
+#pragma unroll
+            for (int i = 0; i <= MT; ++i) {
+                if (i + 1 < MT) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if (i < MT) t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
+                    if (i > 0) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
+                }
+                // nothing moves across a tile row: the lag of one row between product and accumulation stays, and
+                // the fragments of at most two rows are live
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                if (i + 1 < MT) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+                const v8i a = live ? af[i & 1] : zero8;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = mma_plain<KIND>(bf[j], a, acc[i][j]);
+            }
+        }
+    };
+
+    const std::integral_constant<int, 0> c0;
+    const std::integral_constant<int, 1> c1;
+    const std::integral_constant<int, 2> c2;
+    const std::integral_constant<int, 3> c3;
+    const std::integral_constant<int, (MD_RING - 2) * NB> cpro;
+    const std::integral_constant<int, NB> cnb;
+    const std::integral_constant<int, NA + NB> cstep;
+
+
+    // ---- prologue: activations of step 0, weights of steps 0, 1, 2; tables by ordinary loads meanwhile
+    issue_a(0);
+    issue_b(ring[0], 0);
+    issue_b(ring[1], 1);
+    if constexpr (MD_RING == 4) issue_b(ring[2], 2);
+    if constexpr (SCALED) {
+        const int64_t bs_row = (int64_t)(n0 >> 7) * KT_all + kt0;
+        for (int i = tid; i < KT; i += MD_THREADS) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
+    }
+    if constexpr (W4A8) {
+        for (int i = tid; i < 64 * KT; i += MD_THREADS) {
+            const int row = i / KT, kk = i - row * KT;
+            const int64_t at = (int64_t)min(n0 + row, N - 1) * KT_all + kt0 + kk;
+            w4tab[kk * 64 + row] = (uint8_t)p.w4_s4[at];
+            w4tab[(KT + kk) * 64 + row] = (uint8_t)p.w4_z4[at];
+        }
+        __syncthreads();                                    // the table is read by produce()
+    }
+    ring_ready(ring[0], cpro);
+    produce(ring[0], 0);
+
+    // One step: wait for the activations of step s (requested a step ago; only the NB weight loads issued after
+    // them may stay in flight; with four ring slots that also vouches for slot s + 1, requested two steps ago),
+    // meet the others, request the activations of step s + 1 and the weights of step s + MD_RING - 1, multiply
+    // step s, and move the weights of step s + 1 from the ring into the other weight stage (with three slots they
+    // were requested a step ago: everything but this step's own requests has landed by then).
+    auto step = [&](auto slot_c, int s) __attribute__((always_inline)) {
+        constexpr int slot = decltype(slot_c)::value;
+        // (scheduling fences: without them the compiler carries the matrix instructions of a step across the next
+        // barrier, with all fragments of two steps live, and spills)
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MD_RING == 4) ring_ready(ring[(slot + 1) % MD_RING], cnb);
+        else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NB) : "memory");
+        __builtin_amdgcn_s_waitcnt(0xc07f);                 // lgkmcnt(0): this wave's LDS writes of produce() are done
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        issue_a(s + 1);
+        issue_b(ring[(slot + MD_RING - 1) % MD_RING], s + MD_RING - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(s);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MD_RING == 3) ring_ready(ring[(slot + 1) % MD_RING], cstep);
+        produce(ring[(slot + 1) % MD_RING], s + 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int s = 0;
+    for (int rd = nsteps / MD_RING; rd > 0; --rd) {
+        step(c0, s);
+        step(c1, s + 1);
+        step(c2, s + 2);
+        if constexpr (MD_RING == 4) step(c3, s + 3);
+        s += MD_RING;
+    }
+    const int rem = nsteps % MD_RING;
+    // (nested: a later step without the earlier ones is a path the trip count rules out, and the static check of
+    // the assembly would still walk it)
+    if (rem > 0) {
+        step(c0, s);
+        if (rem > 1) {
+            step(c1, s + 1);
+            if constexpr (MD_RING == 4) { if (rem > 2) step(c2, s + 2); }
+        }
+    }
+    // everything requested has landed (also the repeated loads past the end) before the stages are reused
+    if constexpr (NB == 4 && MD_RING == 3) {
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(ring[0][0]), "+v"(ring[0][1]), "+v"(ring[0][2]), "+v"(ring[0][3]), "+v"(ring[1][0]), "+v"(ring[1][1]),
+                       "+v"(ring[1][2]), "+v"(ring[1][3]), "+v"(ring[2][0]), "+v"(ring[2][1]), "+v"(ring[2][2]), "+v"(ring[2][3]) : : "memory");
+    } else if constexpr (NB == 4) {
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(ring[0][0]), "+v"(ring[0][1]), "+v"(ring[0][2]), "+v"(ring[0][3]), "+v"(ring[1][0]), "+v"(ring[1][1]),
+                       "+v"(ring[1][2]), "+v"(ring[1][3]), "+v"(ring[2][0]), "+v"(ring[2][1]), "+v"(ring[2][2]), "+v"(ring[2][3]),
+                       "+v"(ring[3][0]), "+v"(ring[3][1]), "+v"(ring[3][2]), "+v"(ring[3][3]) : : "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(ring[0][0]), "+v"(ring[0][1]), "+v"(ring[1][0]), "+v"(ring[1][1]), "+v"(ring[2][0]), "+v"(ring[2][1]),
+                       "+v"(ring[3][0]), "+v"(ring[3][1]) : : "memory");
+    }
+    __syncthreads();
+
+    // ---- the four sub-block sums of every output meet in LDS: red[kq][row][column], rows of 68 floats
+    float* red = (float*)lds;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            *(v4f*)(red + (kq * BM + 16 * i + r) * MD_RED_ROW + wn * 32 + 16 * j + 4 * g) = acc[i][j];
+    __syncthreads();
+    // thread: row tid >> 3, columns 8 (tid & 7) .. + 7
+    const int orow = tid >> 3, ocol = 8 * (tid & 7);
+    if (orow >= BM) return;
+    const int m = m_start + orow, n = n0 + ocol;
+    if (m >= m_end || n >= N) return;
+    v4f sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (ROWCOL) {
+        v4i ia = {0, 0, 0, 0}, ib = {0, 0, 0, 0};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float* src = red + (q * BM + orow) * MD_RED_ROW + ocol;
+            ia += *(const v4i*)src;
+            ib += *(const v4i*)(src + 4);
+        }
+        __builtin_memcpy(&sa, &ia, 16);
+        __builtin_memcpy(&sb, &ib, 16);
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float* src = red + (q * BM + orow) * MD_RED_ROW + ocol;
+            sa += *(const v4f*)src;
+            sb += *(const v4f*)(src + 4);
+        }
+    }
+    const bool split = p.ksplit > 1;
+    void* cout = split ? (void*)(p.partial + (int64_t)blockIdx.z * p.M * N) : p.c;
+    const int cdt = split ? LLMK_F32 : p.c_dtype;
+    const int esz = cdt == LLMK_F32 ? 4 : 2;
+    const bool vec_ok = ((((uintptr_t)cout) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
+    const int nv = N - n;
+    const int64_t off = (int64_t)m * N + n;
+    if constexpr (ROWCOL) {
+        // (a K slice leaves its int32 sums, bit for bit, in the fp32 partial buffer: the summing pass adds them as
+        // integers and scales once, so the result does not depend on the split)
+        if (!split) {
+            rowcol_epilogue8(p, sa, sb, m, off, n, nv);
+            if (!p.c) return;
+        }
+    }
+    if (cdt == LLMK_BF16) store_run8<LLMK_BF16>(cout, off, sa, sb, nv, vec_ok);
+    else if (cdt == LLMK_F16) store_run8<LLMK_F16>(cout, off, sa, sb, nv, vec_ok);
+    else store_run8<LLMK_F32>(cout, off, sa, sb, nv, vec_ok);
+}
+
+// K slices of the mid-size kernel: as many as bring the grid to about one workgroup per CU, in whole steps of 512
+// bytes, each slice at least four steps long; 1 = no split.
+inline int mid_splitk(int64_t tiles, int64_t kbytes) {
+    if (tiles >= 192) return 1;
+    int64_t z = 256 / tiles;
+    const int64_t steps = kbytes >> 9;
+    if (z > steps / 4) z = steps / 4;
+    return (int)(z > 8 ? 8 : (z < 1 ? 1 : z));
+}
+
+// Shape of a mid-size launch: tile height (16 mt rows) and K slices.  The 32-row tile when the 64-row tile would leave
+// more than half of the CUs without a workgroup.
+struct MidPlan {
+    int mt, z;
+    int64_t tiles;
+};
+inline MidPlan mid_plan(int64_t M, int64_t N, int64_t kbytes) {
+    MidPlan pl;
+    const int64_t gx = (N + MD_BN - 1) / MD_BN;
+    const int64_t t4 = ((M + 63) / 64) * gx, t2 = ((M + 31) / 32) * gx;
+    pl.mt = (t4 <= 128 && t2 > t4) ? 2 : 4;
+    pl.tiles = pl.mt == 4 ? t4 : t2;
+    pl.z = mid_splitk(pl.tiles, kbytes);
+    return pl;
+}
+
+// Eligibility: 32-bit source offsets, whole 128-byte sub-blocks, scale table size (as dma_eligible), and for the
+// K_W4A8 kind room for its table behind the stages.
+template <int KIND>
+inline bool mid_eligible(const DirectArgs& p, int mt, int ksplit) {
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    if (!dma_eligible(p, ESZ)) return false;
+    const int KT_all = (p.K * ESZ) >> 7;
+    const int per = ksplit > 1 ? ((((KT_all + ksplit - 1) / ksplit) + 3) & ~3) : KT_all;
+    return md_lds(mt, KIND == K_W4A8 ? per : 0) <= D_LDS_MAX;
+}
+
+// a_s must be fp32 here (p.a_s); p.s_dtype describes b_s only.  p.ksplit / p.partial select the K split.
+template <int KIND, int MT>
+int launch_mid(const DirectArgs& p, hipStream_t stream, const char* name) {
+    static std::atomic<uint64_t> configured{0};
+    auto kern = gemm_mid_kernel<KIND, MT>;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    const int KT_all = (p.K * ESZ) >> 7;
+    const bool split = p.ksplit > 1 && p.partial;
+    const int per = split ? ((((KT_all + p.ksplit - 1) / p.ksplit) + 3) & ~3) : KT_all;
+    const int lds_bytes = md_lds(MT, KIND == K_W4A8 ? per : 0);
+    if (lds_bytes > D_LDS_MAX) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: %d bytes of LDS needed", name, lds_bytes);
+    if (int rc = llmk_reserve_lds((const void*)kern, D_LDS_MAX, configured, name)) return rc;
+    // slices that would start past the end of K are not launched
+    const int z = split ? (KT_all + per - 1) / per : 1;
+    DirectArgs q = p;
+    q.ksplit = split ? p.ksplit : 1;
+    dim3 grid((unsigned)((p.N + MD_BN - 1) / MD_BN), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)), (unsigned)z);
+    if (grid.x == 0 || grid.y == 0) return LLMK_OK;
+    kern<<<grid, MD_THREADS, lds_bytes, stream>>>(q);
+    LLMK_CHECK_LAUNCH(name);
+    if (split) {
+        const int64_t mn = (int64_t)p.M * p.N;
+        const unsigned blocks = (unsigned)cdiv64(cdiv64(mn, 4), 256);
+        if constexpr (KIND == K_I8_ROWCOL) {
+            const int32_t* part = (const int32_t*)p.partial;
+            if (p.c_dtype == LLMK_BF16) splitk_sum_rowcol_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(part, p, mn, z);
+            else if (p.c_dtype == LLMK_F16) splitk_sum_rowcol_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(part, p, mn, z);
+            else splitk_sum_rowcol_kernel<LLMK_F32><<<blocks, 256, 0, stream>>>(part, p, mn, z);
+        } else {
+            if (p.c_dtype == LLMK_BF16) splitk_sum_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, z);
+            else if (p.c_dtype == LLMK_F16) splitk_sum_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, z);
+            else splitk_sum_kernel<LLMK_F32><<<blocks, 256, 0, stream>>>(p.partial, p.c, mn, z);
+        }
+        LLMK_CHECK_LAUNCH(name);
+    }
+    return LLMK_OK;
+}
+
+}  // namespace llmk

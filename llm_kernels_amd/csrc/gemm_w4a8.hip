@@ -438,11 +438,12 @@ int launch_w4a8_stream(W4A8Args p, void* workspace, int64_t workspace_bytes, hip
 namespace {
 struct W4A8Plan {
     bool stream;          // fused decode kernel
-    int64_t nz;           // its K ranges
+    bool tiles;           // 128-column tile kernels that expand the packed words themselves
+    int64_t nz;           // K ranges of the decode kernel
     int64_t bytes;        // scratch the chosen path uses
 };
 W4A8Plan w4a8_plan(int64_t M, int64_t N, int64_t K, int group_int4) {
-    W4A8Plan pl{false, 1, 0};
+    W4A8Plan pl{false, false, 1, 0};
     if (M <= 0 || N <= 0 || K <= 0) return pl;
     // Measured on MI355X with x = N * K / 4096^2: the fused kernel takes about 5 + 3.4 x microseconds per 32 rows
     // of M; expanding to int8 and running the int8 GEMM about 26 + 3.6 x for x <= 4 and more beyond.
@@ -454,10 +455,52 @@ W4A8Plan w4a8_plan(int64_t M, int64_t N, int64_t K, int group_int4) {
     const bool long_k_ok = pl.nz == 1 || row_blocks <= 2;
     // (the hand-issued loads of the fused kernel take 32-bit lane offsets into the activations and the tables)
     const bool small_offsets = M * K < (1ll << 32) && N * (K / 128) < (1ll << 32);
-    pl.stream = fused_wins && long_k_ok && small_offsets && group_int4 == 128;
+    // 65 to 256 rows on at most one 64-column workgroup per CU: the tile kernel with 512-byte K steps
+    const bool mid = M > 64 && M <= 256 && mid_plan(M, N, K).tiles <= 256 && K <= 16384;
+    pl.stream = fused_wins && long_k_ok && small_offsets && group_int4 == 128 && !mid;
+    // Mid-size M: the tile kernels unpack and dequantise inside their K loop (one pass over the packed words; the
+    // separate expansion writes and re-reads N * K bytes).  Measured (us per launch, fused | expansion + int8 GEMM):
+    // the 64-column kernel with 512-byte K steps on at most one workgroup per CU: 256 x 4096 x 4096 19.4 | 29.8,
+    // 256 x 4096 x 14336 54.2 | 60.6; the 128-column kernel up to 128 rows: 128 x 14336 x 4096 40.5 | 44.6,
+    // 128 x 4096 x 14336 41.2 | 46.5; from there on the two passes win (512 x 4096 x 4096 34 | 30, 512 x 14336 x 4096 80 | 60).
+    DirectArgs q{};
+    q.M = (int)M; q.N = (int)N; q.K = (int)K;
+    pl.tiles = !pl.stream && M > 64 && (mid || M <= 128) && group_int4 == 128 && N <= 0x7fffffff &&
+               K <= 0x7fffffff && dma_eligible(q);
     if (pl.stream) pl.bytes = pl.nz > 1 ? pl.nz * M * N * 4 : 0;
+    else if (pl.tiles) pl.bytes = llmk_gemm_workspace_bytes(M, N, K);      // fp32 activation scales + split-K partial sums
     else pl.bytes = ((N * K + 15) & ~(int64_t)15) + llmk_gemm_workspace_bytes(M, N, K);
     return pl;
+}
+
+// The tile path: 16-bit activation scales are widened into the workspace first (the pipeline streams 4-byte
+// scale elements), few tiles split K over workgroups with fp32 partial sums behind them.
+int launch_w4a8_tiles(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+    const char* name = "gemm_w4a8(fused tiles)";
+    int64_t used = 0;
+    if (p.s_dtype != LLMK_F32) {
+        const int64_t n = (int64_t)p.M * (p.K >> 7);
+        const unsigned blocks = (unsigned)cdiv64(n, 256);
+        if (p.s_dtype == LLMK_F16) scales_to_f32_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
+        else scales_to_f32_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
+        LLMK_CHECK_LAUNCH(name);
+        p.a_s = workspace;
+        used = (n * 4 + 255) & ~(int64_t)255;
+    }
+    if (p.M <= 256 && mid_plan(p.M, p.N, p.K).tiles <= 256 && p.K <= 16384) {
+        MidPlan pl = mid_plan(p.M, p.N, p.K);
+        if (pl.z > 1 && workspace_bytes - used < (int64_t)pl.z * p.M * p.N * 4) pl.z = 1;
+        if (mid_eligible<K_W4A8>(p, pl.mt, pl.z)) {
+            if (pl.z > 1) { p.partial = (float*)((uint8_t*)workspace + used); p.ksplit = pl.z; }
+            return pl.mt == 4 ? launch_mid<K_W4A8, 4>(p, stream, name) : launch_mid<K_W4A8, 2>(p, stream, name);
+        }
+    }
+    const int z = splitk_factor(p.M, p.N, p.K);
+    if (z > 1 && workspace_bytes - used >= (int64_t)z * p.M * p.N * 4) {
+        p.partial = (float*)((uint8_t*)workspace + used);
+        p.ksplit = z;
+    }
+    return launch_dma<K_W4A8, false>(p, stream, name);
 }
 }  // namespace
 
@@ -490,6 +533,16 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
         if (s_dtype == LLMK_F32) LLMK_W4A8_MT(LLMK_F32);
 #undef LLMK_W4A8_MT
         LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: s_dtype %d", s_dtype);
+    }
+    if (pl.tiles && !(((uintptr_t)a | (uintptr_t)b_packed | (uintptr_t)workspace) & 15) && workspace &&
+        workspace_bytes >= ((M * (K / 128) * 4 + 255) & ~(int64_t)255)) {
+        if (s_dtype != LLMK_F32 && s_dtype != LLMK_F16 && s_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: s_dtype %d", s_dtype);
+        if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: c_dtype %d", c_dtype);
+        DirectArgs p{};
+        p.a = (const uint8_t*)a; p.b = (const uint8_t*)b_packed; p.c = c; p.a_s = a_s; p.b_s = b_s;
+        p.w4_s4 = b_s4; p.w4_z4 = b_z4;
+        p.c_dtype = c_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1; p.group = 128;
+        return launch_w4a8_tiles(p, workspace, workspace_bytes, (hipStream_t)stream);
     }
     if (!workspace || workspace_bytes < N * K) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a8: workspace of N*K=%lld bytes required", (long long)(N * K));
     if (K > 0) {

@@ -16,7 +16,7 @@
 // of partial products that carry over from one K step to the next.
 #pragma once
 #include <type_traits>
-#include "gemm_dma.hpp"
+#include "gemm_mid.hpp"
 
 namespace llmk {
 
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     // 4-bit weights (fp16 activations): the weight rows of a stage are not loaded into LDS but expanded there by
     // the threads themselves from packed words that travel HBM -> registers, see w4_request / w4_expand
     constexpr bool W4NK = (KIND == K_W4NK), W4 = W4NK;
-    static_assert(KIND != K_W4MARLIN && !(W4 && GROUPED), "4-bit weights: row-packed layout, dense launches only");
+    static_assert(KIND != K_W4MARLIN && KIND != K_W4A8 && !(W4 && GROUPED), "4-bit weights: row-packed fp16 layout, dense launches only");
     constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4) ? 2 : 1;
     const int N = p.N;
     const int K = p.K * ESZ;                 // row length in bytes
@@ -601,6 +601,15 @@ inline int splitk_factor(int64_t M, int64_t N, int64_t K) {
     return (int)(z > 8 ? 8 : (z < 1 ? 1 : z));
 }
 
+// Shapes for the mid-size kernel (gemm_mid.hpp): more than 64 rows, at most one workgroup per CU and a K range of at
+// most 8 KB per row.  Measured against the 128-column tile kernels (fp8, us per launch, cold weights): 128 x 4096 x 4096
+// 16.7 -> 13.7, 256 x 4096 x 4096 23.1 -> 17.8; beyond one round of workgroups or with longer rows it loses
+// (512 x 4096 x 4096 15.5 -> 23.4, 256 x 6144 x 4096 23.5 -> 27.9, 256 x 4096 x 14336 43.9 -> 47.0).
+inline bool mid_wanted(int64_t M, int64_t N, int64_t kbytes) {
+    if (M <= 64 || M > 512) return false;
+    return mid_plan(M, N, kbytes).tiles <= 256 && kbytes <= 8192;
+}
+
 // 16 < M <= 64: the weight-streaming kernel re-reads the activations for every 16 columns, which costs more
 // than the 64-row tile kernel (with split-K when its tiles are few) once the weight matrix is large (measured
 // crossover between 17 M and 25 M elements).
@@ -616,7 +625,7 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* 
     if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
     // 4-bit weights: the row-packed layout, dense launches (the Marlin scatter of 2-byte pieces measured 4-9 % slower
     // inside the 256-column kernel than the dequantisation pass at every M > 512)
-    constexpr bool HAS_WIDE = KIND != K_W4MARLIN && !(GROUPED && KIND == K_W4NK);
+    constexpr bool HAS_WIDE = KIND != K_W4MARLIN && KIND != K_W4A8 && !(GROUPED && KIND == K_W4NK);
     const int64_t rows = GROUPED ? p.M / (p.E > 0 ? p.E : 1) : p.M;
     const int64_t groups = GROUPED ? p.E : 1;
     // a segment of a grouped GEMM rarely ends on a tile boundary: count one ragged tile per segment on top of
@@ -637,8 +646,12 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* 
         const double t_half = 36.0 * rounds(128, 256);
         if (t_half < t4 && t_half <= t2 && t_half <= t1) return launch_wide<KIND, GROUPED, 4>(p, stream, name, ws, ws_bytes);
     }
-    if (t4 <= t2 && t4 <= t1) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
-    if (t2 <= t1) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
+    int max_mi = 4;
+    if constexpr (KIND == K_W4A8) max_mi = w4a8_max_mi(p);       // the table of zero points and scales must fit behind the stages
+    if constexpr (KIND != K_W4A8) {
+        if (t4 <= t2 && t4 <= t1 && max_mi >= 4) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
+    }
+    if (t2 <= t1 && max_mi >= 2) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
     return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
 }
 
@@ -657,6 +670,18 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
         LLMK_CHECK_LAUNCH(name);
         p.a_s = workspace;
         used = (n * 4 + 255) & ~(int64_t)255;
+    }
+    // Mid-size M on few column tiles: the 64-column kernel with 512-byte K steps
+    if constexpr (!GROUPED) {
+        if (mid_wanted(p.M, p.N, p.K)) {
+            MidPlan pl = mid_plan(p.M, p.N, p.K);
+            const int64_t need = (int64_t)pl.z * p.M * p.N * 4;
+            if (pl.z > 1 && !(workspace && workspace_bytes - used >= need && !(((uintptr_t)workspace + used) & 15))) pl.z = 1;
+            if (mid_eligible<KIND>(p, pl.mt, pl.z)) {
+                if (pl.z > 1) { p.partial = (float*)((uint8_t*)workspace + used); p.ksplit = pl.z; }
+                return pl.mt == 4 ? launch_mid<KIND, 4>(p, stream, name) : launch_mid<KIND, 2>(p, stream, name);
+            }
+        }
     }
     // Few 64-row tiles (mid-size M, moderate N): split K over workgroups so that every CU streams weights,
     // fp32 partials in the workspace, one summing pass.

@@ -196,6 +196,54 @@ def test_w4a8_decode_exact_mixed_wrap(dev, M, N, K, sdt):
     assert torch.equal(c.cpu().long(), a.long() @ b8.long().T)
 
 
+@pytest.mark.parametrize("M,N,K,sdt", [(160, 4096, 1024, torch.float16), (200, 520, 3200, torch.float32),
+                                       (256, 1032, 2176, torch.bfloat16), (161, 8, 128, torch.float16),
+                                       (250, 2048, 8192, torch.float16), (256, 264, 14336, torch.float32),
+                                       (130, 4104, 4096, torch.bfloat16),
+                                       # more than 256 tiles of 64 columns, up to 128 rows: the 128-column tile kernel
+                                       (97, 9000, 4096, torch.float16), (128, 8200, 4224, torch.float32)])
+def test_w4a8_mid_m_fused_tiles_exact_mixed_wrap(dev, M, N, K, sdt):
+    """Mid-size M: the tile kernels unpack and dequantise the packed words inside their K loop (no int8 copy of
+    W).  Unit block scales, fp32 out, 2 % out-of-contract (s4, z4) pairs: exact integers with the int8 wrap,
+    over ragged row and column tiles, K tails, split K (few tiles, long K) and every scale dtype."""
+    announce("w4a8 fused tiles exact", M, N, K, sdt)
+    lib = _lib.load()
+    # these shapes take the fused tile path: their scratch is that of the int8 tile kernels (activation scales,
+    # split-K partial sums) with no int8 copy of the weights in front
+    assert lib.llmk_gemm_w4a8_workspace_bytes(M, N, K, 128) == lib.llmk_gemm_workspace_bytes(M, N, K)
+    torch.manual_seed(M + N)
+    wq = torch.randint(0, 16, (N, K), dtype=torch.uint8)
+    s4 = torch.randint(1, 9, (N, K // 128), dtype=torch.int8)
+    z4 = torch.randint(0, 16, (N, K // 128), dtype=torch.int8)
+    wild = torch.rand(N, K // 128) < 0.02
+    s4[wild] = torch.randint(-128, 128, (int(wild.sum()),), dtype=torch.int8)
+    z4[wild] = torch.randint(-128, 128, (int(wild.sum()),), dtype=torch.int8)
+    a = torch.randint(-3, 4, (M, K), dtype=torch.int8)
+    ones_a = torch.ones(M, K // 128, dtype=sdt)
+    ones_b = torch.ones((N + 127) // 128, K // 128, dtype=sdt)
+    packed, _ = bp.pack_rows(wq.numpy(), 4, 32)
+    with default_dtype(torch.float32):
+        c = w4a8_kernel.w4a8_gemm(a.to(dev), ones_a.to(dev), torch.from_numpy(packed).to(dev), ones_b.to(dev),
+                                  s4.to(dev), z4.to(dev))
+    b8 = q.w4a8_dequant_int8(wq, s4, z4)
+    assert torch.equal(c.cpu().long(), (a.double() @ b8.double().T).long())      # exact: every sum is far below 2^53
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 4096), (256, 1024, 7168), (512, 4096, 4096), (384, 14336, 4096),
+                                   (96, 2056, 14336)])
+def test_w4a8_mid_m_fused_tiles(dev, M, N, K):
+    """The same path on quantised operands with real scales, against the float64 oracle."""
+    announce("w4a8 fused tiles", M, N, K)
+    torch.manual_seed(N + K)
+    wq, s, s4, z4 = q.w4a8_weight_quant_levels(torch.randn(N, K) * 0.02)
+    a, a_s = q.act_quant_int8(torch.randn(M, K).bfloat16(), rounding="up")
+    packed, _ = bp.pack_rows(wq.numpy(), 4, 32)
+    with default_dtype(torch.bfloat16):
+        c = w4a8_kernel.w4a8_gemm(a.to(dev), a_s.to(dev), torch.from_numpy(packed).to(dev), s.to(dev),
+                                  s4.to(dev), z4.to(dev), 128, 8, "row")
+    assert_close_scaled(c, g.w4a8_gemm(a, a_s, wq, s, s4, z4), what="w4a8 fused tiles")
+
+
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("M,N,K,out", [(128, 1024, 4096, torch.bfloat16), (200, 520, 3200, torch.float32),
                                        (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16),
