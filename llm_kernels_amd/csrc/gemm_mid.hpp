@@ -30,6 +30,7 @@
 namespace llmk {
 
 constexpr int MD_BN = 64, MD_THREADS = 512;
+
 constexpr int MD_B = 4 * MD_BN * 128;                       // weight stage: [sub-block][column][128 B] = 32 KB
 constexpr int MD_S = 4 * 64 * 4;                            // activation-scale columns of a step: [sub-block][row] fp32
 constexpr int MD_RED_ROW = 68;                              // floats per row of the final reduction (64 + 4: bank spread)
@@ -41,19 +42,41 @@ constexpr int md_red(int mt) { return 4 * 16 * mt * MD_RED_ROW * 4; }
 // stages (reused by the reduction), weight-scale table, K_W4A8 table of zero points and second-level scales
 constexpr int md_lds(int mt, int kt_tab) { return md_stages(mt) + D_MAX_KT * 4 + 128 * kt_tab; }
 
+// f(integral_constant<I>) for I = FIRST .. LAST - 1 (ring slots are compile-time indices)
+template <int I, int LAST, class F>
+__device__ __forceinline__ void md_static_for(F&& f) {
+    if constexpr (I < LAST) {
+        f(std::integral_constant<int, I>{});
+        md_static_for<I + 1, LAST>(f);
+    }
+}
+// the same, nested: f(I) runs only if rem > I and f(I - 1) ran (a later step without the earlier ones is a path the
+// trip count rules out, and the static check of the assembly would still walk it)
+template <int I, int LAST, class F>
+__device__ __forceinline__ void md_static_nested(int rem, F&& f) {
+    if constexpr (I < LAST) {
+        if (rem > I) {
+            f(std::integral_constant<int, I>{});
+            md_static_nested<I + 1, LAST>(rem, f);
+        }
+    }
+}
+
 template <int KIND, int MT>
 __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     static_assert(MT == 4 || MT == 2, "tile rows");
     constexpr int BM = 16 * MT;
-    constexpr bool W4A8 = (KIND == K_W4A8);
+    constexpr bool W4A8 = (KIND == K_W4A8), W4NK = (KIND == K_W4NK);
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || W4A8);
     constexpr bool ROWCOL = (KIND == K_I8_ROWCOL);
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4NK) ? 2 : 1;
     constexpr int MD_A = md_a(MT);
-    constexpr int NB = W4A8 ? 2 : 4;                        // ring loads per thread and step
+    // ring loads per thread and step (K_W4NK: one vector of packed words in the ring proper, its group scale beside it)
+    constexpr int NB = W4A8 ? 2 : (W4NK ? 1 : 4);
+    constexpr int NBL = W4NK ? 2 : NB;                      // ... counted as loads
     // ring slots: weights are requested MD_RING - 1 steps ahead.  The block-scaled 8-bit kinds on the 64-row tile keep
     // products and accumulators apart and have no registers for a fourth slot (the build refuses spills in a
-    // kernel with hand-issued loads); three slots measured the same.
+    // kernel with hand-issued loads); three, four and five slots measured the same within the noise.
     constexpr int MD_RING = (SCALED && !W4A8 && MT == 4) ? 3 : 4;
     constexpr int NA = MT + (SCALED ? 1 : 0);               // direct-to-LDS loads per thread and step
     static_assert(md_red(MT) <= md_stages(MT), "the reduction reuses the stages");
@@ -99,7 +122,23 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     }
     uint32_t boff[4], blds[4];
     int bsub[4];
-    if constexpr (!W4A8) {
+    uint32_t w4_soff = 0;
+    int w4_shift = 0;
+    if constexpr (W4NK) {
+        // fp16 weight rows expanded from packed words [N, K/8]: thread t takes the 32 weights k = 32 seg .. + 31
+        // (seg = t & 7) of row t >> 3 of the step's 256: 16 bytes of packed words, four 16-byte chunks of the fp16
+        // row of sub-block seg >> 1, and the group scale of those weights (groups of 64 * 2^j elements)
+        const int row = tid >> 3, seg = tid & 7;
+        const uint32_t n = (uint32_t)min(n0 + row, N - 1);
+        boff[0] = n * (uint32_t)(p.K >> 1) + (uint32_t)(seg & 1) * 16u;       // + 32 bytes per sub-block
+        w4_soff = n * (uint32_t)(p.K / p.group) * 2u;
+        w4_shift = __builtin_ctz((unsigned)(p.group >> 6));
+        bsub[0] = seg >> 1;
+        blds[0] = (uint32_t)((seg >> 1) * (MD_BN * 128) + row * 128);
+        blds[1] = (uint32_t)(((4 * (seg & 1)) ^ ((row >> 1) & 7)) * 16);      // first chunk; chunk c is at ^ (c * 16)
+        boff[1] = boff[2] = boff[3] = blds[2] = blds[3] = 0;
+        bsub[1] = bsub[2] = bsub[3] = 0;
+    } else if constexpr (!W4A8) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int pq = 4 * wave + i, sub = pq >> 3, row = 8 * (pq & 7) + row8;
@@ -137,9 +176,16 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     };
     // ring of weight registers: slot = step % 4
     v4i ring[MD_RING][NB];
-    auto issue_b = [&](v4i (&rs)[NB], int s) __attribute__((always_inline)) {
+    unsigned ringsc[MD_RING] = {};                            // K_W4NK: group scale of the slot's weights (fp16 bits)
+    auto issue_b = [&](v4i (&rs)[NB], unsigned& rsc, int s) __attribute__((always_inline)) {
+        if constexpr (W4NK) {
+            // lane-dependent sub-block (the eight lanes of a row cover the four sub-blocks of the step)
+            const int kb0 = kblock(s, 0), kb = kt0 + min(4 * phys(s) + bsub[0], KT - 1);
+            rs[0] = asm_load_b128(boff[0] + (uint32_t)(kb - kb0) * 32u, (const uint8_t*)p.b + (int64_t)kb0 * 32);
+            rsc = asm_load_u16(w4_soff + (uint32_t)(kb >> w4_shift) * 2u, p.b_s);
+        }
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
+        for (int i = 0; i < (W4NK ? 0 : NB); ++i) {
             if constexpr (W4A8) {
                 // lane-dependent sub-block: the two halves of the wave read different 128-word runs of the row
                 const int kb0 = kblock(s, 2 * i), kb1 = kblock(s, 2 * i + 1);
@@ -151,17 +197,24 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
         }
     };
     // the loads of slot `slot` have landed when at most `younger` loads issued after them are in flight
-    auto ring_ready = [&](v4i (&rs)[NB], auto younger_c) __attribute__((always_inline)) {
+    auto ring_ready = [&](v4i (&rs)[NB], unsigned& rsc, auto younger_c) __attribute__((always_inline)) {
         constexpr int Y = decltype(younger_c)::value;
-        if constexpr (NB == 4)
+        if constexpr (W4NK)
+            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(rs[0]), "+v"(rsc) : "n"(Y) : "memory");
+        else if constexpr (NB == 4)
             asm volatile("s_waitcnt vmcnt(%4)" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]) : "n"(Y) : "memory");
         else
             asm volatile("s_waitcnt vmcnt(%2)" : "+v"(rs[0]), "+v"(rs[1]) : "n"(Y) : "memory");
     };
     // ring slot -> weight stage s & 1 (nobody has read that stage since the barrier of step s - 1)
-    auto produce = [&](const v4i (&rs)[NB], int s) __attribute__((always_inline)) {
+    auto produce = [&](const v4i (&rs)[NB], unsigned rsc, int s) __attribute__((always_inline)) {
         uint8_t* st = b_st + (s % MD_NBS) * MD_B;
-        if constexpr (!W4A8) {
+        if constexpr (W4NK) {
+            const v2h sc = w4_as_h2(rsc | (rsc << 16));
+            uint8_t* row = st + blds[0];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) *(v4i*)(row + (blds[1] ^ (uint32_t)(c * 16))) = w4_word_to_f16x8((unsigned)rs[0][c], sc);
+        } else if constexpr (!W4A8) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) *(v4i*)(st + blds[i]) = rs[i];
         } else {
@@ -241,19 +294,14 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     };
 
     const std::integral_constant<int, 0> c0;
-    const std::integral_constant<int, 1> c1;
-    const std::integral_constant<int, 2> c2;
-    const std::integral_constant<int, 3> c3;
-    const std::integral_constant<int, (MD_RING - 2) * NB> cpro;
-    const std::integral_constant<int, NB> cnb;
-    const std::integral_constant<int, NA + NB> cstep;
+    const std::integral_constant<int, (MD_RING - 2) * NBL> cpro;
+    const std::integral_constant<int, NBL> cnb;
+    const std::integral_constant<int, NA + NBL> cstep;
 
 
     // ---- prologue: activations of step 0, weights of steps 0, 1, 2; tables by ordinary loads meanwhile
     issue_a(0);
-    issue_b(ring[0], 0);
-    issue_b(ring[1], 1);
-    if constexpr (MD_RING == 4) issue_b(ring[2], 2);
+    md_static_for<0, MD_RING - 1>([&](auto ic) __attribute__((always_inline)) { issue_b(ring[ic.value], ringsc[ic.value], ic.value); });
     if constexpr (SCALED) {
         const int64_t bs_row = (int64_t)(n0 >> 7) * KT_all + kt0;
         for (int i = tid; i < KT; i += MD_THREADS) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
@@ -267,8 +315,8 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
         }
         __syncthreads();                                    // the table is read by produce()
     }
-    ring_ready(ring[0], cpro);
-    produce(ring[0], 0);
+    ring_ready(ring[0], ringsc[0], cpro);
+    produce(ring[0], ringsc[0], 0);
 
     // One step: wait for the activations of step s (requested a step ago; only the NB weight loads issued after
     // them may stay in flight; with four ring slots that also vouches for slot s + 1, requested two steps ago),
@@ -280,53 +328,28 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
         // (scheduling fences: without them the compiler carries the matrix instructions of a step across the next
         // barrier, with all fragments of two steps live, and spills)
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (MD_RING == 4) ring_ready(ring[(slot + 1) % MD_RING], cnb);
-        else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NB) : "memory");
+        if constexpr (MD_RING >= 4) ring_ready(ring[(slot + 1) % MD_RING], ringsc[(slot + 1) % MD_RING], cnb);
+        else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NBL) : "memory");
         __builtin_amdgcn_s_waitcnt(0xc07f);                 // lgkmcnt(0): this wave's LDS writes of produce() are done
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         issue_a(s + 1);
-        issue_b(ring[(slot + MD_RING - 1) % MD_RING], s + MD_RING - 1);
+        issue_b(ring[(slot + MD_RING - 1) % MD_RING], ringsc[(slot + MD_RING - 1) % MD_RING], s + MD_RING - 1);
         __builtin_amdgcn_sched_barrier(0);
         compute(s);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (MD_RING == 3) ring_ready(ring[(slot + 1) % MD_RING], cstep);
-        produce(ring[(slot + 1) % MD_RING], s + 1);
+        if constexpr (MD_RING == 3) ring_ready(ring[(slot + 1) % MD_RING], ringsc[(slot + 1) % MD_RING], cstep);
+        produce(ring[(slot + 1) % MD_RING], ringsc[(slot + 1) % MD_RING], s + 1);
         __builtin_amdgcn_sched_barrier(0);
     };
     int s = 0;
     for (int rd = nsteps / MD_RING; rd > 0; --rd) {
-        step(c0, s);
-        step(c1, s + 1);
-        step(c2, s + 2);
-        if constexpr (MD_RING == 4) step(c3, s + 3);
+        md_static_for<0, MD_RING>([&](auto ic) __attribute__((always_inline)) { step(ic, s + ic.value); });
         s += MD_RING;
     }
-    const int rem = nsteps % MD_RING;
-    // (nested: a later step without the earlier ones is a path the trip count rules out, and the static check of
-    // the assembly would still walk it)
-    if (rem > 0) {
-        step(c0, s);
-        if (rem > 1) {
-            step(c1, s + 1);
-            if constexpr (MD_RING == 4) { if (rem > 2) step(c2, s + 2); }
-        }
-    }
+    md_static_nested<0, MD_RING - 1>(nsteps % MD_RING, [&](auto ic) __attribute__((always_inline)) { step(ic, s + ic.value); });
     // everything requested has landed (also the repeated loads past the end) before the stages are reused
-    if constexpr (NB == 4 && MD_RING == 3) {
-        asm volatile("s_waitcnt vmcnt(0)"
-                     : "+v"(ring[0][0]), "+v"(ring[0][1]), "+v"(ring[0][2]), "+v"(ring[0][3]), "+v"(ring[1][0]), "+v"(ring[1][1]),
-                       "+v"(ring[1][2]), "+v"(ring[1][3]), "+v"(ring[2][0]), "+v"(ring[2][1]), "+v"(ring[2][2]), "+v"(ring[2][3]) : : "memory");
-    } else if constexpr (NB == 4) {
-        asm volatile("s_waitcnt vmcnt(0)"
-                     : "+v"(ring[0][0]), "+v"(ring[0][1]), "+v"(ring[0][2]), "+v"(ring[0][3]), "+v"(ring[1][0]), "+v"(ring[1][1]),
-                       "+v"(ring[1][2]), "+v"(ring[1][3]), "+v"(ring[2][0]), "+v"(ring[2][1]), "+v"(ring[2][2]), "+v"(ring[2][3]),
-                       "+v"(ring[3][0]), "+v"(ring[3][1]), "+v"(ring[3][2]), "+v"(ring[3][3]) : : "memory");
-    } else {
-        asm volatile("s_waitcnt vmcnt(0)"
-                     : "+v"(ring[0][0]), "+v"(ring[0][1]), "+v"(ring[1][0]), "+v"(ring[1][1]), "+v"(ring[2][0]), "+v"(ring[2][1]),
-                       "+v"(ring[3][0]), "+v"(ring[3][1]) : : "memory");
-    }
+    md_static_for<0, MD_RING>([&](auto ic) __attribute__((always_inline)) { ring_ready(ring[ic.value], ringsc[ic.value], c0); });
     __syncthreads();
 
     // ---- the four sub-block sums of every output meet in LDS: red[kq][row][column], rows of 68 floats
@@ -411,8 +434,9 @@ inline MidPlan mid_plan(int64_t M, int64_t N, int64_t kbytes) {
 // K_W4A8 kind room for its table behind the stages.
 template <int KIND>
 inline bool mid_eligible(const DirectArgs& p, int mt, int ksplit) {
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK) ? 2 : 1;
     if (!dma_eligible(p, ESZ)) return false;
+    if (KIND == K_W4NK && (p.group < 64 || (p.group & (p.group - 1)))) return false;      // groups of 64 * 2^j elements
     const int KT_all = (p.K * ESZ) >> 7;
     const int per = ksplit > 1 ? ((((KT_all + ksplit - 1) / ksplit) + 3) & ~3) : KT_all;
     return md_lds(mt, KIND == K_W4A8 ? per : 0) <= D_LDS_MAX;
@@ -423,7 +447,7 @@ template <int KIND, int MT>
 int launch_mid(const DirectArgs& p, hipStream_t stream, const char* name) {
     static std::atomic<uint64_t> configured{0};
     auto kern = gemm_mid_kernel<KIND, MT>;
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK) ? 2 : 1;
     const int KT_all = (p.K * ESZ) >> 7;
     const bool split = p.ksplit > 1 && p.partial;
     const int per = split ? ((((KT_all + p.ksplit - 1) / p.ksplit) + 3) & ~3) : KT_all;

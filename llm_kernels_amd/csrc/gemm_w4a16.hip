@@ -2,6 +2,7 @@
 //
 // nibble -> fp16 without integer->float converts: (q | 0x6400) is the fp16 number 1024 + q,
 // ((q << 4) | 0x6400) is 1024 + 16 q; one packed subtract / fma gives q - 8 exactly.
+#include <algorithm>
 #include "gemm_wide.hpp"
 #include "stream_ring.hpp"
 
@@ -1003,6 +1004,16 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
         llmk::DirectArgs p{};
         p.a = (const uint8_t*)a; p.b = (const uint8_t*)b_packed; p.b_s = s; p.c = c; p.c_dtype = LLMK_F16;
         p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1; p.group = groupsize;
+        // few column tiles and short rows: the 64-column kernel with 512-byte K steps (128 x 4096 x 4096: 18.3 -> 14 us)
+        if (llmk::mid_wanted(M, N, 2 * K)) {
+            llmk::MidPlan pl = llmk::mid_plan(M, N, 2 * K);
+            if (pl.z > 1 && !(workspace && workspace_bytes >= (int64_t)pl.z * M * N * 4 && !((uintptr_t)workspace & 15))) pl.z = 1;
+            if (llmk::mid_eligible<llmk::K_W4NK>(p, pl.mt, pl.z)) {
+                if (pl.z > 1) { p.partial = (float*)workspace; p.ksplit = pl.z; }
+                return pl.mt == 4 ? llmk::launch_mid<llmk::K_W4NK, 4>(p, st, "gemm_w4a16_nk(mid)")
+                                  : llmk::launch_mid<llmk::K_W4NK, 2>(p, st, "gemm_w4a16_nk(mid)");
+            }
+        }
         if (llmk::dma_eligible(p, 2))
             return llmk::launch_big_half<llmk::K_W4NK, false>(p, st, "gemm_w4a16_nk(fused tiles)", workspace, workspace_bytes);
     }
