@@ -509,8 +509,27 @@ def calibration(dev):
         dt_s = timed(lambda: _lib.call("llmk_calib_mfma", kind, iters, _lib.ptr(ops), _lib.ptr(out), cus, _lib.ptr(clocks), st))
         res["mfma_%s_sustained_tflops" % name] = round(cus * 8 * iters * 32 * flops_per_mfma / dt_s / 1e12, 1)
         ck = clocks.tolist()
-        if ck[1] > 0:
-            res["mfma_%s_loop_ticks_per_100mhz_tick" % name] = round(ck[0] / ck[1], 3)
+        if ck[1] > 0:            # s_memtime counts the shader clock, s_memrealtime a constant 100 MHz
+            res["shader_clock_mhz_in_mfma_%s_loop" % name] = round(100.0 * ck[0] / ck[1], 0)
+    # the shader clock the headline GEMM itself runs at (fp8 4096^3 on random operands, first workgroup's lifetime)
+    from llm_kernels_amd.quantization import fp8_kernel
+    M = N = K = 4096
+    a, a_s = fp8_kernel.act_quant(torch.randn(M, K, device=dev).bfloat16())
+    b, b_s = fp8_kernel.weight_quant(torch.randn(N, K, device=dev) * 0.02)
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    wsp, wsn = _lib.gemm_workspace(dev, M, N, K)
+    clocks.zero_()
+    gemm = lambda: _lib.call("llmk_calib_gemm_fp8_clock", _lib.ptr(a), _lib.ptr(a_s), _lib.ptr(b), _lib.ptr(b_s), _lib.ptr(c),
+                             _lib.BF16, M, N, K, wsp, wsn, _lib.ptr(clocks), st)
+    for _ in range(50):
+        gemm()
+    dt_s = timed(gemm, reps=9)
+    ck = clocks.tolist()
+    if ck[1] > 0:
+        res["shader_clock_mhz_in_fp8_gemm_4096"] = round(100.0 * ck[0] / ck[1], 0)
+        res["fp8_gemm_4096_workgroup_lifetime_us"] = round(ck[1] / 100.0, 2)
+        res["fp8_gemm_4096_eager_us"] = round(dt_s * 1e6, 2)
+    del a, a_s, b, b_s, c
     global _flush_buf
     if _flush_buf is None:
         _flush_buf = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
@@ -519,7 +538,8 @@ def calibration(dev):
         dt_s = timed(lambda: _lib.call("llmk_calib_read", _lib.ptr(_flush_buf), _flush_buf.numel(), pattern, _lib.ptr(sink), wgs, st))
         res[name] = round(_flush_buf.numel() / dt_s / 1e9, 1)
     res["note"] = ("sustained rates of this box by the library's calibration kernels; roofline.peak stays the published "
-                   "figure (HBM 8000 GB/s; fp8 / int8 5000, fp16 / bf16 2500 TFLOP/s)")
+                   "figure (HBM 8000 GB/s; fp8 / int8 5000, fp16 / bf16 2500 TFLOP/s, which assume the 2400 MHz peak "
+                   "engine clock: the shader clocks above are what the chip holds under each load)")
     return res
 
 

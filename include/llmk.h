@@ -272,6 +272,11 @@ int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind, int c_dty
 int llmk_calib_mfma(int kind, int iters, const void* operands, float* out, int workgroups, long long* clocks,
                     void* stream);
 int llmk_calib_read(const void* src, int64_t nbytes, int pattern, int* sink, int workgroups, void* stream);
+/* llmk_gemm_fp8_block (same operands, M > 512) whose first workgroup also reports the shader clock it ran at:
+ * clocks[0] = s_memtime ticks, clocks[1] = s_memrealtime (100 MHz) ticks between its first and its last instruction. */
+int llmk_calib_gemm_fp8_clock(const void* a_e4m3, const float* a_s, const void* b_e4m3, const float* b_s, void* c,
+                              int c_dtype, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                              long long* clocks, void* stream);
 
 #ifdef __cplusplus
 }

@@ -64,6 +64,7 @@ SIGNATURES = {
     "llmk_moe_expert_scales": [_p, _p, _p, _i, _i, _l, _l, _l, _p, _p, _i, _p],
     "llmk_calib_mfma": [_i, _i, _p, _p, _i, _p, _p],
     "llmk_calib_read": [_p, _l, _i, _p, _i, _p],
+    "llmk_calib_gemm_fp8_clock": [_p, _p, _p, _p, _p, _i, _l, _l, _l, _p, _l, _p, _p],
     "llmk_grouped_gemm": [_p, _p, _p, _i, _i, _i, _l, _l, _l, _p, _p, _p, _p, _i, _p, _l, _p],
 }
 _RESTYPE = {"llmk_last_error": _c.c_char_p, "llmk_gemm_workspace_bytes": _l, "llmk_gemm_w4a8_workspace_bytes": _l,

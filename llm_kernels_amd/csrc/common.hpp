@@ -136,6 +136,23 @@ __device__ __forceinline__ v4f mfma_bf16_16x16x32(v8bf a, v8bf b, v4f c) {
 
 static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Compute units of MI355X: the tile kernels plan their launches in rounds of this many workgroups (one per CU).
+// The plans stay correct on a device with another count (every tile is still computed exactly once); the
+// launchers only take the K split of a short last round when the device really has this many.
+constexpr int LLMK_CUS = 256;
+// compute units of the current device (0 if the query fails); cached per process
+static inline int llmk_device_cus() {
+    static std::atomic<int> cache{0};
+    int cus = cache.load(std::memory_order_relaxed);
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 0)
+            cus = 0;
+        cache.store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
 // ------------------------------------------------------------------ one-time launch set-up (host)
 // Opt a kernel into more than 64 KB of dynamic LDS, once per device.  `done` is a bit mask of the device
 // ordinals already configured (one static mask per launch site); the call is idempotent, so two threads that

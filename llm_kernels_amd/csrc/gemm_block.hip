@@ -84,6 +84,21 @@ extern "C" int llmk_gemm_fp8_block(const void* a, const float* a_s, const void* 
     return launch_stream<K_FP8_BLOCK>(p, workspace, workspace_bytes, (hipStream_t)stream, "gemm_fp8_block");
 }
 
+// llmk_gemm_fp8_block for the benchmark's calibration: the same launch, and workgroup 0 of the 256-column tile kernel
+// reports the ticks of the shader clock and of the 100 MHz clock it lived (clocks[0], clocks[1]); shapes that run on
+// other kernels leave clocks untouched.
+extern "C" int llmk_calib_gemm_fp8_clock(const void* a, const float* a_s, const void* b, const float* b_s, void* c,
+                                         int c_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                         int64_t workspace_bytes, long long* clocks, void* stream) {
+    int rc = check_common("calib_gemm_fp8_clock", a, b, M, N, K, c_dtype);
+    if (rc) return rc;
+    if (M <= 512 || N == 0 || !c || !a_s || !b_s || !clocks) LLMK_FAIL(LLMK_ERR_ARG, "calib_gemm_fp8_clock: needs M > 512 and every pointer");
+    DirectArgs p{};
+    p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s; p.clocks = clocks;
+    p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;
+    return launch_big<K_FP8_BLOCK, false>(p, workspace, workspace_bytes, (hipStream_t)stream, "calib_gemm_fp8_clock");
+}
+
 extern "C" int llmk_gemm_i8_block(const int8_t* a, const void* a_s, const int8_t* b, const void* b_s, int s_dtype,
                                   void* c, int c_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                                   int64_t workspace_bytes, void* stream) {

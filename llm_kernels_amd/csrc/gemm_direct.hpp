@@ -100,6 +100,7 @@ struct DirectArgs {
     int ksplit;            // 0 / 1 = no split
     int kc_steps;          // weight-streaming kernel with K ranges: 128-byte steps per range (gridDim.z ranges)
     int group;             // K_W4NK / K_W4MARLIN: K elements per fp16 group scale
+    long long* clocks;     // 256-column tile kernel, calibration only: workgroup 0 leaves the s_memtime and s_memrealtime ticks it lived
     const int8_t* w4_s4;   // K_W4A8: second-level scales [N, K/128]
     const int8_t* w4_z4;   // K_W4A8: zero points [N, K/128]
     int tail_split;        // 256-column tile kernel: the tiles of a short last round are split along K (partial = scratch)

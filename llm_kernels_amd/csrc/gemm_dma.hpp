@@ -37,6 +37,10 @@ __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const vo
 __device__ __forceinline__ void dma4(uint32_t lds_addr, uint32_t voff, const void* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
+// 16-bit element -> one dword per lane in LDS (zero-extended)
+__device__ __forceinline__ void dma2(uint32_t lds_addr, uint32_t voff, const void* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
 // s_waitcnt immediates for gfx9: vmcnt = imm[3:0] | imm[15:14] << 4, expcnt = imm[6:4] (7 = no wait),
 // lgkmcnt = imm[11:8] (15 = no wait)
 #define LLMK_WAIT_VMCNT_7 0x0F77

@@ -62,7 +62,9 @@ __device__ __forceinline__ void md_static_nested(int rem, F&& f) {
     }
 }
 
-template <int KIND, int MT>
+// AS16: the activation scales are 16-bit (fp16 or bf16 by p.s_dtype) and are staged as they are (one zero-extended
+// element per dword slot of the scale column) instead of being widened to fp32 by a kernel of their own first.
+template <int KIND, int MT, bool AS16 = false>
 __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     static_assert(MT == 4 || MT == 2, "tile rows");
     constexpr int BM = 16 * MT;
@@ -158,7 +160,8 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
         boff[2] = boff[3] = blds[2] = blds[3] = 0;
         bsub[2] = bsub[3] = 0;
     }
-    const uint32_t soff = (uint32_t)min(m_start + min(lane, BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
+    constexpr uint32_t SSZ = AS16 ? 2u : 4u;                // bytes per activation scale
+    const uint32_t soff = (uint32_t)min(m_start + min(lane, BM - 1), m_end - 1) * (uint32_t)KT_all * SSZ;
 
     // sub-block `sub` of step s, clamped to the last one of the range (loads past the end repeat it)
     // requests past the end repeat the last step
@@ -171,7 +174,8 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
         for (int i = 0; i < MT; ++i) dma16(st + alds[i], aoff[i], p.a + (int64_t)kblock(s, asub[i]) * 128);
         if constexpr (SCALED) {
             const uint32_t ss = lds_base + MD_NA * MD_A + MD_NBS * MD_B + (uint32_t)(s % MD_NA) * MD_S + (uint32_t)(wave & 3) * 256u;
-            dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 4);
+            if constexpr (AS16) dma2(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 2);
+            else dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 4);
         }
     };
     // ring of weight registers: slot = step % 4
@@ -267,7 +271,14 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
             const float bs = live ? bsl[min(kb, KT - 1)] : 0.f;
             float sa[MT];
 #pragma unroll
-            for (int i = 0; i < MT; ++i) sa[i] = Ss[16 * i] * bs;
+            for (int i = 0; i < MT; ++i) {
+                if constexpr (AS16) {
+                    const unsigned raw = ((const unsigned*)Ss)[16 * i];
+                    sa[i] = (p.s_dtype == LLMK_F16 ? f16_to_f32((unsigned short)raw) : bf16_to_f32((unsigned short)raw)) * bs;
+                } else {
+                    sa[i] = Ss[16 * i] * bs;
+                }
+            }
             // the products of tile row i are scaled and accumulated while the matrix instructions of row i + 1 run
             v4f t[2][2];
 #pragma unroll
@@ -407,8 +418,8 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
 // K slices of the mid-size kernel: as many as bring the grid to about one workgroup per CU, in whole steps of 512
 // bytes, each slice at least four steps long; 1 = no split.
 inline int mid_splitk(int64_t tiles, int64_t kbytes) {
-    if (tiles >= 192) return 1;
-    int64_t z = 256 / tiles;
+    if (tiles >= 3 * LLMK_CUS / 4) return 1;
+    int64_t z = LLMK_CUS / tiles;
     const int64_t steps = kbytes >> 9;
     if (z > steps / 4) z = steps / 4;
     return (int)(z > 8 ? 8 : (z < 1 ? 1 : z));
@@ -424,7 +435,7 @@ inline MidPlan mid_plan(int64_t M, int64_t N, int64_t kbytes) {
     MidPlan pl;
     const int64_t gx = (N + MD_BN - 1) / MD_BN;
     const int64_t t4 = ((M + 63) / 64) * gx, t2 = ((M + 31) / 32) * gx;
-    pl.mt = (t4 <= 128 && t2 > t4) ? 2 : 4;
+    pl.mt = (t4 <= LLMK_CUS / 2 && t2 > t4) ? 2 : 4;
     pl.tiles = pl.mt == 4 ? t4 : t2;
     pl.z = mid_splitk(pl.tiles, kbytes);
     return pl;
@@ -442,11 +453,12 @@ inline bool mid_eligible(const DirectArgs& p, int mt, int ksplit) {
     return md_lds(mt, KIND == K_W4A8 ? per : 0) <= D_LDS_MAX;
 }
 
-// a_s must be fp32 here (p.a_s); p.s_dtype describes b_s only.  p.ksplit / p.partial select the K split.
-template <int KIND, int MT>
+// p.a_s: fp32, or with AS16 the 16-bit scales of dtype p.s_dtype as the caller passed them; p.s_dtype describes b_s
+// (and those).  p.ksplit / p.partial select the K split.
+template <int KIND, int MT, bool AS16 = false>
 int launch_mid(const DirectArgs& p, hipStream_t stream, const char* name) {
     static std::atomic<uint64_t> configured{0};
-    auto kern = gemm_mid_kernel<KIND, MT>;
+    auto kern = gemm_mid_kernel<KIND, MT, AS16>;
     constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK) ? 2 : 1;
     const int KT_all = (p.K * ESZ) >> 7;
     const bool split = p.ksplit > 1 && p.partial;

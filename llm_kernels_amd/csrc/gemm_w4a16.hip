@@ -764,7 +764,8 @@ int launch_nk_ring(const void* A, const int32_t* B, const _Float16* S, void* C, 
     // One workgroup per CU and row tile, ring depth = tiles per workgroup (two to four).  Two workgroups per CU
     // with rings of two measured slower (20.4 vs 18.2 us at N = 28672): every workgroup reads all the activations
     // of its row tile, and that traffic doubles.
-    const int wg = min(ntiles, max(1, 256 / min(rows, 256)));
+    const int cus = std::max(1, llmk_device_cus() > 0 ? llmk_device_cus() : LLMK_CUS);
+    const int wg = min(ntiles, max(1, cus / min(rows, cus)));
     const int per_wg = (ntiles + wg - 1) / wg;
     dim3 rgrid((unsigned)((ntiles + per_wg - 1) / per_wg), (unsigned)mtiles, (unsigned)nz);
     // reduction buffers + the wave-private staging area of the activations

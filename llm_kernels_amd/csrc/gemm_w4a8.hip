@@ -406,14 +406,8 @@ int launch_w4a8_stream(W4A8Args p, void* workspace, int64_t workspace_bytes, hip
     static std::atomic<uint64_t> cfg1{0}, cfg2{0};
     if (int rc = llmk_reserve_lds((const void*)k1, 160 * 1024, cfg1, "gemm_w4a8")) return rc;
     if (int rc = llmk_reserve_lds((const void*)k2, 160 * 1024, cfg2, "gemm_w4a8")) return rc;
-    static std::atomic<int> cus_cache{0};
-    int cus = cus_cache.load(std::memory_order_relaxed);
-    if (cus == 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot query the device");
-        cus_cache.store(cus, std::memory_order_relaxed);
-    }
+    const int cus = llmk_device_cus();
+    if (cus <= 0) LLMK_FAIL(LLMK_ERR_LAUNCH, "gemm_w4a8: cannot query the device");
     const int rows = mtiles * nz;                                      // workgroup rows that share the column tiles
     int gx = min(ntiles, max(1, cus / min(rows, cus)));                // one workgroup per CU (LDS bound)
     { const int per_wg = (ntiles + gx - 1) / gx; gx = (ntiles + per_wg - 1) / per_wg; }   // equal tile counts
@@ -456,7 +450,7 @@ W4A8Plan w4a8_plan(int64_t M, int64_t N, int64_t K, int group_int4) {
     // (the hand-issued loads of the fused kernel take 32-bit lane offsets into the activations and the tables)
     const bool small_offsets = M * K < (1ll << 32) && N * (K / 128) < (1ll << 32);
     // 65 to 256 rows on at most one 64-column workgroup per CU: the tile kernel with 512-byte K steps
-    const bool mid = M > 64 && M <= 256 && mid_plan(M, N, K).tiles <= 256 && K <= 16384;
+    const bool mid = M > 64 && M <= 256 && mid_plan(M, N, K).tiles <= LLMK_CUS && K <= 16384;
     pl.stream = fused_wins && long_k_ok && small_offsets && group_int4 == 128 && !mid;
     // Mid-size M: the tile kernels unpack and dequantise inside their K loop (one pass over the packed words; the
     // separate expansion writes and re-reads N * K bytes).  Measured (us per launch, fused | expansion + int8 GEMM):
@@ -477,6 +471,18 @@ W4A8Plan w4a8_plan(int64_t M, int64_t N, int64_t K, int group_int4) {
 // scale elements), few tiles split K over workgroups with fp32 partial sums behind them.
 int launch_w4a8_tiles(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
     const char* name = "gemm_w4a8(fused tiles)";
+    // the 64-column kernel takes 16-bit activation scales as they are
+    if (p.M <= 256 && mid_plan(p.M, p.N, p.K).tiles <= LLMK_CUS && p.K <= 16384) {
+        MidPlan pl = mid_plan(p.M, p.N, p.K);
+        if (pl.z > 1 && workspace_bytes < (int64_t)pl.z * p.M * p.N * 4) pl.z = 1;
+        if (mid_eligible<K_W4A8>(p, pl.mt, pl.z)) {
+            if (pl.z > 1) { p.partial = (float*)workspace; p.ksplit = pl.z; }
+            if (p.s_dtype != LLMK_F32)
+                return pl.mt == 4 ? launch_mid<K_W4A8, 4, true>(p, stream, name) : launch_mid<K_W4A8, 2, true>(p, stream, name);
+            return pl.mt == 4 ? launch_mid<K_W4A8, 4>(p, stream, name) : launch_mid<K_W4A8, 2>(p, stream, name);
+        }
+    }
+    // the 128-column kernels stream 4-byte scale elements: 16-bit scales are widened into the workspace first
     int64_t used = 0;
     if (p.s_dtype != LLMK_F32) {
         const int64_t n = (int64_t)p.M * (p.K >> 7);
@@ -486,14 +492,6 @@ int launch_w4a8_tiles(DirectArgs p, void* workspace, int64_t workspace_bytes, hi
         LLMK_CHECK_LAUNCH(name);
         p.a_s = workspace;
         used = (n * 4 + 255) & ~(int64_t)255;
-    }
-    if (p.M <= 256 && mid_plan(p.M, p.N, p.K).tiles <= 256 && p.K <= 16384) {
-        MidPlan pl = mid_plan(p.M, p.N, p.K);
-        if (pl.z > 1 && workspace_bytes - used < (int64_t)pl.z * p.M * p.N * 4) pl.z = 1;
-        if (mid_eligible<K_W4A8>(p, pl.mt, pl.z)) {
-            if (pl.z > 1) { p.partial = (float*)((uint8_t*)workspace + used); p.ksplit = pl.z; }
-            return pl.mt == 4 ? launch_mid<K_W4A8, 4>(p, stream, name) : launch_mid<K_W4A8, 2>(p, stream, name);
-        }
     }
     const int z = splitk_factor(p.M, p.N, p.K);
     if (z > 1 && workspace_bytes - used >= (int64_t)z * p.M * p.N * 4) {

@@ -52,9 +52,9 @@ __device__ __forceinline__ WideTile wide_tile_of(const DirectArgs& p, int lin, i
         constexpr int H = 4;      // strips of 8 or 16 tile rows measured 1-13 % slower
         if (gy % H == 0) {
             int lp = lin;
-            if (lin < (total & ~255)) {
-                const int w = lin & 255;
-                lp = (lin & ~255) + (w & 7) * 32 + (w >> 3);
+            if (lin < (total & ~(LLMK_CUS - 1))) {
+                const int w = lin & (LLMK_CUS - 1);
+                lp = (lin & ~(LLMK_CUS - 1)) + (w & 7) * (LLMK_CUS / 8) + (w >> 3);
             }
             const int strip = lp / (H * gx), rr = lp % (H * gx);
             bx = rr / H;
@@ -131,12 +131,12 @@ struct WideTail {
 constexpr int W_TAIL_MIN_KT = 64;
 __host__ __device__ inline WideTail wide_tail_plan(int total, int KT) {
     WideTail w;
-    w.full = total & ~255;
+    w.full = total & ~(LLMK_CUS - 1);
     w.ntail = total - w.full;
     w.z = 1;
     w.ktz = KT;
-    if (w.ntail > 0 && w.ntail <= 128 && KT >= W_TAIL_MIN_KT) {
-        int z = 256 / w.ntail;
+    if (w.ntail > 0 && w.ntail <= LLMK_CUS / 2 && KT >= W_TAIL_MIN_KT) {
+        int z = LLMK_CUS / w.ntail;
         if (z > 8) z = 8;
         int ktz = ((KT + z - 1) / z + 1) & ~1;
         if (ktz < 8) ktz = 8;
@@ -149,7 +149,7 @@ __host__ __device__ inline WideTail wide_tail_plan(int total, int KT) {
     }
     return w;
 }
-constexpr int W_TAIL_ITEMS = 256;               // upper bound of ntail * z
+constexpr int W_TAIL_ITEMS = LLMK_CUS;          // upper bound of ntail * z
 
 template <int KIND, bool GROUPED, int R = 8>
 __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
@@ -177,6 +177,10 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     float* part = nullptr;
     const int gx = gridDim.x;
     int lin = blockIdx.y * gx + blockIdx.x;
+    // calibration runs only: the shader clock this workgroup saw (ticks of the core clock per tick of the 100 MHz clock)
+    const bool clocked = p.clocks && lin == 0 && tid == 0;
+    long long clk0 = 0, wall0 = 0;
+    if (clocked) { clk0 = clock64(); wall0 = wall_clock64(); }
     WideTile wt = wide_tile_of<GROUPED, R>(p, lin, gx);
     if (p.tail_split) {
         // (the tiles of all but the last round need nothing of this: for them the plan only confirms lin < full;
@@ -513,9 +517,15 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     }
 
     // ---- epilogue: the rows not yet stored by the last K step
-    if (KT > 0) { store_row(R - 1); return; }
+    if (KT > 0) store_row(R - 1);
+    else {
 #pragma unroll
-    for (int i = 0; i < R; ++i) store_row(i);
+        for (int i = 0; i < R; ++i) store_row(i);
+    }
+    if (clocked) {
+        p.clocks[0] = clock64() - clk0;
+        p.clocks[1] = wall_clock64() - wall0;
+    }
 }
 
 // Adds the partial sums of the split last round (see wide_tail_plan) and writes the outputs of its tiles: grid
@@ -572,8 +582,9 @@ int launch_wide(const DirectArgs& p0, hipStream_t stream, const char* name, void
     p.tail_split = 0;
     if constexpr (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || KIND == K_F16 || KIND == K_BF16) {
         const int KT = (p.K * ESZ) >> 7;
-        if (ws && ws_bytes >= w_tail_bytes() && !((uintptr_t)ws & 15) && KT >= W_TAIL_MIN_KT && p.c)
-            tail = GROUPED ? (int64_t)grid.x * grid.y >= 256 : wide_tail_plan((int)(grid.x * grid.y), KT).z > 1;
+        // (the split is planned for rounds of LLMK_CUS workgroups: taken only on a device with that many CUs)
+        if (ws && ws_bytes >= w_tail_bytes() && !((uintptr_t)ws & 15) && KT >= W_TAIL_MIN_KT && p.c && llmk_device_cus() == LLMK_CUS)
+            tail = GROUPED ? (int64_t)grid.x * grid.y >= LLMK_CUS : wide_tail_plan((int)(grid.x * grid.y), KT).z > 1;
     }
     if (tail) {
         p.tail_split = 1;
@@ -583,7 +594,7 @@ int launch_wide(const DirectArgs& p0, hipStream_t stream, const char* name, void
     kern<<<grid, W_THREADS, W_LDS, stream>>>(p);
     LLMK_CHECK_LAUNCH(name);
     if (tail) {
-        wide_tail_sum_kernel<GROUPED, R><<<dim3(128, W_BM / 32), 256, 0, stream>>>(p, ESZ);
+        wide_tail_sum_kernel<GROUPED, R><<<dim3(LLMK_CUS / 2, W_BM / 32), 256, 0, stream>>>(p, ESZ);
         LLMK_CHECK_LAUNCH(name);
     }
     return LLMK_OK;
@@ -595,8 +606,8 @@ int launch_wide(const DirectArgs& p0, hipStream_t stream, const char* name, void
 inline int splitk_factor(int64_t M, int64_t N, int64_t K) {
     if (M <= 16 || M > 512) return 1;
     const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
-    if (tiles >= 256 || (tiles >= 128 && K < 8192)) return 1;
-    int64_t z = (255 + tiles) / tiles;
+    if (tiles >= LLMK_CUS || (tiles >= LLMK_CUS / 2 && K < 8192)) return 1;
+    int64_t z = (LLMK_CUS - 1 + tiles) / tiles;
     z = z < (K >> 10) ? z : (K >> 10);
     return (int)(z > 8 ? 8 : (z < 1 ? 1 : z));
 }
@@ -607,7 +618,7 @@ inline int splitk_factor(int64_t M, int64_t N, int64_t K) {
 // (512 x 4096 x 4096 15.5 -> 23.4, 256 x 6144 x 4096 23.5 -> 27.9, 256 x 4096 x 14336 43.9 -> 47.0).
 inline bool mid_wanted(int64_t M, int64_t N, int64_t kbytes) {
     if (M <= 64 || M > 512) return false;
-    return mid_plan(M, N, kbytes).tiles <= 256 && kbytes <= 8192;
+    return mid_plan(M, N, kbytes).tiles <= LLMK_CUS && kbytes <= 8192;
 }
 
 // 16 < M <= 64: the weight-streaming kernel re-reads the activations for every 16 columns, which costs more
@@ -631,7 +642,7 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* 
     // a segment of a grouped GEMM rarely ends on a tile boundary: count one ragged tile per segment on top of
     // the full ones (with the plain ceiling, segments of 128 +- a few rows looked like one 128-row tile each and
     // went to a tile shape that needed two; -8 % on the Mixtral forward at 256 and 512 tokens)
-    auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * (GROUPED ? rows / bm + 1 : (rows + bm - 1) / bm) + 255) / 256; };
+    auto rounds = [&](int bm, int bn) { return (((p.N + bn - 1) / bn) * groups * (GROUPED ? rows / bm + 1 : (rows + bm - 1) / bm) + LLMK_CUS - 1) / LLMK_CUS; };
     const double t_wide = 60.0 * rounds(256, 256), t4 = 43.0 * rounds(256, 128), t2 = 26.0 * rounds(128, 128),
                  t1 = 16.0 * rounds(64, 128);
     if constexpr (HAS_WIDE) {
@@ -660,6 +671,23 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* 
 template <int KIND, bool GROUPED>
 int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream_t stream, const char* name) {
     if (!dma_eligible(p)) return launch_tiled<KIND, GROUPED>(p, stream, name);
+    // Mid-size M on few column tiles: the 64-column kernel with 512-byte K steps; it stages 16-bit activation scales
+    // as they are, so no widening pass runs in front of it
+    if constexpr (!GROUPED) {
+        if (mid_wanted(p.M, p.N, p.K) && (KIND != K_FP8_BLOCK || p.s_dtype == LLMK_F32)) {
+            MidPlan pl = mid_plan(p.M, p.N, p.K);
+            const int64_t need = (int64_t)pl.z * p.M * p.N * 4;
+            if (pl.z > 1 && !(workspace && workspace_bytes >= need && !(((uintptr_t)workspace) & 15))) pl.z = 1;
+            if (mid_eligible<KIND>(p, pl.mt, pl.z)) {
+                if (pl.z > 1) { p.partial = (float*)workspace; p.ksplit = pl.z; }
+                if (p.s_dtype != LLMK_F32) {
+                    if constexpr (KIND != K_FP8_BLOCK)
+                        return pl.mt == 4 ? launch_mid<KIND, 4, true>(p, stream, name) : launch_mid<KIND, 2, true>(p, stream, name);
+                }
+                return pl.mt == 4 ? launch_mid<KIND, 4>(p, stream, name) : launch_mid<KIND, 2>(p, stream, name);
+            }
+        }
+    }
     int64_t used = 0;
     if (p.s_dtype != LLMK_F32) {
         const int64_t n = (int64_t)p.M * (p.K >> 7);
@@ -670,18 +698,6 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
         LLMK_CHECK_LAUNCH(name);
         p.a_s = workspace;
         used = (n * 4 + 255) & ~(int64_t)255;
-    }
-    // Mid-size M on few column tiles: the 64-column kernel with 512-byte K steps
-    if constexpr (!GROUPED) {
-        if (mid_wanted(p.M, p.N, p.K)) {
-            MidPlan pl = mid_plan(p.M, p.N, p.K);
-            const int64_t need = (int64_t)pl.z * p.M * p.N * 4;
-            if (pl.z > 1 && !(workspace && workspace_bytes - used >= need && !(((uintptr_t)workspace + used) & 15))) pl.z = 1;
-            if (mid_eligible<KIND>(p, pl.mt, pl.z)) {
-                if (pl.z > 1) { p.partial = (float*)((uint8_t*)workspace + used); p.ksplit = pl.z; }
-                return pl.mt == 4 ? launch_mid<KIND, 4>(p, stream, name) : launch_mid<KIND, 2>(p, stream, name);
-            }
-        }
     }
     // Few 64-row tiles (mid-size M, moderate N): split K over workgroups so that every CU streams weights,
     // fp32 partials in the workspace, one summing pass.

@@ -244,6 +244,21 @@ def test_w4a8_mid_m_fused_tiles(dev, M, N, K):
     assert_close_scaled(c, g.w4a8_gemm(a, a_s, wq, s, s4, z4), what="w4a8 fused tiles")
 
 
+@pytest.mark.parametrize("sdt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 4096), (200, 520, 3200), (257, 1032, 8192)])
+def test_int8_mid_m_scale_dtypes(dev, M, N, K, sdt):
+    """Mid-size M, int8 blocks: the kernel stages 16-bit activation scales as they are; every scale dtype gives the
+    oracle's result on the same (rounded) scales."""
+    announce("int8 mid-M scale dtype", M, N, K, sdt)
+    torch.manual_seed(M + K)
+    a, a_s = q.act_quant_int8(torch.randn(M, K).bfloat16() * 3)
+    b, b_s = q.weight_quant_int8(torch.randn(N, K) * 0.02)
+    a_s, b_s = a_s.to(sdt), b_s.to(sdt)
+    with default_dtype(torch.float32):
+        c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+    assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="int8 mid-M scales " + str(sdt))
+
+
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("M,N,K,out", [(128, 1024, 4096, torch.bfloat16), (200, 520, 3200, torch.float32),
                                        (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16),
