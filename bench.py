@@ -566,7 +566,10 @@ def main():
     if args.workload == "copy_256m":
         op, M, N, K = "copy", 0, 0, 0
         case = CopyCase(args.workload, 256 << 20)
-    elif args.workload in MOE_WORKLOADS:
+    elif args.workload in MOE_WORKLOADS or re.fullmatch(r"moe_mixtral_(fp8|int8)_t(\d+)", args.workload):
+        if args.workload not in MOE_WORKLOADS:          # any other token count of the registered expert layer
+            mm = re.fullmatch(r"moe_mixtral_(fp8|int8)_t(\d+)", args.workload)
+            MOE_WORKLOADS[args.workload] = (mm.group(1), int(mm.group(2)))
         case = MoECase(args.workload, *MOE_WORKLOADS[args.workload])
         op, M, N, K = "moe", case.M, case.N, case.K
     else:
