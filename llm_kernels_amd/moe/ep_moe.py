@@ -2,11 +2,15 @@
 
 The call order, buffer shapes and dtypes are those of EPMoE.forward in the reference
 (moe/sglang_moe_all_gather_all_reduce.py:267-446) with all experts local; the final all-reduce across
-ranks is outside this path.
+ranks is outside this path.  `ep_moe_forward` is that forward as a function of (tokens, routing, weights);
+`EPMoE` is the reference's module around it (gate + expert weights + scales, same attribute names), and
+`MoEGate` the DeepSeek-V3 router it owns (moe/all2all_moe.py:31-118).
 """
+import math
 from typing import List, Optional
 
 import torch
+from torch import nn
 
 from .group_gemm_kernel import (grouped_gemm_triton, post_reorder, pre_reorder, run_moe_ep_preproess,
                                 silu_and_mul, gelu_and_mul, pre_reorder_quant, act_and_mul_quant)
@@ -86,3 +90,113 @@ def ep_moe_forward(hidden_states: torch.Tensor, topk_ids: torch.Tensor, topk_wei
     output = torch.empty((T, H), device=dev, dtype=dt)
     post_reorder(down_output, output, src2dst, topk_ids, topk_weights, start_expert_id, end_expert_id, top_k, H)
     return output
+
+
+class MoEGate(nn.Module):
+    """Sigmoid scores, group-limited top-k ("noaux_tc"), as moe/all2all_moe.py:60-118.
+
+    Per token: scores = sigmoid(x W^T) in fp32; the experts are split into n_group groups, a group is ranked by
+    the sum of its two largest (score + e_score_correction_bias), only the experts of the best topk_group groups
+    keep their biased score (the others count as 0.0), the top_k of those are the token's experts; their weights
+    are the unbiased scores, normalised to sum 1 when norm_topk_prob (denominator + 1e-20), times
+    routed_scaling_factor.  Plain torch on whatever device the module lives on: routing is not part of the GEMM path.
+    """
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.top_k = config.num_experts_per_tok
+        self.n_routed_experts = config.n_routed_experts
+        self.routed_scaling_factor = config.routed_scaling_factor
+        self.scoring_func = config.scoring_func
+        self.topk_method = config.topk_method
+        self.n_group = config.n_group
+        self.topk_group = config.topk_group
+        self.norm_topk_prob = config.norm_topk_prob
+        self.gating_dim = config.hidden_size
+        self.weight = nn.Parameter(torch.empty((self.n_routed_experts, self.gating_dim)))
+        if self.topk_method == "noaux_tc":
+            self.e_score_correction_bias = nn.Parameter(torch.zeros((self.n_routed_experts,)))
+        nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+
+    def forward(self, hidden_states):
+        if self.scoring_func != "sigmoid":
+            raise NotImplementedError(f"insupportable scoring function for MoE gating: {self.scoring_func}")
+        if self.topk_method != "noaux_tc":
+            raise NotImplementedError(f"insupportable TopK function for MoE gating: {self.topk_method}")
+        assert not self.training
+        x = hidden_states.reshape(-1, hidden_states.shape[-1])
+        n, E, G = x.shape[0], self.n_routed_experts, self.n_group
+        scores = torch.sigmoid(x.float() @ self.weight.float().t())
+        biased = scores + self.e_score_correction_bias.float()[None, :]
+        per_group = biased.view(n, G, E // G)
+        group_rank = per_group.topk(2, dim=-1).values.sum(dim=-1)                  # [n, G]
+        keep = torch.zeros_like(group_rank, dtype=torch.bool)
+        keep.scatter_(1, group_rank.topk(self.topk_group, dim=-1, sorted=False).indices, True)
+        candidates = torch.where(keep[:, :, None], per_group, torch.zeros((), device=x.device)).reshape(n, E)
+        topk_idx = candidates.topk(self.top_k, dim=-1, sorted=False).indices
+        topk_weight = scores.gather(1, topk_idx)
+        if self.top_k > 1 and self.norm_topk_prob:
+            topk_weight = topk_weight / (topk_weight.sum(dim=-1, keepdim=True) + 1e-20)
+        return topk_idx, topk_weight * self.routed_scaling_factor
+
+
+class EPMoE(nn.Module):
+    """The reference's module (moe/sglang_moe_all_gather_all_reduce.py:162-446): a MoEGate, the stacked expert
+    weights w13_weight [E, 2I, H] / w2_weight [E, H, I] in config.w_dtype (or the default dtype when
+    config.quantize_method is None) and, with block quantisation, their fp16 scales w13_weight_scale
+    [E, 2 ceil(I / bn), ceil(H / bk)] / w2_weight_scale [E, ceil(H / bn), ceil(I / bk)], all initialised to ones
+    as there (the weight-init recipe of sglang_moe_all_gather_all_reduce_test.py:29-69 fills them).
+
+    forward(hidden_states [B, S, H]) -> [B, S, H].  One GPU holds every expert here: config.ep_size must be 1, the
+    reference's closing all-reduce over the expert-parallel ranks (:442-443) has nothing to add and is not issued.
+    """
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.tp_size = config.ep_size or 1
+        if self.tp_size != 1:
+            raise NotImplementedError("EPMoE: this build runs every expert on one GPU (config.ep_size must be 1)")
+        self.tp_rank = 0
+        self.num_experts = config.n_routed_experts
+        self.num_experts_per_partition = self.num_experts
+        self.start_expert_id = 0
+        self.end_expert_id = self.num_experts - 1
+        self.top_k = config.num_experts_per_tok
+        self.hidden_size = config.hidden_size
+        self.intermediate_size = config.moe_intermediate_size
+        self.activation = config.hidden_act
+        self.gate = MoEGate(config)
+        quantised = config.quantize_method is not None
+        params_dtype = config.w_dtype if quantised else torch.get_default_dtype()
+        E, I, H = self.num_experts, self.intermediate_size, self.hidden_size
+
+        def ones(*shape, dtype):
+            # (torch.ones has no fp8 kernel: build in fp32 and cast)
+            return nn.Parameter(torch.ones(*shape, dtype=torch.float32).to(dtype), requires_grad=False)
+
+        self.w13_weight = ones(E, 2 * I, H, dtype=params_dtype)
+        self.w2_weight = ones(E, H, I, dtype=params_dtype)
+        self.w13_input_scale = None
+        self.w2_input_scale = None
+        self.use_fp8_w8a8 = False
+        self.use_block_quant = config.use_block_quant
+        if config.use_block_quant and quantised:
+            bn, bk = config.w_quant_block_size
+            self.w13_weight_scale = ones(E, 2 * ((I + bn - 1) // bn), (H + bk - 1) // bk, dtype=torch.float16)
+            self.w2_weight_scale = ones(E, (H + bn - 1) // bn, (I + bk - 1) // bk, dtype=torch.float16)
+            self.block_shape = list(config.w_quant_block_size)
+        else:
+            self.w13_weight_scale = None
+            self.w2_weight_scale = None
+            self.block_shape = None
+
+    def forward(self, hidden_states: torch.Tensor, router_logits: Optional[torch.Tensor] = None):
+        batch_size, seq_len, _ = hidden_states.shape
+        topk_ids, topk_weights = self.gate(hidden_states)
+        out = ep_moe_forward(hidden_states.reshape(-1, self.hidden_size), topk_ids.reshape(-1, self.top_k),
+                             topk_weights.reshape(-1, self.top_k), self.w13_weight, self.w2_weight,
+                             self.w13_weight_scale, self.w2_weight_scale, self.block_shape, self.activation,
+                             self.start_expert_id, self.end_expert_id)
+        return out.reshape(batch_size, seq_len, self.hidden_size)

@@ -138,3 +138,33 @@ def ep_moe_forward(x, topk_ids, topk_w, w13, w13_s, w2, w2_s, act_quant, dtype=t
     dq, ds = act_quant(di)
     do = grouped_gemm(dq, w2, seg, widx, ds, w2_s).to(dtype)
     return post_reorder(do, src2dst, topk_ids, topk_w, 0, E - 1, topk)
+
+
+def deepseek_gate(x, weight, bias, top_k, n_group, topk_group, norm_topk_prob=True, routed_scaling_factor=1.0):
+    """The router EPMoE owns (MoEGate.forward, moe/all2all_moe.py:60-118), token by token in float64 loops.
+
+    Returns (list of expert-id sets, list of {expert: weight}) so that the order inside a token's top-k, which
+    the reference leaves open (topk(..., sorted=False)), does not enter a comparison."""
+    import math
+    xs = x.reshape(-1, x.shape[-1]).double()
+    E = weight.shape[0]
+    per = E // n_group
+    ids_out, w_out = [], []
+    for t in range(xs.shape[0]):
+        score = [1.0 / (1.0 + math.exp(-float(xs[t] @ weight[e].double()))) for e in range(E)]     # :64-68
+        biased = [score[e] + float(bias[e]) for e in range(E)]                                       # :77
+        rank = []
+        for gi in range(n_group):                                                                    # :80-82
+            best = sorted(biased[gi * per:(gi + 1) * per], reverse=True)[:2]
+            rank.append(sum(best))
+        groups = sorted(range(n_group), key=lambda gi: -rank[gi])[:topk_group]                       # :84-85
+        cand = [biased[e] if e // per in groups else 0.0 for e in range(E)]                          # :88-101
+        chosen = sorted(range(E), key=lambda e: -cand[e])[:top_k]                                    # :104-106
+        w = {e: score[e] for e in chosen}                                                            # :107 (unbiased)
+        if top_k > 1 and norm_topk_prob:                                                             # :114-116
+            den = sum(w.values()) + 1e-20
+            w = {e: v / den for e, v in w.items()}
+        w = {e: v * routed_scaling_factor for e, v in w.items()}                                     # :117
+        ids_out.append(set(chosen))
+        w_out.append(w)
+    return ids_out, w_out

@@ -28,6 +28,8 @@ IMPORTS = textwrap.dedent("""
     from moe.group_gemm_kernel import (run_moe_ep_preproess, grouped_gemm_triton, pre_reorder_triton_kernel,
                                        silu_and_mul_triton_kernel, gelu_and_mul_triton_kernel, post_reorder_triton_kernel)
     from moe.ep_moe import ep_moe_forward
+    from moe.sglang_moe_all_gather_all_reduce import EPMoE
+    from moe.config import Config
     from quant_communication.quant_utils import int8_quant, int8_dequant, fp8_quant, fp8_dequant
     from fast_dequant.fast_dtype_convert import uint4_to_fp16, uint8_to_fp16, uint8_to_bf16, mma_fp16
     import quantization.fp8_kernel as m

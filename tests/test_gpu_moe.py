@@ -4,7 +4,8 @@ import torch
 
 from oracle import moe_ref as m, quant_ref as q, gemm_ref as g
 from llm_kernels_amd.moe import group_gemm_kernel as gk
-from llm_kernels_amd.moe.ep_moe import ep_moe_forward, softmax_topk_router
+from llm_kernels_amd.moe.ep_moe import ep_moe_forward, softmax_topk_router, EPMoE
+from llm_kernels_amd.moe.config import Config
 from llm_kernels_amd.quantization import int8_kernel, fp8_kernel
 from helpers import announce, assert_close_scaled
 
@@ -290,6 +291,61 @@ def test_ep_moe_forward_small(dev, kind):
     dense = m.dense_moe_forward(x, ids, w, w13, w2)
     cos = torch.nn.functional.cosine_similarity(out.float().cpu().flatten(), dense.float().flatten(), dim=0)
     assert cos > 0.99
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8", "fp16"])
+def test_epmoe_module(dev, kind):
+    """The module as the reference's own test drives it (sglang_moe_all_gather_all_reduce_test.py:29-110): gate weight
+    ~ N(0, 0.1), expert weights ~ N(0, 0.01) quantised per expert in 128 x 128 blocks, fp16 tokens [2, 24, H];
+    forward against the oracle's forward on the module's own routing."""
+    announce("EPMoE module", kind)
+    torch.manual_seed(42)
+    dt = torch.float16
+    qm = {"int8": "blockwise_w8a8_int8_gemm", "fp8": "blockwise_w8a8_fp8_gemm", "fp16": None}[kind]
+    wdt = {"int8": torch.int8, "fp8": torch.float8_e4m3fn, "fp16": dt}[kind]
+    cfg = Config(hidden_size=256, moe_intermediate_size=384, n_routed_experts=16, num_experts_per_tok=4, n_group=4,
+                 topk_group=2, quantize_method=qm, w_dtype=wdt, a_dtype=wdt)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(dt)
+    try:
+        mod = EPMoE(cfg).eval()
+    finally:
+        torch.set_default_dtype(old)
+    E, I, H = 16, 384, 256
+    w13 = torch.randn(E, 2 * I, H) * 0.01
+    w2 = torch.randn(E, H, I) * 0.01
+    with torch.no_grad():
+        mod.gate.weight.normal_(0.0, 0.1)
+        if kind == "fp16":
+            mod.w13_weight.copy_(w13)
+            mod.w2_weight.copy_(w2)
+        else:
+            wq = q.weight_quant_int8 if kind == "int8" else q.weight_quant_fp8
+            for e in range(E):
+                a, s_a = wq(w13[e])
+                b, s_b = wq(w2[e])
+                mod.w13_weight[e] = a
+                mod.w13_weight_scale[e] = s_a
+                mod.w2_weight[e] = b
+                mod.w2_weight_scale[e] = s_b
+    x = torch.randn(2, 24, H).to(dt)
+    mod = mod.to(dev)
+    with torch.no_grad():
+        out = mod(x.to(dev))
+        ids, w = mod.gate(x.to(dev))
+    assert out.shape == (2, 24, H) and out.dtype == dt
+    ids, w = ids.cpu(), w.cpu()
+    # the routing itself: the token's expert set against the loop oracle (scores are far from ties at this size)
+    oids, _ = m.deepseek_gate(x, mod.gate.weight.detach().cpu(), mod.gate.e_score_correction_bias.detach().cpu(), 4, 4, 2, True, 2.5)
+    assert sum(set(ids[t].tolist()) == oids[t] for t in range(48)) >= 47
+    if kind == "fp16":
+        dense = m.dense_moe_forward(x.reshape(-1, H), ids, w, mod.w13_weight.detach().cpu(), mod.w2_weight.detach().cpu())
+        assert_close_scaled(out.reshape(-1, H), dense, rtol=3e-2, atol=3e-2, what="EPMoE fp16 vs dense")
+        return
+    aq = q.act_quant_int8 if kind == "int8" else q.act_quant_fp8
+    ref = m.ep_moe_forward(x.reshape(-1, H), ids, w, mod.w13_weight.detach().cpu(), mod.w13_weight_scale.detach().cpu(),
+                           mod.w2_weight.detach().cpu(), mod.w2_weight_scale.detach().cpu(), aq, dtype=dt)
+    assert_close_scaled(out.reshape(-1, H), ref, rtol=5e-2, atol=5e-2, what="EPMoE " + kind)
 
 
 def test_router(dev):
