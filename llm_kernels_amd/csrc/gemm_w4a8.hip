@@ -6,10 +6,26 @@ using namespace llmk;
 
 namespace {
 
+// 16-bit block scales that the same launch widens to fp32 for the int8 GEMM behind it (blocks past the expansion's):
+// saves that GEMM a launch of its own for the activation scales
+struct W4A8Widen {
+    const void* a_s; const void* b_s;
+    float* a_s32; float* b_s32;
+    int64_t n_a, n_b;
+    int s_dtype;
+    unsigned first_block;       // 0: nothing to widen
+};
+
 // packed [N/8, K] int32 -> b8 [N, K] int8 with b8 = int8(int8(q - z4) * s4) (two's-complement wrap)
 __global__ void w4a8_expand_kernel(const int32_t* __restrict__ packed, const int8_t* __restrict__ s4,
                                    const int8_t* __restrict__ z4, int8_t* __restrict__ out,
-                                   int64_t N, int64_t K, int group) {
+                                   int64_t N, int64_t K, int group, W4A8Widen wd) {
+    if (wd.first_block && blockIdx.x >= wd.first_block) {
+        const int64_t i = (int64_t)(blockIdx.x - wd.first_block) * blockDim.x + threadIdx.x;
+        if (i < wd.n_a) wd.a_s32[i] = ld_scale(wd.a_s, i, wd.s_dtype);
+        else if (i < wd.n_a + wd.n_b) wd.b_s32[i - wd.n_a] = ld_scale(wd.b_s, i - wd.n_a, wd.s_dtype);
+        return;
+    }
     // one thread: 8 rows x 4 consecutive k
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t kq = K / 4;
@@ -436,6 +452,13 @@ struct W4A8Plan {
     int64_t nz;           // K ranges of the decode kernel
     int64_t bytes;        // scratch the chosen path uses
 };
+// scratch layout of the two-pass path: int8 copy of W | fp32 activation scales | fp32 weight scales | the int8 GEMM's own
+inline int64_t w4a8_two_pass_scales_off(int64_t N, int64_t K) { return (N * K + 255) & ~(int64_t)255; }
+inline int64_t w4a8_a_s32_bytes(int64_t M, int64_t K) { return (M * (K / 128) * 4 + 255) & ~(int64_t)255; }
+inline int64_t w4a8_widened_bytes(int64_t M, int64_t N, int64_t K) {
+    return w4a8_a_s32_bytes(M, K) + ((((N + 127) / 128) * (K / 128) * 4 + 255) & ~(int64_t)255);
+}
+
 W4A8Plan w4a8_plan(int64_t M, int64_t N, int64_t K, int group_int4) {
     W4A8Plan pl{false, false, 1, 0};
     if (M <= 0 || N <= 0 || K <= 0) return pl;
@@ -463,7 +486,7 @@ W4A8Plan w4a8_plan(int64_t M, int64_t N, int64_t K, int group_int4) {
                K <= 0x7fffffff && dma_eligible(q);
     if (pl.stream) pl.bytes = pl.nz > 1 ? pl.nz * M * N * 4 : 0;
     else if (pl.tiles) pl.bytes = llmk_gemm_workspace_bytes(M, N, K);      // fp32 activation scales + split-K partial sums
-    else pl.bytes = ((N * K + 15) & ~(int64_t)15) + llmk_gemm_workspace_bytes(M, N, K);
+    else pl.bytes = w4a8_two_pass_scales_off(N, K) + w4a8_widened_bytes(M, N, K) + llmk_gemm_workspace_bytes(M, N, K);
     return pl;
 }
 
@@ -543,14 +566,32 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
         return launch_w4a8_tiles(p, workspace, workspace_bytes, (hipStream_t)stream);
     }
     if (!workspace || workspace_bytes < N * K) LLMK_FAIL(LLMK_ERR_ARG, "gemm_w4a8: workspace of N*K=%lld bytes required", (long long)(N * K));
+    // 16-bit block scales are widened by spare blocks of the expansion launch when the scratch has room for them
+    W4A8Widen wd{};
+    int64_t used = (N * K + 15) & ~(int64_t)15;
+    const int64_t soff = w4a8_two_pass_scales_off(N, K);
+    if ((s_dtype == LLMK_F16 || s_dtype == LLMK_BF16) && K > 0 && !((uintptr_t)workspace & 255) &&
+        workspace_bytes >= soff + w4a8_widened_bytes(M, N, K)) {
+        wd.a_s = a_s; wd.b_s = b_s; wd.s_dtype = s_dtype;
+        wd.n_a = M * (K / 128); wd.n_b = ((N + 127) / 128) * (K / 128);
+        wd.a_s32 = (float*)((uint8_t*)workspace + soff);
+        wd.b_s32 = (float*)((uint8_t*)workspace + soff + w4a8_a_s32_bytes(M, K));
+        used = soff + w4a8_widened_bytes(M, N, K);
+    }
     if (K > 0) {
-        dim3 grid((unsigned)cdiv64((N / 8) * (K / 4), 256)), blk(256);
-        w4a8_expand_kernel<<<grid, blk, 0, (hipStream_t)stream>>>(b_packed, b_s4, b_z4, (int8_t*)workspace, N, K, group_int4);
+        const unsigned expand_blocks = (unsigned)cdiv64((N / 8) * (K / 4), 256);
+        unsigned blocks = expand_blocks;
+        if (wd.a_s32) {
+            wd.first_block = expand_blocks;
+            blocks += (unsigned)cdiv64(wd.n_a + wd.n_b, 256);
+        }
+        w4a8_expand_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(b_packed, b_s4, b_z4, (int8_t*)workspace, N, K, group_int4, wd);
         LLMK_CHECK_LAUNCH("gemm_w4a8(expand)");
     }
     // what is left of the workspace behind the expanded weights (16-byte aligned) serves the int8 GEMM
-    const int64_t used = (N * K + 15) & ~(int64_t)15;
     void* rest = workspace_bytes > used ? (void*)((uint8_t*)workspace + used) : nullptr;
     const int64_t rest_bytes = rest ? workspace_bytes - used : 0;
+    if (wd.a_s32)
+        return llmk_gemm_i8_block(a, wd.a_s32, (const int8_t*)workspace, wd.b_s32, LLMK_F32, c, c_dtype, M, N, K, rest, rest_bytes, stream);
     return llmk_gemm_i8_block(a, a_s, (const int8_t*)workspace, b_s, s_dtype, c, c_dtype, M, N, K, rest, rest_bytes, stream);
 }
