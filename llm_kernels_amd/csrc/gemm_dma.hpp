@@ -210,7 +210,9 @@ __device__ __forceinline__ void rowcol_epilogue8(const DirectArgs& p, v4f& a, v4
 }
 
 // MI = 16-row tiles per wave along M (4, 2 or 1): the workgroup tile is 64*MI rows x 128 columns.
-template <int KIND, bool GROUPED, int MI>
+// AS16: the activation scales are 16-bit (fp16 or bf16 by p.s_dtype) and are staged as they are, one zero-extended
+// element per dword slot of the scale column (global_load_lds_ushort), instead of being widened by a pass of their own.
+template <int KIND, bool GROUPED, int MI, bool AS16 = false>
 __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     constexpr int BM = 64 * MI;              // tile rows
     constexpr int WR = 16 * MI;              // rows per wave
@@ -296,7 +298,11 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const int col = (R & 64) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
-    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
+    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, BM - 1), m_end - 1) * (uint32_t)KT_all * (AS16 ? 2u : 4u);
+    auto dma_scale = [&](uint32_t lds_addr, int kt_abs) {
+        if constexpr (AS16) dma2(lds_addr, soff, (const uint8_t*)p.a_s + (int64_t)kt_abs * 2);
+        else dma4(lds_addr, soff, (const uint8_t*)p.a_s + (int64_t)kt_abs * 4);
+    };
     // K_W4NK: thread t expands quarter (t & 3) of LDS row t >> 2 (16 weights of a 64-element K step)
     uint32_t w4_off = 0, w4_soff = 0, w4_lds = 0;
     if constexpr (W4M) {
@@ -339,12 +345,11 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
     auto issue_b_half = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
         const uint8_t* gb = bbase + (int64_t)(kt0 + kt) * 128;
-        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
         if constexpr (!W4) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) dma16(st + D_A + (uint32_t)(wave * 2 + i) * 1024u, boff[i], gb);
         }
-        if constexpr (SCALED) dma4(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+        if constexpr (SCALED) dma_scale(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, kt0 + kt);
     };
     auto issue_a_half = [&](int kt) {
         const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
@@ -356,14 +361,13 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         const uint32_t st = lds_base + (uint32_t)(kt % D_NSTAGE) * D_STAGE;
         const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
         const uint8_t* gb = bbase + (int64_t)(kt0 + kt) * 128;
-        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
 #pragma unroll
         for (int i = 0; i < MI; ++i) dma16(st + (uint32_t)(wave * MI + i) * 1024u, aoff[i], ga);
         if constexpr (!W4) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) dma16(st + D_A + (uint32_t)(wave * 2 + i) * 1024u, boff[i], gb);
         }
-        if constexpr (SCALED) dma4(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+        if constexpr (SCALED) dma_scale(st + D_A + D_B + (uint32_t)(wave & 3) * 256u, kt0 + kt);
     };
     // K_W4NK: packed words and group scale of K step kt -> registers (requested before the activation loads
     // of the same step, so that waiting for them leaves exactly those MI loads in flight) ...
@@ -526,7 +530,14 @@ __global__ __launch_bounds__(D_THREADS) void gemm_dma_kernel(DirectArgs p) {
         if constexpr (SCALED) {
             const float bs = bsl[kt];
 #pragma unroll
-            for (int i = 0; i < MI; ++i) sa[i] = Ss[i * 16] * bs;
+            for (int i = 0; i < MI; ++i) {
+                if constexpr (AS16) {
+                    const unsigned raw = ((const unsigned*)Ss)[i * 16];
+                    sa[i] = (p.s_dtype == LLMK_F16 ? f16_to_f32((unsigned short)raw) : bf16_to_f32((unsigned short)raw)) * bs;
+                } else {
+                    sa[i] = Ss[i * 16] * bs;
+                }
+            }
         }
     };
     // The weight fragment is the MFMA row operand and the activation fragment the column operand, i.e.
@@ -771,11 +782,11 @@ inline int w4a8_max_mi(const DirectArgs& p) {
     return d_lds(2) + tab <= D_LDS_MAX ? 2 : (d_lds(1) + tab <= D_LDS_MAX ? 1 : 0);
 }
 
-// a_s must be fp32 here (p.a_s); p.s_dtype describes b_s only.
-template <int KIND, bool GROUPED, int MI>
+// p.a_s: fp32, or with AS16 the 16-bit scales of dtype p.s_dtype as the caller passed them; p.s_dtype describes b_s.
+template <int KIND, bool GROUPED, int MI, bool AS16 = false>
 int launch_dma_mi(const DirectArgs& p, hipStream_t stream, const char* name) {
     static std::atomic<uint64_t> configured{0};
-    auto kern = gemm_dma_kernel<KIND, GROUPED, MI>;
+    auto kern = gemm_dma_kernel<KIND, GROUPED, MI, AS16>;
     constexpr int BM = 64 * MI;
     const int tiles_m = GROUPED ? grouped_row_tiles(p.M, p.E, BM) : (p.M + BM - 1) / BM;
     const bool split = !GROUPED && p.ksplit > 1 && p.partial;

@@ -505,22 +505,14 @@ int launch_w4a8_tiles(DirectArgs p, void* workspace, int64_t workspace_bytes, hi
             return pl.mt == 4 ? launch_mid<K_W4A8, 4>(p, stream, name) : launch_mid<K_W4A8, 2>(p, stream, name);
         }
     }
-    // the 128-column kernels stream 4-byte scale elements: 16-bit scales are widened into the workspace first
-    int64_t used = 0;
-    if (p.s_dtype != LLMK_F32) {
-        const int64_t n = (int64_t)p.M * (p.K >> 7);
-        const unsigned blocks = (unsigned)cdiv64(n, 256);
-        if (p.s_dtype == LLMK_F16) scales_to_f32_kernel<LLMK_F16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
-        else scales_to_f32_kernel<LLMK_BF16><<<blocks, 256, 0, stream>>>(p.a_s, (float*)workspace, n);
-        LLMK_CHECK_LAUNCH(name);
-        p.a_s = workspace;
-        used = (n * 4 + 255) & ~(int64_t)255;
-    }
+    // the 128-column kernels stage 16-bit scales as they are, too
+    const int64_t used = 0;
     const int z = splitk_factor(p.M, p.N, p.K);
     if (z > 1 && workspace_bytes - used >= (int64_t)z * p.M * p.N * 4) {
         p.partial = (float*)((uint8_t*)workspace + used);
         p.ksplit = z;
     }
+    if (p.s_dtype != LLMK_F32) return launch_dma<K_W4A8, false, true>(p, stream, name);
     return launch_dma<K_W4A8, false>(p, stream, name);
 }
 }  // namespace
@@ -555,8 +547,8 @@ extern "C" int llmk_gemm_w4a8(const int8_t* a, const void* a_s, const int32_t* b
 #undef LLMK_W4A8_MT
         LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: s_dtype %d", s_dtype);
     }
-    if (pl.tiles && !(((uintptr_t)a | (uintptr_t)b_packed | (uintptr_t)workspace) & 15) && workspace &&
-        workspace_bytes >= ((M * (K / 128) * 4 + 255) & ~(int64_t)255)) {
+    if (pl.tiles && !(((uintptr_t)a | (uintptr_t)b_packed | (uintptr_t)workspace) & 15)) {
+        if (!workspace) workspace_bytes = 0;                // no scratch: no K split, everything else as with it
         if (s_dtype != LLMK_F32 && s_dtype != LLMK_F16 && s_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: s_dtype %d", s_dtype);
         if (c_dtype != LLMK_F32 && c_dtype != LLMK_F16 && c_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "gemm_w4a8: c_dtype %d", c_dtype);
         DirectArgs p{};

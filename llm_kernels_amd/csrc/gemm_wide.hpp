@@ -153,6 +153,7 @@ constexpr int W_TAIL_ITEMS = LLMK_CUS;          // upper bound of ntail * z
 
 template <int KIND, bool GROUPED, int R = 8>
 __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
+    constexpr bool AS16 = false;             // 16-bit activation scales are widened before this kernel, see launch_big
     static_assert(R == 8 || R == 4, "tile rows per wave");
     constexpr int W_BM = w_bm(R), W_A = W_BM * 128, W_STAGE = w_stage(R);
     constexpr int AL = R / 2;                    // activation loads per thread and stage
@@ -235,7 +236,12 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const int col = (row & 192) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
         boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
     }
-    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT_all * 4u;
+    const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT_all * (AS16 ? 2u : 4u);
+    // (AS16: 16-bit activation scales staged as they are, see gemm_dma_kernel)
+    auto dma_scale = [&](uint32_t lds_addr, int kt_abs) {
+        if constexpr (AS16) dma2(lds_addr, soff, (const uint8_t*)p.a_s + (int64_t)kt_abs * 2);
+        else dma4(lds_addr, soff, (const uint8_t*)p.a_s + (int64_t)kt_abs * 4);
+    };
 
     // ---- 4-bit weights: a thread owns the same piece of the 128-column half h = 0, 1 of the tile as in the
     // 128-column tile kernel (gemm_dma.hpp): per K step and half one 8-byte load of packed weights and one load
@@ -304,7 +310,6 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
         const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
         const uint8_t* gb = bbase + (int64_t)(kt0 + kt) * 128;
-        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
         if constexpr (W4) w4_request(kt);          // in front of the activation loads: see w4_expand
 #pragma unroll
         for (int i = 0; i < AL; ++i) dma16(st + (uint32_t)(wave * AL + i) * 1024u, aoff[i], ga);
@@ -312,7 +317,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) dma16(st + W_A + (uint32_t)(wave * 4 + i) * 1024u, boff[i], gb);
         }
-        if constexpr (SCALED) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+        if constexpr (SCALED) dma_scale(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, kt0 + kt);
     };
 
     // The loads of a stage inside the loop, a quarter at a time (part 0..3): the weight rows behind the
@@ -320,9 +325,8 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     auto issue_part = [&](int kt, int part) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
         const uint8_t* ga = p.a + (int64_t)(kt0 + kt) * 128;
-        const uint8_t* gs = (const uint8_t*)p.a_s + (int64_t)(kt0 + kt) * 4;
         if (part < AL) dma16(st + (uint32_t)(wave * AL + part) * 1024u, aoff[part < AL ? part : 0], ga);
-        if constexpr (SCALED) if (part == 3) dma4(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, soff, gs);
+        if constexpr (SCALED) if (part == 3) dma_scale(st + W_A + W_B + (uint32_t)(wave & 3) * 256u, kt0 + kt);
     };
     auto issue_b_part = [&](int kt, int part) {
         const uint32_t st = lds_base + (uint32_t)(kt & 1) * W_STAGE;
@@ -422,7 +426,14 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
             const float* Ss = (const float*)(lds + (kt & 1) * W_STAGE + W_A + W_B) + wm * 16 * R + r;
             const float bs = bsl[(wn >> 1) * D_MAX_KT + kt];
 #pragma unroll
-            for (int i = 0; i < NR; ++i) sa[i] = Ss[i * 16] * bs;
+            for (int i = 0; i < NR; ++i) {
+                if constexpr (AS16) {
+                    const unsigned raw = ((const unsigned*)Ss)[i * 16];
+                    sa[i] = (p.s_dtype == LLMK_F16 ? f16_to_f32((unsigned short)raw) : bf16_to_f32((unsigned short)raw)) * bs;
+                } else {
+                    sa[i] = Ss[i * 16] * bs;
+                }
+            }
         }
 #pragma unroll
         for (int i = 0; i < R; ++i) {
@@ -631,9 +642,9 @@ inline bool mid_m_prefers_tiles(int64_t M, int64_t N, int64_t K) {
 // Tile shape by estimated time: rounds of 256 workgroups times the measured cost of one round of each tile
 // shape (60 / 36 / 43 / 26 / 16 microseconds for 256 x 256, 128 x 256, 256 x 128, 128 x 128 and 64 x 128 at K = 4096
 // for fp8; the ratios hold for the other kinds and K).  Ties go to the larger tile (less operand re-reading).  Segments of a grouped GEMM are judged by their average length.
+// which tile shape the estimate picks: 8 / 9 = the 256 x 256 / 128 x 256 tile of gemm_wide_kernel, 4 / 2 / 1 = MI of gemm_dma_kernel
 template <int KIND, bool GROUPED>
-int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* ws = nullptr, int64_t ws_bytes = 0) {
-    if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
+int dma_tile_choice(const DirectArgs& p) {
     // 4-bit weights: the row-packed layout, dense launches (the Marlin scatter of 2-byte pieces measured 4-9 % slower
     // inside the 256-column kernel than the dequantisation pass at every M > 512)
     constexpr bool HAS_WIDE = KIND != K_W4MARLIN && KIND != K_W4A8 && !(GROUPED && KIND == K_W4NK);
@@ -651,19 +662,37 @@ int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* 
             // (a tie goes to the 128-row tile for block-scaled int8, whose per-step conversions leave the tall
             // tile less of its advantage: grouped Mixtral down projection -3 %; +1 % for fp8)
             const double t_half = 36.0 * rounds(128, 256);
-            if (t_half < t_wide || (KIND == K_I8_BLOCK && GROUPED && t_half == t_wide)) return launch_wide<KIND, GROUPED, 4>(p, stream, name, ws, ws_bytes);
-            return launch_wide<KIND, GROUPED>(p, stream, name, ws, ws_bytes);
+            if (t_half < t_wide || (KIND == K_I8_BLOCK && GROUPED && t_half == t_wide)) return 9;
+            return 8;
         }
         const double t_half = 36.0 * rounds(128, 256);
-        if (t_half < t4 && t_half <= t2 && t_half <= t1) return launch_wide<KIND, GROUPED, 4>(p, stream, name, ws, ws_bytes);
+        if (t_half < t4 && t_half <= t2 && t_half <= t1) return 9;
     }
     int max_mi = 4;
     if constexpr (KIND == K_W4A8) max_mi = w4a8_max_mi(p);       // the table of zero points and scales must fit behind the stages
     if constexpr (KIND != K_W4A8) {
-        if (t4 <= t2 && t4 <= t1 && max_mi >= 4) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
+        if (t4 <= t2 && t4 <= t1 && max_mi >= 4) return 4;
     }
-    if (t2 <= t1 && max_mi >= 2) return launch_dma_mi<KIND, GROUPED, 2>(p, stream, name);
-    return launch_dma_mi<KIND, GROUPED, 1>(p, stream, name);
+    if (t2 <= t1 && max_mi >= 2) return 2;
+    return 1;
+}
+
+// AS16 (16-bit activation scales staged as they are): the 64- and 128-row tiles of gemm_dma_kernel only, see launch_big
+template <int KIND, bool GROUPED, bool AS16 = false>
+int launch_dma(const DirectArgs& p, hipStream_t stream, const char* name, void* ws = nullptr, int64_t ws_bytes = 0) {
+    if (!GROUPED && p.ksplit > 1) return launch_dma_mi<KIND, GROUPED, 1, AS16>(p, stream, name);
+    const int choice = dma_tile_choice<KIND, GROUPED>(p);
+    if constexpr (!AS16) {
+        if constexpr (KIND != K_W4MARLIN && KIND != K_W4A8 && !(GROUPED && KIND == K_W4NK)) {
+            if (choice == 9) return launch_wide<KIND, GROUPED, 4>(p, stream, name, ws, ws_bytes);
+            if (choice == 8) return launch_wide<KIND, GROUPED, 8>(p, stream, name, ws, ws_bytes);
+        }
+        if constexpr (KIND != K_W4A8) {
+            if (choice == 4) return launch_dma_mi<KIND, GROUPED, 4>(p, stream, name);
+        }
+    }
+    if (choice == 2) return launch_dma_mi<KIND, GROUPED, 2, AS16>(p, stream, name);
+    return launch_dma_mi<KIND, GROUPED, 1, AS16>(p, stream, name);
 }
 
 // Dispatch for the compute-bound block-scaled GEMM: direct-to-LDS kernels when eligible (converting
@@ -689,7 +718,20 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
         }
     }
     int64_t used = 0;
-    if (p.s_dtype != LLMK_F32) {
+    // 16-bit activation scales: the int8 kind stages them as they are (AS16 instantiations); fp8 callers pass fp32
+    // scales as a rule, 16-bit ones are widened into the workspace first
+    constexpr bool HAS_AS16 = (KIND == K_I8_BLOCK);
+    // (only where the launch is short: the conversion inside the K loop costs the vector-ALU-bound int8 loop 4-5 %,
+    // the widening pass a launch of 5-7 us: 512 x 4096 x 4096 21.4 -> 17.8 us, 1024 x 4096 x 4096 28.0 -> 26.5 us, but
+    // 4096 x 14336 x 4096 277.6 -> 291 us when forced; the 64- and 128-row tiles are the short launches)
+    bool as16 = false;
+    if constexpr (HAS_AS16) {
+        if (p.s_dtype != LLMK_F32) {
+            const int z = GROUPED ? 1 : splitk_factor(p.M, p.N, p.K);
+            as16 = z > 1 || dma_tile_choice<KIND, GROUPED>(p) <= 2;
+        }
+    }
+    if (p.s_dtype != LLMK_F32 && !as16) {
         const int64_t n = (int64_t)p.M * (p.K >> 7);
         if (!workspace || workspace_bytes < n * 4) return launch_tiled<KIND, GROUPED>(p, stream, name);
         const unsigned blocks = (unsigned)cdiv64(n, 256);
@@ -707,6 +749,12 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
         if (z > 1 && workspace && workspace_bytes - used >= need && !(((uintptr_t)workspace + used) & 15)) {
             p.partial = (float*)((uint8_t*)workspace + used);
             p.ksplit = z;
+        }
+    }
+    if constexpr (HAS_AS16) {
+        if (as16) {
+            if (p.ksplit > 1 || !workspace) return launch_dma<KIND, GROUPED, true>(p, stream, name);
+            return launch_dma<KIND, GROUPED, true>(p, stream, name, workspace, workspace_bytes);                  // split last round
         }
     }
     if (p.ksplit > 1 || !workspace || workspace_bytes <= used) return launch_dma<KIND, GROUPED>(p, stream, name);
