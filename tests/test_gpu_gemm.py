@@ -259,6 +259,43 @@ def test_int8_mid_m_scale_dtypes(dev, M, N, K, sdt):
     assert_close_scaled(c, g.gemm_blockwise(a, a_s, b, b_s), what="int8 mid-M scales " + str(sdt))
 
 
+def _random_mid_shapes(n, seed):
+    import random
+    rnd = random.Random(seed)
+    shapes = []
+    for _ in range(n):
+        M = rnd.choice([65, 66, 96, 127, 128, 129, 160, 255, 256, 257, 300, 384, 511, 512, 513, 700, 1024])
+        N = rnd.choice([8, 24, 64, 72, 128, 136, 520, 1000, 2048, 2056, 4096, 4104, 6144])
+        K = 128 * rnd.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 17, 32, 40, 64])
+        shapes.append((M, N, K))
+    return shapes
+
+
+@pytest.mark.parametrize("M,N,K", _random_mid_shapes(28, 7))
+def test_mid_and_small_tile_kernels_exact_integers(dev, M, N, K):
+    """Random mid-size shapes (ragged row and column tiles, K tails, split K, one or more rounds of tiles) with small
+    integer operands, unit block scales of a random dtype and fp32 output: the block-scaled int8 and fp8 GEMMs and the
+    per-token int8 GEMM must return the exact integer product (every partial sum is below 2^24)."""
+    announce("mid-size exact", M, N, K)
+    torch.manual_seed(M * 7 + N + K)
+    a = torch.randint(-7, 8, (M, K), dtype=torch.int8)
+    b = torch.randint(-7, 8, (N, K), dtype=torch.int8)
+    ref = (a.double() @ b.double().T).long()
+    sdt = [torch.float16, torch.bfloat16, torch.float32][(M + N + K // 128) % 3]
+    a_s = torch.ones(M, K // 128, dtype=sdt)
+    b_s = torch.ones((N + 127) // 128, K // 128, dtype=sdt)
+    with default_dtype(torch.float32):
+        c = int8_kernel.int8_gemm(a.to(dev), a_s.to(dev), b.to(dev), b_s.to(dev))
+        assert torch.equal(c.cpu().long(), ref), "int8 block"
+        # the same integers are exact in e4m3 (|v| <= 7)
+        c8 = fp8_kernel.fp8_gemm(a.float().to(torch.float8_e4m3fn).to(dev), a_s.float().to(dev),
+                                 b.float().to(torch.float8_e4m3fn).to(dev), b_s.float().to(dev))
+        assert torch.equal(c8.cpu().long(), ref), "fp8 block"
+        _, acc = int8_kernel.int8_gemm_per_token(a.to(dev), torch.ones(M).to(dev), b.to(dev), torch.ones(N).to(dev),
+                                                 return_int32=True)
+        assert torch.equal(acc.cpu().long(), ref), "int8 per token"
+
+
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("M,N,K,out", [(128, 1024, 4096, torch.bfloat16), (200, 520, 3200, torch.float32),
                                        (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16),
