@@ -92,7 +92,7 @@ extern "C" int llmk_calib_gemm_fp8_clock(const void* a, const float* a_s, const 
                                          int64_t workspace_bytes, long long* clocks, void* stream) {
     int rc = check_common("calib_gemm_fp8_clock", a, b, M, N, K, c_dtype);
     if (rc) return rc;
-    if (M <= 512 || N == 0 || !c || !a_s || !b_s || !clocks) LLMK_FAIL(LLMK_ERR_ARG, "calib_gemm_fp8_clock: needs M > 512 and every pointer");
+    if (M <= 64 || N == 0 || !c || !a_s || !b_s || !clocks) LLMK_FAIL(LLMK_ERR_ARG, "calib_gemm_fp8_clock: needs M > 512 and every pointer");
     DirectArgs p{};
     p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = c; p.a_s = a_s; p.b_s = b_s; p.clocks = clocks;
     p.c_dtype = c_dtype; p.s_dtype = LLMK_F32; p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1;

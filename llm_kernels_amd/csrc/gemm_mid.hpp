@@ -415,6 +415,275 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     else store_run8<LLMK_F32>(cout, off, sa, sb, nv, vec_ok);
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Producer / consumer form of the same tile for 8- and 16-bit operands.  A cycle count of the kernel above (per wave and
+// phase) showed that it never waits for data: what a step costs is ISSUING its loads.  The CU's vector-memory path takes
+// about 16 cycles per 1 KB instruction (64 bytes per clock, the 110 GB/s per CU), a step of a 64 x 64 tile is 64 such
+// instructions (about 1100 cycles), and a wave that is issuing loads cannot multiply: with all eight waves issuing behind
+// the barrier, then multiplying, then writing weight rows, the phases add up to 2900 cycles per step.  Here the roles are
+// split so that they overlap:
+//   waves 4 .. 7 (producers, one per SIMD): wave 4 + q moves sub-block q of the step for BOTH operands: activation rows
+//       by direct-to-LDS loads one step ahead, weight rows by hand-issued register loads MDP_RB steps ahead (ring of
+//       MDP_RB register sets), written into the weight stage one step ahead.  They issue loads all the time.
+//   waves 0 .. 3 (consumers, one per SIMD): wave q multiplies sub-block q of the step for the whole 16 MT x 64 tile
+//       (4 MT matrix instructions for MT + 4 fragment reads) and never touches global memory inside the loop.
+// Two stages (activations | weights | activation-scale column); one barrier per step, after which the stage just filled
+// is complete and the one just multiplied is free.  The four sub-block sums meet in LDS at the end as before.
+constexpr int MDP_RB = 3;
+constexpr int mdp_stage(int mt) { return md_a(mt) + MD_B + MD_S; }
+constexpr int mdp_lds(int mt) { return (2 * mdp_stage(mt) > md_red(mt) ? 2 * mdp_stage(mt) : md_red(mt)) + D_MAX_KT * 4; }
+
+template <int KIND, int MT, bool AS16 = false>
+__global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
+    static_assert(MT == 4 || MT == 2, "tile rows");
+    static_assert(KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || KIND == K_I8_ROWCOL || KIND == K_F16 || KIND == K_BF16, "8- and 16-bit operands");
+    constexpr int BM = 16 * MT;
+    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
+    constexpr bool ROWCOL = (KIND == K_I8_ROWCOL);
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    constexpr int MD_A = md_a(MT), STAGE = mdp_stage(MT);
+    constexpr int RB = MDP_RB;
+    constexpr int NAP = 2 * MT + (SCALED ? 1 : 0);          // direct-to-LDS loads per producer wave and step
+    constexpr int NBP = 8;                                  // register loads per producer wave and step
+    constexpr int LP = NAP + NBP;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4, q = wave & 3;
+    const bool producer = wave >= 4;
+    const int N = p.N;
+    const int K = p.K * ESZ;                                // row length in bytes
+    const int KT_all = K >> 7;                              // 128-byte sub-blocks per row
+    int kt0 = 0, KT = KT_all;                               // sub-blocks [kt0, kt0 + KT) of this workgroup
+    if (p.ksplit > 1) {
+        const int per = (((KT_all + p.ksplit - 1) / p.ksplit) + 3) & ~3;
+        kt0 = (int)blockIdx.z * per;
+        KT = max(0, min(per, KT_all - kt0));
+    }
+    const int nsteps = (KT + 3) >> 2;
+    const int n0 = blockIdx.x * MD_BN, m_start = blockIdx.y * BM, m_end = min(p.M, m_start + BM);
+    float* const bsl = (float*)(lds + (mdp_lds(MT) - D_MAX_KT * 4));
+
+    // acc[i][j][e] = C[row 16 i + r][column 16 j + 4 g + e] summed over sub-blocks q of all steps (consumers)
+    v4f acc[MT][4];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    if (producer) {
+        // ---- source offsets.  A piece = 8 rows x 128 bytes = one load instruction of the wave (lane: row lane >> 3,
+        // 16-byte chunk lane & 7); the chunk index is XOR-swizzled with (row >> 1) & 7, on the global side for the
+        // direct-to-LDS loads and on the LDS side for the weight rows, so that the fragment reads are conflict-free.
+        const int row8 = lane >> 3;
+        uint32_t aoff[2 * MT], boff[NBP], blds[NBP];
+#pragma unroll
+        for (int i = 0; i < 2 * MT; ++i) {
+            const int row = 8 * i + row8;
+            aoff[i] = (uint32_t)min(m_start + row, m_end - 1) * (uint32_t)K + (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
+        }
+#pragma unroll
+        for (int i = 0; i < NBP; ++i) {
+            const int row = 8 * i + row8;
+            boff[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (uint32_t)(lane & 7) * 16u;
+            blds[i] = (uint32_t)(MD_A + q * (MD_BN * 128) + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16));
+        }
+        constexpr uint32_t SSZ = AS16 ? 2u : 4u;
+        const uint32_t soff = (uint32_t)min(m_start + min(lane, BM - 1), m_end - 1) * (uint32_t)KT_all * SSZ;
+        // sub-block q of step s, clamped to the last one of the range (requests past the end repeat it)
+        auto kblock = [&](int s) { return kt0 + min(4 * min(max(s, 0), nsteps - 1) + q, KT - 1); };
+        auto issue_a = [&](int s) {
+            const uint32_t st = lds_base + (uint32_t)(s & 1) * STAGE;
+            const int kb = kblock(s);
+#pragma unroll
+            for (int i = 0; i < 2 * MT; ++i) dma16(st + (uint32_t)(q * (BM * 128) + 8 * i * 128), aoff[i], p.a + (int64_t)kb * 128);
+            if constexpr (SCALED) {
+                const uint32_t ss = st + MD_A + MD_B + (uint32_t)q * 256u;
+                if constexpr (AS16) dma2(ss, soff, (const uint8_t*)p.a_s + (int64_t)kb * 2);
+                else dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kb * 4);
+            }
+        };
+        v4i ring[RB][NBP];
+        auto issue_b = [&](v4i (&rs)[NBP], int s) __attribute__((always_inline)) {
+            const uint8_t* base = p.b + (int64_t)kblock(s) * 128;
+#pragma unroll
+            for (int i = 0; i < NBP; ++i) rs[i] = asm_load_b128(boff[i], base);
+        };
+        auto ring_ready = [&](v4i (&rs)[NBP], auto younger_c) __attribute__((always_inline)) {
+            constexpr int Y = decltype(younger_c)::value;
+            asm volatile("s_waitcnt vmcnt(%8)" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]), "+v"(rs[7]) : "n"(Y) : "memory");
+        };
+        auto write_b = [&](const v4i (&rs)[NBP], int s) __attribute__((always_inline)) {
+            uint8_t* st = lds + (s & 1) * STAGE;
+#pragma unroll
+            for (int i = 0; i < NBP; ++i) *(v4i*)(st + blds[i]) = rs[i];
+        };
+        static_assert(RB == 3, "the prologue below spells out three ring slots");
+        const std::integral_constant<int, 0> c0;
+        const std::integral_constant<int, (RB - 1) * LP> cb;
+        const std::integral_constant<int, (RB - 1) * NBP> cb_pro;      // step -1: only weight requests behind those of step 0
+        const std::integral_constant<int, LP + NBP> cb_first;          // step 0: one full step and the weights of step 2
+        // Step s of a producer, behind barrier s: request the activations of step s + 1 and the weights of step s + RB; the
+        // weights of step s + 1, requested RB - 1 steps ago, have landed when only the loads of the steps since are in
+        // flight: write them into the other stage; the activations just requested have landed when only the NBP weight
+        // loads behind them are in flight; barrier s + 1.
+        auto pstep = [&](auto slot_c, auto count_c, int s) __attribute__((always_inline)) {
+            constexpr int slot = decltype(slot_c)::value;    // = s mod RB
+            __builtin_amdgcn_sched_barrier(0);
+            issue_a(s + 1);
+            issue_b(ring[slot], s + RB);
+            __builtin_amdgcn_sched_barrier(0);
+            ring_ready(ring[(slot + 1) % RB], count_c);
+            write_b(ring[(slot + 1) % RB], s + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NBP) : "memory");
+            __builtin_amdgcn_s_waitcnt(0xc07f);             // lgkmcnt(0): the weight rows are in LDS
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // prologue: activations of step 0, weights of steps 0 .. RB - 1; the weights of step 0 have landed when only the
+        // two weight requests behind them are in flight (the activations, requested before them, then have too)
+        issue_a(0);
+        md_static_for<0, RB>([&](auto ic) __attribute__((always_inline)) { issue_b(ring[ic.value], ic.value); });
+        ring_ready(ring[0], cb_pro);
+        write_b(ring[0], 0);
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __syncthreads();                                    // barrier 0
+        __builtin_amdgcn_sched_barrier(0);
+        // step 0 has a wait count of its own (no activation requests in the prologue steps before it), then rounds of the
+        // three ring slots starting at slot 1
+        int s = 0;
+        if (nsteps > 0) {
+            pstep(std::integral_constant<int, 0>{}, cb_first, 0);
+            s = 1;
+            for (int rd = (nsteps - 1) / RB; rd > 0; --rd) {
+                md_static_for<0, RB>([&](auto ic) __attribute__((always_inline)) { pstep(std::integral_constant<int, (1 + ic.value) % RB>{}, cb, s + ic.value); });
+                s += RB;
+            }
+            md_static_nested<0, RB - 1>((nsteps - 1) % RB, [&](auto ic) __attribute__((always_inline)) { pstep(std::integral_constant<int, (1 + ic.value) % RB>{}, cb, s + ic.value); });
+        }
+        // everything requested has landed (also the repeated loads past the end) before the stages are reused
+        md_static_for<0, RB>([&](auto ic) __attribute__((always_inline)) { ring_ready(ring[ic.value], c0); });
+    } else {
+        // ---- consumer: fragment read offsets inside a 16-row slab: chunks g and g + 4 of row r, swizzled
+        const int lo = r * 128 + ((g ^ ((r >> 1) & 7)) * 16);
+        const int hi = r * 128 + (((g + 4) ^ ((r >> 1) & 7)) * 16);
+        auto ldfrag = [&](const uint8_t* base) {
+            const v4i x = *(const v4i*)(base + lo), y = *(const v4i*)(base + hi);
+            return (v8i){x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+        };
+        // weight scales of the tile's column block, while the producers request the first steps; barrier 0 publishes them
+        if constexpr (SCALED) {
+            const int64_t bs_row = (int64_t)(n0 >> 7) * KT_all + kt0;
+            for (int i = tid; i < KT; i += MD_THREADS / 2) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
+        }
+        __syncthreads();                                    // barrier 0
+        for (int s = 0; s < nsteps; ++s) {
+            const uint8_t* st = lds + (s & 1) * STAGE;
+            const uint8_t* As = st + q * (BM * 128);
+            const uint8_t* Bs = st + MD_A + q * (MD_BN * 128);
+            const int kb = 4 * s + q;
+            const bool live = kb < KT;                     // wave-uniform: sub-blocks past the range add nothing
+            v8i bf[4], af[2];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bf[j] = ldfrag(Bs + j * 2048);
+            af[0] = ldfrag(As);
+            if constexpr (SCALED) {
+                const float* Ss = (const float*)(st + MD_A + MD_B) + q * 64 + r;
+                const float bs = live ? bsl[min(kb, KT - 1)] : 0.f;
+                float sa[MT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    if constexpr (AS16) {
+                        const unsigned raw = ((const unsigned*)Ss)[16 * i];
+                        sa[i] = (p.s_dtype == LLMK_F16 ? f16_to_f32((unsigned short)raw) : bf16_to_f32((unsigned short)raw)) * bs;
+                    } else {
+                        sa[i] = Ss[16 * i] * bs;
+                    }
+                }
+                // the products of tile row i are scaled and accumulated while the matrix instructions of row i + 1 run
+                v4f t[2][4];
+#pragma unroll
+                for (int i = 0; i <= MT; ++i) {
+                    if (i + 1 < MT) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (i < MT) t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
+                        if (i > 0) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                const v8i zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    if (i + 1 < MT) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+                    const v8i a = live ? af[i & 1] : zero8;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] = mma_plain<KIND>(bf[j], a, acc[i][j]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();                                // barrier s + 1: this stage is free, the other one complete
+        }
+    }
+    __syncthreads();
+
+    // ---- the four sub-block sums of every output meet in LDS: red[q][row][column], rows of 68 floats
+    float* red = (float*)lds;
+    if (!producer) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *(v4f*)(red + (q * BM + 16 * i + r) * MD_RED_ROW + 16 * j + 4 * g) = acc[i][j];
+    }
+    __syncthreads();
+    // thread: row tid >> 3, columns 8 (tid & 7) .. + 7
+    const int orow = tid >> 3, ocol = 8 * (tid & 7);
+    if (orow >= BM) return;
+    const int m = m_start + orow, n = n0 + ocol;
+    if (m >= m_end || n >= N) return;
+    v4f sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (ROWCOL) {
+        v4i ia = {0, 0, 0, 0}, ib = {0, 0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float* src = red + (k * BM + orow) * MD_RED_ROW + ocol;
+            ia += *(const v4i*)src;
+            ib += *(const v4i*)(src + 4);
+        }
+        __builtin_memcpy(&sa, &ia, 16);
+        __builtin_memcpy(&sb, &ib, 16);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float* src = red + (k * BM + orow) * MD_RED_ROW + ocol;
+            sa += *(const v4f*)src;
+            sb += *(const v4f*)(src + 4);
+        }
+    }
+    const bool split = p.ksplit > 1;
+    void* cout = split ? (void*)(p.partial + (int64_t)blockIdx.z * p.M * N) : p.c;
+    const int cdt = split ? LLMK_F32 : p.c_dtype;
+    const int esz = cdt == LLMK_F32 ? 4 : 2;
+    const bool vec_ok = ((((uintptr_t)cout) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
+    const int nv = N - n;
+    const int64_t off = (int64_t)m * N + n;
+    if constexpr (ROWCOL) {
+        // (a K slice leaves its int32 sums, bit for bit, in the fp32 partial buffer: the summing pass adds them as
+        // integers and scales once, so the result does not depend on the split)
+        if (!split) {
+            rowcol_epilogue8(p, sa, sb, m, off, n, nv);
+            if (!p.c) return;
+        }
+    }
+    if (cdt == LLMK_BF16) store_run8<LLMK_BF16>(cout, off, sa, sb, nv, vec_ok);
+    else if (cdt == LLMK_F16) store_run8<LLMK_F16>(cout, off, sa, sb, nv, vec_ok);
+    else store_run8<LLMK_F32>(cout, off, sa, sb, nv, vec_ok);
+}
+
 // K slices of the mid-size kernel: as many as bring the grid to about one workgroup per CU, in whole steps of 512
 // bytes, each slice at least four steps long; 1 = no split.
 inline int mid_splitk(int64_t tiles, int64_t kbytes) {
@@ -458,12 +727,17 @@ inline bool mid_eligible(const DirectArgs& p, int mt, int ksplit) {
 template <int KIND, int MT, bool AS16 = false>
 int launch_mid(const DirectArgs& p, hipStream_t stream, const char* name) {
     static std::atomic<uint64_t> configured{0};
-    auto kern = gemm_mid_kernel<KIND, MT, AS16>;
+    constexpr bool W4 = (KIND == K_W4A8 || KIND == K_W4NK);
+    // 8- and 16-bit operands: the producer / consumer form; 4-bit weights: the form that unpacks on the way into LDS
+    auto kern = [] {
+        if constexpr (W4) return gemm_mid_kernel<KIND, MT, AS16>;
+        else return gemm_mid_pc_kernel<KIND, MT, AS16>;
+    }();
     constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK) ? 2 : 1;
     const int KT_all = (p.K * ESZ) >> 7;
     const bool split = p.ksplit > 1 && p.partial;
     const int per = split ? ((((KT_all + p.ksplit - 1) / p.ksplit) + 3) & ~3) : KT_all;
-    const int lds_bytes = md_lds(MT, KIND == K_W4A8 ? per : 0);
+    const int lds_bytes = W4 ? md_lds(MT, KIND == K_W4A8 ? per : 0) : mdp_lds(MT);
     if (lds_bytes > D_LDS_MAX) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: %d bytes of LDS needed", name, lds_bytes);
     if (int rc = llmk_reserve_lds((const void*)kern, D_LDS_MAX, configured, name)) return rc;
     // slices that would start past the end of K are not launched
