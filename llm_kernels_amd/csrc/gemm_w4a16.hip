@@ -1006,7 +1006,7 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
         p.a = (const uint8_t*)a; p.b = (const uint8_t*)b_packed; p.b_s = s; p.c = c; p.c_dtype = LLMK_F16;
         p.M = (int)M; p.N = (int)N; p.K = (int)K; p.E = 1; p.group = groupsize;
         // few column tiles and short rows: the 64-column kernel with 512-byte K steps (128 x 4096 x 4096: 18.3 -> 14 us)
-        if (llmk::mid_wanted(M, N, 2 * K)) {
+        if (2 * K <= 8192 && llmk::mid_wanted(M, N, 2 * K)) {       // (rows beyond 8 KB: measured only for the 8-bit kinds)
             llmk::MidPlan pl = llmk::mid_plan(M, N, 2 * K);
             if (pl.z > 1 && !(workspace && workspace_bytes >= (int64_t)pl.z * M * N * 4 && !((uintptr_t)workspace & 15))) pl.z = 1;
             if (llmk::mid_eligible<llmk::K_W4NK>(p, pl.mt, pl.z)) {

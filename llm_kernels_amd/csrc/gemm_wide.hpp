@@ -624,12 +624,15 @@ inline int splitk_factor(int64_t M, int64_t N, int64_t K) {
 }
 
 // Shapes for the mid-size kernel (gemm_mid.hpp): more than 64 rows, at most one workgroup per CU and a K range of at
-// most 8 KB per row.  Measured against the 128-column tile kernels (fp8, us per launch, cold weights): 128 x 4096 x 4096
-// 16.7 -> 13.7, 256 x 4096 x 4096 23.1 -> 17.8; beyond one round of workgroups or with longer rows it loses
-// (512 x 4096 x 4096 15.5 -> 23.4, 256 x 6144 x 4096 23.5 -> 27.9, 256 x 4096 x 14336 43.9 -> 47.0).
+// most 8 KB per row, 16 KB on the 64-row tile.  Measured against the 128-column tile kernels (fp8, us per launch, cold
+// weights): 128 x 4096 x 4096 16.7 -> 12.7, 256 x 4096 x 4096 23.1 -> 15.3, 256 x 4096 x 8192 28.7 -> 24.2,
+// 256 x 4096 x 14336 44.2 -> 39.0 (K slices of the 64 x 128 tile before); with more than one round of workgroups, or on
+// the 32-row tile with rows beyond 8 KB, it loses (512 x 4096 x 4096 15.5 -> 23.4, 256 x 6144 x 4096 23.5 -> 27.9,
+// 128 x 4096 x 14336 28.4 -> 29.2, per-token int8 26.2 -> 30.4).
 inline bool mid_wanted(int64_t M, int64_t N, int64_t kbytes) {
     if (M <= 64 || M > 512) return false;
-    return mid_plan(M, N, kbytes).tiles <= LLMK_CUS && kbytes <= 8192;
+    const MidPlan pl = mid_plan(M, N, kbytes);
+    return pl.tiles <= LLMK_CUS && kbytes <= (pl.mt == 4 ? 16384 : 8192);
 }
 
 // 16 < M <= 64: the weight-streaming kernel re-reads the activations for every 16 columns, which costs more
