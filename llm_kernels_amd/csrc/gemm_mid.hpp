@@ -1,26 +1,22 @@
-// Tile kernel for mid-size M (about 65 to 512 rows) on few column tiles: problems that neither fill the chip with
+// Tile kernels for mid-size M (about 65 to 512 rows) on few column tiles: problems that neither fill the chip with
 // 128- or 256-column tiles nor fit the weight-streaming kernels, and whose weights mostly come cold from HBM.
 //
 // What bounds the 64 x 128 tile of gemm_dma.hpp there is the per-step overhead: one barrier, twelve fragment reads
-// and a dependent wait per wave for four matrix instructions on 128 bytes of K.  Here a K step is 512 bytes and
-// the eight waves of a workgroup split it four ways:
+// and a dependent wait per wave for four matrix instructions on 128 bytes of K.  Here a K step is 512 bytes = four
+// 128-byte sub-blocks, the tile is 16 MT x 64 (MT = 4 or 2), a wave multiplies ONE sub-block of the step, and the four
+// partial sums of an output meet in LDS once, at the end of the tile (a K split inside the workgroup: one barrier per
+// 512 bytes of K).  Activations (hot in L2: every workgroup of a row tile reads the same rows) go global -> LDS by
+// direct-to-LDS loads one step ahead, two stages.  Weights (cold: each byte is needed by M / (16 MT) workgroups only)
+// go global -> registers several steps ahead, coalesced (eight lanes per 128-byte line), by hand-issued loads into a
+// ring of register sets, and from there into one of two LDS stages one step before they are multiplied: weight bytes
+// in flight without spending LDS on them, and a natural place to unpack 4-bit weights.  The row tiles that share a
+// column tile land on one XCD (same workgroup id modulo 8 when the column tiles are a multiple of 8) and walk K in
+// step, so that a weight line comes from HBM once.
 //
-//   tile 16 MT x 64 (MT = 4 or 2), wave (wn, kq): all 16 MT rows x 32 columns (wn = wave & 1) of the 128-byte
-//   sub-block kq = wave >> 1 of the step: 2 MT matrix-instruction tiles for 2 MT + 4 fragment reads, one barrier
-//   per 512 bytes of K; the four partial sums of an output meet in LDS once, at the end of the tile.
-//
-// Activations (hot in L2: every workgroup of a row tile reads the same rows) go global -> LDS by direct-to-LDS
-// loads, one step ahead, two stages.  Weights (cold: each byte is needed by M / (16 MT) workgroups only) go
-// global -> registers three steps ahead, coalesced (eight lanes per 128-byte line), by hand-issued loads into a
-// ring of four register sets, and from there into one of two LDS stages one step before they are multiplied:
-// 1.5 KB per weight row in flight without spending LDS on it, and a natural place to unpack 4-bit weights
-// (K_W4A8: packed words in the ring, int8 rows in LDS).  The row tiles that share a column tile land on one XCD
-// (same workgroup id modulo 8 when the column tiles are a multiple of 8) and walk K in step, so that a weight line
-// comes from HBM once.
-//
-// What bounds it (measured): a CU takes about 110 GB/s from its L2, and a 64 x 64 tile needs 128 bytes per byte of
-// K (0.6 us per step); three activation stages with the weights through a single stage between two barriers, and
-// row tiles that start their K walk at different steps, were both slower.
+// Two forms:
+//   gemm_mid_kernel     (K_W4A8): all eight waves load, unpack and multiply: wave (wn, kq) takes 32 columns of sub-block
+//                       kq.  The unpacking (q - z4) * s4 is vector-ALU work that wants every wave.
+//   gemm_mid_pc_kernel  (every other kind): four waves only request and stage operands, four only multiply; see there.
 //
 // All loads of a step are issued unconditionally (steps past the end repeat the last one) so that one
 // hand-counted s_waitcnt per step is exact; check_asm.py proves the register loads on every build.
@@ -67,20 +63,12 @@ __device__ __forceinline__ void md_static_nested(int rem, F&& f) {
 template <int KIND, int MT, bool AS16 = false>
 __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     static_assert(MT == 4 || MT == 2, "tile rows");
+    static_assert(KIND == K_W4A8, "the other kinds run on gemm_mid_pc_kernel");
     constexpr int BM = 16 * MT;
-    constexpr bool W4A8 = (KIND == K_W4A8), W4NK = (KIND == K_W4NK);
-    constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || W4A8);
-    constexpr bool ROWCOL = (KIND == K_I8_ROWCOL);
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4NK) ? 2 : 1;
     constexpr int MD_A = md_a(MT);
-    // ring loads per thread and step (K_W4NK: one vector of packed words in the ring proper, its group scale beside it)
-    constexpr int NB = W4A8 ? 2 : (W4NK ? 1 : 4);
-    constexpr int NBL = W4NK ? 2 : NB;                      // ... counted as loads
-    // ring slots: weights are requested MD_RING - 1 steps ahead.  The block-scaled 8-bit kinds on the 64-row tile keep
-    // products and accumulators apart and have no registers for a fourth slot (the build refuses spills in a
-    // kernel with hand-issued loads); three, four and five slots measured the same within the noise.
-    constexpr int MD_RING = (SCALED && !W4A8 && MT == 4) ? 3 : 4;
-    constexpr int NA = MT + (SCALED ? 1 : 0);               // direct-to-LDS loads per thread and step
+    constexpr int NB = 2;                                   // ring loads per thread and step
+    constexpr int MD_RING = 4;                              // ring slots: weights are requested MD_RING - 1 steps ahead
+    constexpr int NA = MT + 1;                              // direct-to-LDS loads per thread and step (activation pieces, scale column)
     static_assert(md_red(MT) <= md_stages(MT), "the reduction reuses the stages");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
@@ -88,7 +76,7 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4, wn = wave & 1, kq = wave >> 1;
     const int N = p.N;
-    const int K = p.K * ESZ;                                // row length in bytes
+    const int K = p.K;                                      // row length in bytes (int8 activations)
     const int KT_all = K >> 7;                              // 128-byte sub-blocks per row
     int kt0 = 0, KT = KT_all;                               // sub-blocks [kt0, kt0 + KT) of this workgroup
     if (p.ksplit > 1) {
@@ -110,7 +98,7 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     // ---- per-thread source offsets.  A piece = 8 rows x 128 bytes = what one load instruction of a wave covers
     // (lane: row lane >> 3, 16-byte chunk lane & 7, XOR-swizzled with (row >> 1) & 7 on the global side so that
     // the fragment reads are conflict-free).  Wave w moves pieces MT w .. MT w + MT - 1 of the 4 x 2 MT activation
-    // pieces and pieces 4 w .. 4 w + 3 of the 4 x 8 weight pieces of a step: piece = (sub-block, row group).
+    // pieces of a step: piece = (sub-block, row group).
     const int row8 = lane >> 3;
     uint32_t aoff[MT], alds[MT];
     int asub[MT];
@@ -122,49 +110,13 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
         alds[i] = (uint32_t)(sub * (BM * 128) + 8 * (pq % (2 * MT)) * 128);     // + lane * 16 by the hardware
         asub[i] = sub;
     }
-    uint32_t boff[4], blds[4];
-    int bsub[4];
-    uint32_t w4_soff = 0;
-    int w4_shift = 0;
-    if constexpr (W4NK) {
-        // fp16 weight rows expanded from packed words [N, K/8]: thread t takes the 32 weights k = 32 seg .. + 31
-        // (seg = t & 7) of row t >> 3 of the step's 256: 16 bytes of packed words, four 16-byte chunks of the fp16
-        // row of sub-block seg >> 1, and the group scale of those weights (groups of 64 * 2^j elements)
-        const int row = tid >> 3, seg = tid & 7;
-        const uint32_t n = (uint32_t)min(n0 + row, N - 1);
-        boff[0] = n * (uint32_t)(p.K >> 1) + (uint32_t)(seg & 1) * 16u;       // + 32 bytes per sub-block
-        w4_soff = n * (uint32_t)(p.K / p.group) * 2u;
-        w4_shift = __builtin_ctz((unsigned)(p.group >> 6));
-        bsub[0] = seg >> 1;
-        blds[0] = (uint32_t)((seg >> 1) * (MD_BN * 128) + row * 128);
-        blds[1] = (uint32_t)(((4 * (seg & 1)) ^ ((row >> 1) & 7)) * 16);      // first chunk; chunk c is at ^ (c * 16)
-        boff[1] = boff[2] = boff[3] = blds[2] = blds[3] = 0;
-        bsub[1] = bsub[2] = bsub[3] = 0;
-    } else if constexpr (!W4A8) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int pq = 4 * wave + i, sub = pq >> 3, row = 8 * (pq & 7) + row8;
-            boff[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (uint32_t)(lane & 7) * 16u;
-            blds[i] = (uint32_t)(sub * (MD_BN * 128) + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16));
-            bsub[i] = sub;
-        }
-    } else {
-        // one wave per packed row (eight weight rows): lane l takes words 4 l .. 4 l + 3 of sub-blocks l >> 5 (load 0)
-        // and 2 + (l >> 5) (load 1) of the step's 512 words
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            boff[i] = (uint32_t)min((n0 >> 3) + wave, (N >> 3) - 1) * (uint32_t)(p.K * 4) + (uint32_t)(lane & 31) * 16u;
-            bsub[i] = 2 * i + (lane >> 5);
-            blds[i] = 0;
-        }
-        boff[2] = boff[3] = blds[2] = blds[3] = 0;
-        bsub[2] = bsub[3] = 0;
-    }
+    // weights: one wave per packed row (eight weight rows): lane l takes words 4 l .. 4 l + 3 of sub-blocks l >> 5
+    // (load 0) and 2 + (l >> 5) (load 1) of the step's 512 words
+    const uint32_t boff = (uint32_t)min((n0 >> 3) + wave, (N >> 3) - 1) * (uint32_t)(p.K * 4) + (uint32_t)(lane & 31) * 16u;
     constexpr uint32_t SSZ = AS16 ? 2u : 4u;                // bytes per activation scale
     const uint32_t soff = (uint32_t)min(m_start + min(lane, BM - 1), m_end - 1) * (uint32_t)KT_all * SSZ;
 
-    // sub-block `sub` of step s, clamped to the last one of the range (loads past the end repeat it)
-    // requests past the end repeat the last step
+    // sub-block `sub` of step s, clamped to the last one of the range: requests past the end repeat the last step
     auto phys = [&](int s) { return min(s, nsteps - 1); };
     auto kblock = [&](int s, int sub) { return kt0 + min(4 * phys(s) + sub, KT - 1); };
 
@@ -172,73 +124,45 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
         const uint32_t st = lds_base + (uint32_t)(s % MD_NA) * MD_A;
 #pragma unroll
         for (int i = 0; i < MT; ++i) dma16(st + alds[i], aoff[i], p.a + (int64_t)kblock(s, asub[i]) * 128);
-        if constexpr (SCALED) {
-            const uint32_t ss = lds_base + MD_NA * MD_A + MD_NBS * MD_B + (uint32_t)(s % MD_NA) * MD_S + (uint32_t)(wave & 3) * 256u;
-            if constexpr (AS16) dma2(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 2);
-            else dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 4);
-        }
+        const uint32_t ss = lds_base + MD_NA * MD_A + MD_NBS * MD_B + (uint32_t)(s % MD_NA) * MD_S + (uint32_t)(wave & 3) * 256u;
+        if constexpr (AS16) dma2(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 2);
+        else dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kblock(s, wave & 3) * 4);
     };
     // ring of weight registers: slot = step % 4
     v4i ring[MD_RING][NB];
-    unsigned ringsc[MD_RING] = {};                            // K_W4NK: group scale of the slot's weights (fp16 bits)
-    auto issue_b = [&](v4i (&rs)[NB], unsigned& rsc, int s) __attribute__((always_inline)) {
-        if constexpr (W4NK) {
-            // lane-dependent sub-block (the eight lanes of a row cover the four sub-blocks of the step)
-            const int kb0 = kblock(s, 0), kb = kt0 + min(4 * phys(s) + bsub[0], KT - 1);
-            rs[0] = asm_load_b128(boff[0] + (uint32_t)(kb - kb0) * 32u, (const uint8_t*)p.b + (int64_t)kb0 * 32);
-            rsc = asm_load_u16(w4_soff + (uint32_t)(kb >> w4_shift) * 2u, p.b_s);
-        }
+    auto issue_b = [&](v4i (&rs)[NB], int s) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < (W4NK ? 0 : NB); ++i) {
-            if constexpr (W4A8) {
-                // lane-dependent sub-block: the two halves of the wave read different 128-word runs of the row
-                const int kb0 = kblock(s, 2 * i), kb1 = kblock(s, 2 * i + 1);
-                const uint32_t off = boff[i] + (uint32_t)((lane >> 5) ? kb1 - kb0 : 0) * 512u;
-                rs[i] = asm_load_b128(off, (const uint8_t*)p.b + (int64_t)kb0 * 512);
-            } else {
-                rs[i] = asm_load_b128(boff[i], p.b + (int64_t)kblock(s, bsub[i]) * 128);
-            }
+        for (int i = 0; i < NB; ++i) {
+            // lane-dependent sub-block: the two halves of the wave read different 128-word runs of the row
+            const int kb0 = kblock(s, 2 * i), kb1 = kblock(s, 2 * i + 1);
+            const uint32_t off = boff + (uint32_t)((lane >> 5) ? kb1 - kb0 : 0) * 512u;
+            rs[i] = asm_load_b128(off, (const uint8_t*)p.b + (int64_t)kb0 * 512);
         }
     };
     // the loads of slot `slot` have landed when at most `younger` loads issued after them are in flight
-    auto ring_ready = [&](v4i (&rs)[NB], unsigned& rsc, auto younger_c) __attribute__((always_inline)) {
+    auto ring_ready = [&](v4i (&rs)[NB], auto younger_c) __attribute__((always_inline)) {
         constexpr int Y = decltype(younger_c)::value;
-        if constexpr (W4NK)
-            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(rs[0]), "+v"(rsc) : "n"(Y) : "memory");
-        else if constexpr (NB == 4)
-            asm volatile("s_waitcnt vmcnt(%4)" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]) : "n"(Y) : "memory");
-        else
-            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(rs[0]), "+v"(rs[1]) : "n"(Y) : "memory");
+        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(rs[0]), "+v"(rs[1]) : "n"(Y) : "memory");
     };
-    // ring slot -> weight stage s & 1 (nobody has read that stage since the barrier of step s - 1)
-    auto produce = [&](const v4i (&rs)[NB], unsigned rsc, int s) __attribute__((always_inline)) {
+    // ring slot -> weight stage s & 1 (nobody has read that stage since the barrier of step s - 1), as int8 rows
+    // (q - z4) * s4.  Lane: words 4 kc .. 4 kc + 3 (kc = lane & 31) of sub-block 2 i + (lane >> 5); packed row = wave;
+    // row j of the packed row is tile column 8 wave + j.
+    auto produce = [&](const v4i (&rs)[NB], int s) __attribute__((always_inline)) {
         uint8_t* st = b_st + (s % MD_NBS) * MD_B;
-        if constexpr (W4NK) {
-            const v2h sc = w4_as_h2(rsc | (rsc << 16));
-            uint8_t* row = st + blds[0];
+        const int kc = lane & 31;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) *(v4i*)(row + (blds[1] ^ (uint32_t)(c * 16))) = w4_word_to_f16x8((unsigned)rs[0][c], sc);
-        } else if constexpr (!W4A8) {
+        for (int i = 0; i < 2; ++i) {
+            const int sub = 2 * i + (lane >> 5);
+            const int kb = min(4 * phys(s) + sub, KT - 1);
+            const uint8_t* tabk = w4tab + kb * 64 + 8 * wave;
+            unsigned sp[4], cp[4], rows[8];
+            w4a8_row_consts(*(const uint2*)tabk, *(const uint2*)(tabk + 64 * KT), sp, cp);
+            w4a8_words_to_i8(rs[i], sp, cp, rows);
+            uint8_t* dst = st + sub * (MD_BN * 128) + (kc & 3) * 4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) *(v4i*)(st + blds[i]) = rs[i];
-        } else {
-            // lane: words 4 kc .. 4 kc + 3 (kc = lane & 31) of sub-block 2 i + (lane >> 5); packed row = wave.  Row j of
-            // the packed row is tile column 8 wave + j.
-            const int kc = lane & 31;
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int sub = 2 * i + (lane >> 5);
-                const int kb = min(4 * phys(s) + sub, KT - 1);
-                const uint8_t* tabk = w4tab + kb * 64 + 8 * wave;
-                unsigned sp[4], cp[4], rows[8];
-                w4a8_row_consts(*(const uint2*)tabk, *(const uint2*)(tabk + 64 * KT), sp, cp);
-                w4a8_words_to_i8(rs[i], sp, cp, rows);
-                uint8_t* dst = st + sub * (MD_BN * 128) + (kc & 3) * 4;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int R = 8 * wave + j;
-                    *(unsigned*)(dst + R * 128 + (((kc >> 2) ^ ((R >> 1) & 7)) * 16)) = rows[j];
-                }
+            for (int j = 0; j < 8; ++j) {
+                const int R = 8 * wave + j;
+                *(unsigned*)(dst + R * 128 + (((kc >> 2) ^ ((R >> 1) & 7)) * 16)) = rows[j];
             }
         }
     };
@@ -265,92 +189,72 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) bf[j] = ldfrag(Bs + j * 2048);
         af[0] = ldfrag(As);
-        const v8i zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-        if constexpr (SCALED) {
-            const float* Ss = (const float*)(s_st + (s % MD_NA) * MD_S) + kq * 64 + r;
-            const float bs = live ? bsl[min(kb, KT - 1)] : 0.f;
-            float sa[MT];
+        const float* Ss = (const float*)(s_st + (s % MD_NA) * MD_S) + kq * 64 + r;
+        const float bs = live ? bsl[min(kb, KT - 1)] : 0.f;
+        float sa[MT];
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                if constexpr (AS16) {
-                    const unsigned raw = ((const unsigned*)Ss)[16 * i];
-                    sa[i] = (p.s_dtype == LLMK_F16 ? f16_to_f32((unsigned short)raw) : bf16_to_f32((unsigned short)raw)) * bs;
-                } else {
-                    sa[i] = Ss[16 * i] * bs;
-                }
+        for (int i = 0; i < MT; ++i) {
+            if constexpr (AS16) {
+                const unsigned raw = ((const unsigned*)Ss)[16 * i];
+                sa[i] = (p.s_dtype == LLMK_F16 ? f16_to_f32((unsigned short)raw) : bf16_to_f32((unsigned short)raw)) * bs;
+            } else {
+                sa[i] = Ss[16 * i] * bs;
             }
-            // the products of tile row i are scaled and accumulated while the matrix instructions of row i + 1 run
-            v4f t[2][2];
+        }
+        // the products of tile row i are scaled and accumulated while the matrix instructions of row i + 1 run
+        v4f t[2][2];
 #pragma unroll
-            for (int i = 0; i <= MT; ++i) {
-                if (i + 1 < MT) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
+        for (int i = 0; i <= MT; ++i) {
+            if (i + 1 < MT) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    if (i < MT) t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
-                    if (i > 0) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
-                }
-                // nothing moves across a tile row: the lag of one row between product and accumulation stays, and
-                // the fragments of at most two rows are live
-                __builtin_amdgcn_sched_barrier(0);
+            for (int j = 0; j < 2; ++j) {
+                if (i < MT) t[i & 1][j] = step_dot<KIND>(bf[j], af[i & 1]);
+                if (i > 0) acc[i - 1][j] += t[(i - 1) & 1][j] * sa[i - 1];
             }
-        } else {
-#pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                if (i + 1 < MT) af[(i + 1) & 1] = ldfrag(As + (i + 1) * 2048);
-                const v8i a = live ? af[i & 1] : zero8;
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = mma_plain<KIND>(bf[j], a, acc[i][j]);
-            }
+            // nothing moves across a tile row: the lag of one row between product and accumulation stays, and
+            // the fragments of at most two rows are live
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
     const std::integral_constant<int, 0> c0;
-    const std::integral_constant<int, (MD_RING - 2) * NBL> cpro;
-    const std::integral_constant<int, NBL> cnb;
-    const std::integral_constant<int, NA + NBL> cstep;
-
+    const std::integral_constant<int, (MD_RING - 2) * NB> cpro;
+    const std::integral_constant<int, NB> cnb;
 
     // ---- prologue: activations of step 0, weights of steps 0, 1, 2; tables by ordinary loads meanwhile
     issue_a(0);
-    md_static_for<0, MD_RING - 1>([&](auto ic) __attribute__((always_inline)) { issue_b(ring[ic.value], ringsc[ic.value], ic.value); });
-    if constexpr (SCALED) {
-        const int64_t bs_row = (int64_t)(n0 >> 7) * KT_all + kt0;
-        for (int i = tid; i < KT; i += MD_THREADS) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
+    md_static_for<0, MD_RING - 1>([&](auto ic) __attribute__((always_inline)) { issue_b(ring[ic.value], ic.value); });
+    const int64_t bs_row = (int64_t)(n0 >> 7) * KT_all + kt0;
+    for (int i = tid; i < KT; i += MD_THREADS) bsl[i] = ld_scale(p.b_s, bs_row + i, p.s_dtype);
+    for (int i = tid; i < 64 * KT; i += MD_THREADS) {
+        const int row = i / KT, kk = i - row * KT;
+        const int64_t at = (int64_t)min(n0 + row, N - 1) * KT_all + kt0 + kk;
+        w4tab[kk * 64 + row] = (uint8_t)p.w4_s4[at];
+        w4tab[(KT + kk) * 64 + row] = (uint8_t)p.w4_z4[at];
     }
-    if constexpr (W4A8) {
-        for (int i = tid; i < 64 * KT; i += MD_THREADS) {
-            const int row = i / KT, kk = i - row * KT;
-            const int64_t at = (int64_t)min(n0 + row, N - 1) * KT_all + kt0 + kk;
-            w4tab[kk * 64 + row] = (uint8_t)p.w4_s4[at];
-            w4tab[(KT + kk) * 64 + row] = (uint8_t)p.w4_z4[at];
-        }
-        __syncthreads();                                    // the table is read by produce()
-    }
-    ring_ready(ring[0], ringsc[0], cpro);
-    produce(ring[0], ringsc[0], 0);
+    __syncthreads();                                        // the table is read by produce()
+    ring_ready(ring[0], cpro);
+    produce(ring[0], 0);
 
     // One step: wait for the activations of step s (requested a step ago; only the NB weight loads issued after
     // them may stay in flight; with four ring slots that also vouches for slot s + 1, requested two steps ago),
     // meet the others, request the activations of step s + 1 and the weights of step s + MD_RING - 1, multiply
-    // step s, and move the weights of step s + 1 from the ring into the other weight stage (with three slots they
-    // were requested a step ago: everything but this step's own requests has landed by then).
+    // step s, and move the weights of step s + 1 from the ring into the other weight stage.
     auto step = [&](auto slot_c, int s) __attribute__((always_inline)) {
         constexpr int slot = decltype(slot_c)::value;
         // (scheduling fences: without them the compiler carries the matrix instructions of a step across the next
         // barrier, with all fragments of two steps live, and spills)
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (MD_RING >= 4) ring_ready(ring[(slot + 1) % MD_RING], ringsc[(slot + 1) % MD_RING], cnb);
-        else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NBL) : "memory");
+        ring_ready(ring[(slot + 1) % MD_RING], cnb);
         __builtin_amdgcn_s_waitcnt(0xc07f);                 // lgkmcnt(0): this wave's LDS writes of produce() are done
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         issue_a(s + 1);
-        issue_b(ring[(slot + MD_RING - 1) % MD_RING], ringsc[(slot + MD_RING - 1) % MD_RING], s + MD_RING - 1);
+        issue_b(ring[(slot + MD_RING - 1) % MD_RING], s + MD_RING - 1);
         __builtin_amdgcn_sched_barrier(0);
         compute(s);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (MD_RING == 3) ring_ready(ring[(slot + 1) % MD_RING], ringsc[(slot + 1) % MD_RING], cstep);
-        produce(ring[(slot + 1) % MD_RING], ringsc[(slot + 1) % MD_RING], s + 1);
+        produce(ring[(slot + 1) % MD_RING], s + 1);
         __builtin_amdgcn_sched_barrier(0);
     };
     int s = 0;
@@ -360,7 +264,7 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     }
     md_static_nested<0, MD_RING - 1>(nsteps % MD_RING, [&](auto ic) __attribute__((always_inline)) { step(ic, s + ic.value); });
     // everything requested has landed (also the repeated loads past the end) before the stages are reused
-    md_static_for<0, MD_RING>([&](auto ic) __attribute__((always_inline)) { ring_ready(ring[ic.value], ringsc[ic.value], c0); });
+    md_static_for<0, MD_RING>([&](auto ic) __attribute__((always_inline)) { ring_ready(ring[ic.value], c0); });
     __syncthreads();
 
     // ---- the four sub-block sums of every output meet in LDS: red[kq][row][column], rows of 68 floats
@@ -377,23 +281,11 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     const int m = m_start + orow, n = n0 + ocol;
     if (m >= m_end || n >= N) return;
     v4f sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (ROWCOL) {
-        v4i ia = {0, 0, 0, 0}, ib = {0, 0, 0, 0};
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float* src = red + (q * BM + orow) * MD_RED_ROW + ocol;
-            ia += *(const v4i*)src;
-            ib += *(const v4i*)(src + 4);
-        }
-        __builtin_memcpy(&sa, &ia, 16);
-        __builtin_memcpy(&sb, &ib, 16);
-    } else {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float* src = red + (q * BM + orow) * MD_RED_ROW + ocol;
-            sa += *(const v4f*)src;
-            sb += *(const v4f*)(src + 4);
-        }
+    for (int q = 0; q < 4; ++q) {
+        const float* src = red + (q * BM + orow) * MD_RED_ROW + ocol;
+        sa += *(const v4f*)src;
+        sb += *(const v4f*)(src + 4);
     }
     const bool split = p.ksplit > 1;
     void* cout = split ? (void*)(p.partial + (int64_t)blockIdx.z * p.M * N) : p.c;
@@ -402,14 +294,6 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     const bool vec_ok = ((((uintptr_t)cout) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
     const int nv = N - n;
     const int64_t off = (int64_t)m * N + n;
-    if constexpr (ROWCOL) {
-        // (a K slice leaves its int32 sums, bit for bit, in the fp32 partial buffer: the summing pass adds them as
-        // integers and scales once, so the result does not depend on the split)
-        if (!split) {
-            rowcol_epilogue8(p, sa, sb, m, off, n, nv);
-            if (!p.c) return;
-        }
-    }
     if (cdt == LLMK_BF16) store_run8<LLMK_BF16>(cout, off, sa, sb, nv, vec_ok);
     else if (cdt == LLMK_F16) store_run8<LLMK_F16>(cout, off, sa, sb, nv, vec_ok);
     else store_run8<LLMK_F32>(cout, off, sa, sb, nv, vec_ok);
@@ -436,15 +320,20 @@ constexpr int mdp_lds(int mt) { return (2 * mdp_stage(mt) > md_red(mt) ? 2 * mdp
 template <int KIND, int MT, bool AS16 = false>
 __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
     static_assert(MT == 4 || MT == 2, "tile rows");
-    static_assert(KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || KIND == K_I8_ROWCOL || KIND == K_F16 || KIND == K_BF16, "8- and 16-bit operands");
+    static_assert(KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || KIND == K_I8_ROWCOL || KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK,
+                  "8- and 16-bit operands, or fp16 activations with row-packed 4-bit weights");
     constexpr int BM = 16 * MT;
+    // K_W4NK: the producers load packed words [N, K/8] and their group scales (fp16, groups of 64 * 2^j elements) and write
+    // fp16 weight rows (q - 8) * scale into the weight stage; the rest is the fp16 kind
+    constexpr bool W4NK = (KIND == K_W4NK);
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
     constexpr bool ROWCOL = (KIND == K_I8_ROWCOL);
-    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16) ? 2 : 1;
+    constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4NK) ? 2 : 1;
     constexpr int MD_A = md_a(MT), STAGE = mdp_stage(MT);
     constexpr int RB = MDP_RB;
     constexpr int NAP = 2 * MT + (SCALED ? 1 : 0);          // direct-to-LDS loads per producer wave and step
-    constexpr int NBP = 8;                                  // register loads per producer wave and step
+    constexpr int NBR = W4NK ? 2 : 8;                       // 16-byte weight registers per producer lane and step
+    constexpr int NBP = W4NK ? 4 : 8;                       // register loads per producer wave and step (K_W4NK: + two scales)
     constexpr int LP = NAP + NBP;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
@@ -477,18 +366,34 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
         // 16-byte chunk lane & 7); the chunk index is XOR-swizzled with (row >> 1) & 7, on the global side for the
         // direct-to-LDS loads and on the LDS side for the weight rows, so that the fragment reads are conflict-free.
         const int row8 = lane >> 3;
-        uint32_t aoff[2 * MT], boff[NBP], blds[NBP];
+        uint32_t aoff[2 * MT], boff[NBR], blds[NBR], w4_soff[2] = {0, 0}, w4_chunk[2] = {0, 0};
+        int w4_shift = 0;
+        const int w4_sub = (tid >> 1) & 3;                  // K_W4NK: sub-block of this lane's 32 weights
 #pragma unroll
         for (int i = 0; i < 2 * MT; ++i) {
             const int row = 8 * i + row8;
             aoff[i] = (uint32_t)min(m_start + row, m_end - 1) * (uint32_t)K + (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
         }
 #pragma unroll
-        for (int i = 0; i < NBP; ++i) {
-            const int row = 8 * i + row8;
-            boff[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (uint32_t)(lane & 7) * 16u;
-            blds[i] = (uint32_t)(MD_A + q * (MD_BN * 128) + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16));
+        for (int i = 0; i < NBR; ++i) {
+            if constexpr (W4NK) {
+                // producer thread t = 0 .. 255: the 32 weights k = 32 seg .. + 31 (seg = t & 7) of the step's 256 of rows
+                // t >> 3 and 32 + (t >> 3): 16 bytes of packed words each, four 16-byte chunks of the fp16 row of
+                // sub-block seg >> 1, and the group scale of those weights
+                const int row = ((tid - 256) >> 3) + 32 * i, seg = tid & 7;
+                const uint32_t n = (uint32_t)min(n0 + row, N - 1);
+                boff[i] = n * (uint32_t)(p.K >> 1) + (uint32_t)(seg & 1) * 16u;       // + 32 bytes per sub-block
+                w4_soff[i] = n * (uint32_t)(p.K / p.group) * 2u;
+                blds[i] = (uint32_t)(MD_A + (seg >> 1) * (MD_BN * 128) + row * 128);
+                w4_chunk[i] = (uint32_t)(((4 * (seg & 1)) ^ ((row >> 1) & 7)) * 16);  // first chunk; chunk c is at ^ (c * 16)
+            } else {
+                const int row = 8 * i + row8;
+                boff[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (uint32_t)(lane & 7) * 16u;
+                blds[i] = (uint32_t)(MD_A + q * (MD_BN * 128) + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16));
+            }
         }
+        if constexpr (W4NK) w4_shift = __builtin_ctz((unsigned)(p.group >> 6));
+        auto kblock_sub = [&](int s, int sub) { return kt0 + min(4 * min(max(s, 0), nsteps - 1) + sub, KT - 1); };
         constexpr uint32_t SSZ = AS16 ? 2u : 4u;
         const uint32_t soff = (uint32_t)min(m_start + min(lane, BM - 1), m_end - 1) * (uint32_t)KT_all * SSZ;
         // sub-block q of step s, clamped to the last one of the range (requests past the end repeat it)
@@ -504,20 +409,43 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
                 else dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kb * 4);
             }
         };
-        v4i ring[RB][NBP];
-        auto issue_b = [&](v4i (&rs)[NBP], int s) __attribute__((always_inline)) {
-            const uint8_t* base = p.b + (int64_t)kblock(s) * 128;
+        v4i ring[RB][NBR];
+        unsigned ringsc[RB][2] = {};                        // K_W4NK: group scales of the slot's weights (fp16 bits)
+        auto issue_b = [&](v4i (&rs)[NBR], unsigned (&rsc)[2], int s) __attribute__((always_inline)) {
+            if constexpr (W4NK) {
+                // lane-dependent sub-block (the eight lanes of a row cover the four sub-blocks of the step)
+                const int kb0 = kblock_sub(s, 0), kb = kblock_sub(s, w4_sub);
 #pragma unroll
-            for (int i = 0; i < NBP; ++i) rs[i] = asm_load_b128(boff[i], base);
+                for (int i = 0; i < 2; ++i) {
+                    rs[i] = asm_load_b128(boff[i] + (uint32_t)(kb - kb0) * 32u, (const uint8_t*)p.b + (int64_t)kb0 * 32);
+                    rsc[i] = asm_load_u16(w4_soff[i] + (uint32_t)(kb >> w4_shift) * 2u, p.b_s);
+                }
+            } else {
+                const uint8_t* base = p.b + (int64_t)kblock(s) * 128;
+#pragma unroll
+                for (int i = 0; i < NBR; ++i) rs[i] = asm_load_b128(boff[i], base);
+            }
         };
-        auto ring_ready = [&](v4i (&rs)[NBP], auto younger_c) __attribute__((always_inline)) {
+        auto ring_ready = [&](v4i (&rs)[NBR], unsigned (&rsc)[2], auto younger_c) __attribute__((always_inline)) {
             constexpr int Y = decltype(younger_c)::value;
-            asm volatile("s_waitcnt vmcnt(%8)" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]), "+v"(rs[7]) : "n"(Y) : "memory");
+            if constexpr (W4NK)
+                asm volatile("s_waitcnt vmcnt(%4)" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rsc[0]), "+v"(rsc[1]) : "n"(Y) : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(%8)" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]), "+v"(rs[4]), "+v"(rs[5]), "+v"(rs[6]), "+v"(rs[7]) : "n"(Y) : "memory");
         };
-        auto write_b = [&](const v4i (&rs)[NBP], int s) __attribute__((always_inline)) {
+        auto write_b = [&](const v4i (&rs)[NBR], const unsigned (&rsc)[2], int s) __attribute__((always_inline)) {
             uint8_t* st = lds + (s & 1) * STAGE;
+            if constexpr (W4NK) {
 #pragma unroll
-            for (int i = 0; i < NBP; ++i) *(v4i*)(st + blds[i]) = rs[i];
+                for (int i = 0; i < 2; ++i) {
+                    const v2h sc = w4_as_h2(rsc[i] | (rsc[i] << 16));
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) *(v4i*)(st + blds[i] + (w4_chunk[i] ^ (uint32_t)(c * 16))) = w4_word_to_f16x8((unsigned)rs[i][c], sc);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NBR; ++i) *(v4i*)(st + blds[i]) = rs[i];
+            }
         };
         static_assert(RB == 3, "the prologue below spells out three ring slots");
         const std::integral_constant<int, 0> c0;
@@ -532,10 +460,10 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
             constexpr int slot = decltype(slot_c)::value;    // = s mod RB
             __builtin_amdgcn_sched_barrier(0);
             issue_a(s + 1);
-            issue_b(ring[slot], s + RB);
+            issue_b(ring[slot], ringsc[slot], s + RB);
             __builtin_amdgcn_sched_barrier(0);
-            ring_ready(ring[(slot + 1) % RB], count_c);
-            write_b(ring[(slot + 1) % RB], s + 1);
+            ring_ready(ring[(slot + 1) % RB], ringsc[(slot + 1) % RB], count_c);
+            write_b(ring[(slot + 1) % RB], ringsc[(slot + 1) % RB], s + 1);
             __builtin_amdgcn_sched_barrier(0);
             asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NBP) : "memory");
             __builtin_amdgcn_s_waitcnt(0xc07f);             // lgkmcnt(0): the weight rows are in LDS
@@ -545,9 +473,9 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
         // prologue: activations of step 0, weights of steps 0 .. RB - 1; the weights of step 0 have landed when only the
         // two weight requests behind them are in flight (the activations, requested before them, then have too)
         issue_a(0);
-        md_static_for<0, RB>([&](auto ic) __attribute__((always_inline)) { issue_b(ring[ic.value], ic.value); });
-        ring_ready(ring[0], cb_pro);
-        write_b(ring[0], 0);
+        md_static_for<0, RB>([&](auto ic) __attribute__((always_inline)) { issue_b(ring[ic.value], ringsc[ic.value], ic.value); });
+        ring_ready(ring[0], ringsc[0], cb_pro);
+        write_b(ring[0], ringsc[0], 0);
         __builtin_amdgcn_s_waitcnt(0xc07f);
         __syncthreads();                                    // barrier 0
         __builtin_amdgcn_sched_barrier(0);
@@ -564,7 +492,7 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
             md_static_nested<0, RB - 1>((nsteps - 1) % RB, [&](auto ic) __attribute__((always_inline)) { pstep(std::integral_constant<int, (1 + ic.value) % RB>{}, cb, s + ic.value); });
         }
         // everything requested has landed (also the repeated loads past the end) before the stages are reused
-        md_static_for<0, RB>([&](auto ic) __attribute__((always_inline)) { ring_ready(ring[ic.value], c0); });
+        md_static_for<0, RB>([&](auto ic) __attribute__((always_inline)) { ring_ready(ring[ic.value], ringsc[ic.value], c0); });
     } else {
         // ---- consumer: fragment read offsets inside a 16-row slab: chunks g and g + 4 of row r, swizzled
         const int lo = r * 128 + ((g ^ ((r >> 1) & 7)) * 16);
@@ -727,8 +655,8 @@ inline bool mid_eligible(const DirectArgs& p, int mt, int ksplit) {
 template <int KIND, int MT, bool AS16 = false>
 int launch_mid(const DirectArgs& p, hipStream_t stream, const char* name) {
     static std::atomic<uint64_t> configured{0};
-    constexpr bool W4 = (KIND == K_W4A8 || KIND == K_W4NK);
-    // 8- and 16-bit operands: the producer / consumer form; 4-bit weights: the form that unpacks on the way into LDS
+    constexpr bool W4 = (KIND == K_W4A8);
+    // the producer / consumer form, except for w4a8 (whose expansion is vector-ALU work that wants all eight waves)
     auto kern = [] {
         if constexpr (W4) return gemm_mid_kernel<KIND, MT, AS16>;
         else return gemm_mid_pc_kernel<KIND, MT, AS16>;
@@ -737,7 +665,7 @@ int launch_mid(const DirectArgs& p, hipStream_t stream, const char* name) {
     const int KT_all = (p.K * ESZ) >> 7;
     const bool split = p.ksplit > 1 && p.partial;
     const int per = split ? ((((KT_all + p.ksplit - 1) / p.ksplit) + 3) & ~3) : KT_all;
-    const int lds_bytes = W4 ? md_lds(MT, KIND == K_W4A8 ? per : 0) : mdp_lds(MT);
+    const int lds_bytes = W4 ? md_lds(MT, per) : mdp_lds(MT);
     if (lds_bytes > D_LDS_MAX) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: %d bytes of LDS needed", name, lds_bytes);
     if (int rc = llmk_reserve_lds((const void*)kern, D_LDS_MAX, configured, name)) return rc;
     // slices that would start past the end of K are not launched
