@@ -238,6 +238,23 @@ int llmk_moe_pre_reorder_quant(const void* x, int x_dtype, void* q_out, void* s_
                                int round_mode, const int32_t* src2dst, const void* topk_ids,
                                int ids_bytes, const float* a1_scales, int start_expert, int end_expert,
                                int topk, int64_t T, int64_t hidden, void* stream);
+/* Grouped gate / up projection with the gated activation and the 1 x 128 quantiser of the down projection in its
+ * epilogue: q_out, s_out = llmk_moe_act_and_mul_quant(llmk_grouped_gemm(a, b) rounded to mid_dtype), bit for bit, without
+ * the [M, 2I] tensor in between (the reference runs grouped_gemm_triton, silu_and_mul_triton_kernel and the activation
+ * quantiser of the next grouped_gemm_triton one after the other: moe/sglang_moe_all_gather_all_reduce.py:330-408).
+ * a [M, K] and b [E, 2I, K] (gate rows first) in the operand type of `kind` (LLMK_KIND_FP8 or LLMK_KIND_I8) with block
+ * scales scale_a [M, K/128], scale_b [E, 2I/128, K/128] of s_dtype; mid_dtype LLMK_F16 or LLMK_BF16 = the dtype the
+ * separate GEMM would have written; act 0 silu, 1 tanh-gelu; q_out [M, I], s_out [M, I/128] as in
+ * llmk_moe_act_and_mul_quant (no per-expert scales).  Rows outside every segment are left unwritten.  16-bit scales
+ * need M * K/128 * 4 bytes of workspace.  Taken only for shapes that run on the 256-column tile kernel:
+ * llmk_grouped_gemm_swiglu_quant_fused returns 1 for those, 0 otherwise (then run the three calls), and the fused entry
+ * fails with LLMK_ERR_SHAPE on a shape it does not take. */
+int llmk_grouped_gemm_swiglu_quant_fused(int kind, int E, int64_t M, int64_t two_i, int64_t K);
+int llmk_grouped_gemm_swiglu_quant(const void* a, const void* b, void* q_out, void* s_out, int kind,
+                                   int mid_dtype, int round_mode, int E, int64_t M, int64_t two_i, int64_t K,
+                                   const int64_t* seg_indptr, const int64_t* weight_indices,
+                                   const void* scale_a, const void* scale_b, int s_dtype, int act,
+                                   void* workspace, int64_t workspace_bytes, void* stream);
 /* w_dtype: dtype code of topk_weights. */
 int llmk_moe_post_reorder(const void* down_out, void* out, int dtype, const int32_t* src2dst,
                           const void* topk_ids, int ids_bytes, const void* topk_weights, int w_dtype,

@@ -59,6 +59,8 @@ SIGNATURES = {
     "llmk_moe_pre_reorder": [_p, _i, _p, _i, _p, _p, _i, _p, _i, _i, _i, _l, _l, _p],
     "llmk_moe_act_and_mul": [_p, _i, _p, _i, _p, _i, _p, _i, _i, _l, _l, _i, _p],
     "llmk_moe_act_and_mul_quant": [_p, _i, _p, _p, _i, _i, _p, _i, _p, _i, _i, _l, _l, _i, _p],
+    "llmk_grouped_gemm_swiglu_quant_fused": [_i, _i, _l, _l, _l],
+    "llmk_grouped_gemm_swiglu_quant": [_p, _p, _p, _p, _i, _i, _i, _i, _l, _l, _l, _p, _p, _p, _p, _i, _i, _p, _l, _p],
     "llmk_moe_pre_reorder_quant": [_p, _i, _p, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _l, _l, _p],
     "llmk_moe_post_reorder": [_p, _p, _i, _p, _p, _i, _p, _i, _i, _i, _i, _l, _l, _p],
     "llmk_moe_expert_scales": [_p, _p, _p, _i, _i, _l, _l, _l, _p, _p, _i, _p],

@@ -103,7 +103,11 @@ struct DirectArgs {
     long long* clocks;     // 256-column tile kernel, calibration only: workgroup 0 leaves the s_memtime and s_memrealtime ticks it lived
     const int8_t* w4_s4;   // K_W4A8: second-level scales [N, K/128]
     const int8_t* w4_z4;   // K_W4A8: zero points [N, K/128]
-    int tail_split;        // 256-column tile kernel: the tiles of a short last round are split along K (partial = scratch)
+    int tail_split;        // 256-column tile kernel: the tiles of a short last round are split along K (partial = scratch)    // 256-column tile kernel with the gated-activation epilogue (grouped gate / up projection, N = 2 I): c receives the
+    // 1 x 128 quantised activations [M, I] in the operand type, q_scale their scales [M, I / 128]
+    void* q_scale;
+    int act;               // 0 = SiLU, 1 = GELU (tanh form)
+    int round_mode;        // int8 rounding of the quantiser
 };
 
 // Upper bound of the row tiles of a grouped GEMM (segment ends are only known on the device): every segment

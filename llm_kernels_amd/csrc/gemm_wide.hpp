@@ -17,6 +17,7 @@
 #pragma once
 #include <type_traits>
 #include "gemm_mid.hpp"
+#include "quant_util.hpp"
 
 namespace llmk {
 
@@ -151,10 +152,17 @@ __host__ __device__ inline WideTail wide_tail_plan(int total, int KT) {
 }
 constexpr int W_TAIL_ITEMS = LLMK_CUS;          // upper bound of ntail * z
 
-template <int KIND, bool GROUPED, int R = 8>
+// SWIGLU (grouped gate / up projection of a gated MLP, weights [E, 2 I, K] with the I gate rows first): the tile's 256
+// columns are gate columns n0 .. n0 + 127 and up columns I + n0 .. I + n0 + 127 (n0 = 128 blockIdx.x), and instead of
+// storing them the workgroup applies the gated activation and the 1 x 128 activation quantiser of the next projection:
+// p.c receives [M, I] quantised values, p.q_scale their scales.  Every rounding point of the separate kernels is kept
+// (sums rounded to the tensor dtype p.c_dtype, activation and product in that dtype, the quantiser's own arithmetic), so
+// the outputs equal those of GEMM + activation + quantiser bit for bit; the [M, 2 I] tensor never exists.
+template <int KIND, bool GROUPED, int R = 8, bool SWIGLU = false>
 __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     constexpr bool AS16 = false;             // 16-bit activation scales are widened before this kernel, see launch_big
     static_assert(R == 8 || R == 4, "tile rows per wave");
+    static_assert(!SWIGLU || (GROUPED && (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK)), "gated epilogue: grouped block-scaled kinds");
     constexpr int W_BM = w_bm(R), W_A = W_BM * 128, W_STAGE = w_stage(R);
     constexpr int AL = R / 2;                    // activation loads per thread and stage
     constexpr int W_EARLY_ROW = R == 8 ? 5 : 2;  // tile row in front of which the mid-step barrier sits
@@ -207,7 +215,8 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         bbase += widx * (int64_t)N * K;
         bs_off = widx * (int64_t)((N + 127) / 128) * KT_all;
     }
-    const int n0 = bx * W_BN;
+    const int n0 = bx * (SWIGLU ? 128 : W_BN);
+    const int I_half = N >> 1;               // SWIGLU: gate rows [0, I), up rows [I, 2 I) of the weight matrix
 
     // weight scales of the tile's two 128-column blocks, for every K step
     float* bsl = (float*)(lds + 2 * W_STAGE);
@@ -234,7 +243,8 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         const uint32_t chunk = (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
         const int rho = row & 63;
         const int col = (row & 192) + 32 * (rho >> 5) + 8 * ((rho & 15) >> 2) + 4 * ((rho >> 4) & 1) + (rho & 3);
-        boff[i] = (uint32_t)min(n0 + col, N - 1) * (uint32_t)K + chunk;
+        const int wrow = SWIGLU ? (col < 128 ? n0 + col : I_half + n0 + col - 128) : min(n0 + col, N - 1);
+        boff[i] = (uint32_t)wrow * (uint32_t)K + chunk;
     }
     const uint32_t soff = (uint32_t)min(m_start + min((wave & 3) * 64 + lane, W_BM - 1), m_end - 1) * (uint32_t)KT_all * (AS16 ? 2u : 4u);
     // (AS16: 16-bit activation scales staged as they are, see gemm_dma_kernel)
@@ -345,7 +355,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     if constexpr (SCALED) {
         for (int i = tid; i < 2 * KT; i += W_THREADS) {
             const int c = i >= KT ? 1 : 0, kk = i - c * KT;
-            const int64_t blk = min(bx * 2 + c, nblk - 1);
+            const int64_t blk = SWIGLU ? (c ? (I_half >> 7) + bx : bx) : min(bx * 2 + c, nblk - 1);
             bsl[c * D_MAX_KT + kk] = ld_scale(p.b_s, bs_off + blk * KT_all + kt0 + kk, p.s_dtype);
         }
     }
@@ -379,6 +389,7 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
     const int esz = p.c_dtype == LLMK_F32 ? 4 : 2;
     const bool vec_ok = ((((uintptr_t)p.c) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
     auto store_row = [&](int i) {
+        if constexpr (SWIGLU) return;        // nothing is stored before the epilogue below
         const int m = m_start + wm * 16 * R + 16 * i + r;
         if (m >= m_end) return;
         if constexpr (KIND != K_I8_ROWCOL) {
@@ -527,6 +538,99 @@ __global__ __launch_bounds__(W_THREADS) void gemm_wide_kernel(DirectArgs p) {
         run(std::integral_constant<int, R>{});
     }
 
+    if constexpr (SWIGLU) {
+        // ---- gated activation + 1 x 128 quantiser.  Waves wn = 0, 1 hold the gate columns of the wave's 16 R rows, waves
+        // wn = 2, 3 the up columns of the same rows, same lane and register for the same (row, column).  The pair (wn,
+        // wn + 2) splits the rows: the gate wave finishes tile rows 0 .. R/2 - 1, the up wave rows R/2 .. R - 1, after each
+        // has passed the other its half through LDS (16-bit values, as the GEMM would have stored them).  A group of
+        // 128 outputs of a row lies in two waves (wn & 1), whose row maxima meet in LDS.
+        constexpr int RH = R / 2;
+        constexpr bool FP8Q = (KIND == K_FP8_BLOCK);
+        uint8_t* const xch = lds;                                        // [wave][RH][2][64 lanes] x 16 bytes
+        float* const rowmax = (float*)(lds + 8 * RH * 2 * 1024);         // [wm][half][wn & 1][16 RH rows]
+        const int half = wn >> 1, w1 = wn & 1;
+        const int gcols = I_half >> 7;                                   // scale groups per output row
+        auto pack8 = [&](const v4f& x, const v4f& y) {
+            v4i w;
+            if (p.c_dtype == LLMK_F16) {
+                w[0] = (int)pack_f16x2(x[0], x[1]); w[1] = (int)pack_f16x2(x[2], x[3]);
+                w[2] = (int)pack_f16x2(y[0], y[1]); w[3] = (int)pack_f16x2(y[2], y[3]);
+            } else {
+                w[0] = (int)pack_bf16x2(x[0], x[1]); w[1] = (int)pack_bf16x2(x[2], x[3]);
+                w[2] = (int)pack_bf16x2(y[0], y[1]); w[3] = (int)pack_bf16x2(y[2], y[3]);
+            }
+            return w;
+        };
+        auto epilogue = [&](auto half_c, auto idt_c) {
+            constexpr int HALF = decltype(half_c)::value, IDT = decltype(idt_c)::value;
+            constexpr int OWN = RH * HALF, OTH = RH * (1 - HALF);
+            __syncthreads();                                             // every wave is done with the stages
+            {
+                uint8_t* dst = xch + (uint32_t)(wave * RH * 2) * 1024u + (uint32_t)lane * 16u;
+#pragma unroll
+                for (int i = 0; i < RH; ++i)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) *(v4i*)(dst + (i * 2 + h) * 1024) = pack8(acc[OTH + i][2 * h], acc[OTH + i][2 * h + 1]);
+            }
+            __syncthreads();
+            // partner: same wm and wn & 1, other half
+            const int partner = wm * 4 + (1 - HALF) * 2 + w1;
+            const uint8_t* src = xch + (uint32_t)(partner * RH * 2) * 1024u + (uint32_t)lane * 16u;
+            float y[RH][2][EPL], mx[RH];
+#pragma unroll
+            for (int i = 0; i < RH; ++i) {
+                float m = 0.f;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    float other[EPL], own[EPL];
+                    const v4i wo = *(const v4i*)(src + (i * 2 + h) * 1024);
+                    const v4i wm_ = pack8(acc[OWN + i][2 * h], acc[OWN + i][2 * h + 1]);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const unsigned a = (unsigned)wo[q], b = (unsigned)wm_[q];
+                        if constexpr (IDT == LLMK_F16) {
+                            other[2 * q] = f16_to_f32((unsigned short)a); other[2 * q + 1] = f16_to_f32((unsigned short)(a >> 16));
+                            own[2 * q] = f16_to_f32((unsigned short)b); own[2 * q + 1] = f16_to_f32((unsigned short)(b >> 16));
+                        } else {
+                            other[2 * q] = bf16_to_f32((unsigned short)a); other[2 * q + 1] = bf16_to_f32((unsigned short)(a >> 16));
+                            own[2 * q] = bf16_to_f32((unsigned short)b); own[2 * q + 1] = bf16_to_f32((unsigned short)(b >> 16));
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < EPL; ++q) {
+                        const float gv = HALF == 0 ? own[q] : other[q], up = HALF == 0 ? other[q] : own[q];
+                        y[i][h][q] = gated_act<IDT>(gv, up, p.act, false, 1.0f);
+                        m = fmaxf(m, fabsf(y[i][h][q]));
+                    }
+                }
+                m = fmaxf(m, __shfl_xor(m, 16, 64));
+                m = fmaxf(m, __shfl_xor(m, 32, 64));
+                mx[i] = m;
+                if (g == 0) rowmax[((wm * 2 + HALF) * 2 + w1) * (16 * RH) + 16 * i + r] = m;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < RH; ++i) {
+                const float m = fmaxf(mx[i], rowmax[((wm * 2 + HALF) * 2 + (1 - w1)) * (16 * RH) + 16 * i + r]);
+                const int row = m_start + wm * 16 * R + 16 * (OWN + i) + r;
+                if (row >= m_end) continue;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int col = n0 + 64 * w1 + 32 * h + 8 * g;
+                    quant_store8<FP8Q>(y[i][h], m, p.c, (int64_t)row * I_half + col, p.q_scale, (int64_t)row * gcols + bx,
+                                       w1 == 0 && g == 0 && h == 0, p.round_mode);
+                }
+            }
+        };
+        const std::integral_constant<int, 0> h0;
+        const std::integral_constant<int, 1> h1;
+        const std::integral_constant<int, LLMK_F16> tf16;
+        const std::integral_constant<int, LLMK_BF16> tbf16;
+        if (p.c_dtype == LLMK_F16) { if (half == 0) epilogue(h0, tf16); else epilogue(h1, tf16); }
+        else { if (half == 0) epilogue(h0, tbf16); else epilogue(h1, tbf16); }
+        return;
+    }
+
     // ---- epilogue: the rows not yet stored by the last K step
     if (KT > 0) store_row(R - 1);
     else {
@@ -608,6 +712,22 @@ int launch_wide(const DirectArgs& p0, hipStream_t stream, const char* name, void
         wide_tail_sum_kernel<GROUPED, R><<<dim3(LLMK_CUS / 2, W_BM / 32), 256, 0, stream>>>(p, ESZ);
         LLMK_CHECK_LAUNCH(name);
     }
+    return LLMK_OK;
+}
+
+// The gated-activation form of the kernel (grouped gate / up projection, p.N = 2 I, I % 128 == 0): one column tile per
+// 128 gate columns; no split of the last round (its tiles would have to meet before the activation).
+template <int KIND, int R>
+int launch_wide_swiglu(const DirectArgs& p, hipStream_t stream, const char* name) {
+    static std::atomic<uint64_t> configured{0};
+    auto kern = gemm_wide_kernel<KIND, true, R, true>;
+    constexpr int W_BM = w_bm(R), W_LDS = w_lds(R);
+    static_assert(8 * (R / 2) * 2 * 1024 + 2 * 2 * 2 * 16 * (R / 2) * 4 <= W_LDS, "exchange area and row maxima fit in the stages");
+    if (int rc = llmk_reserve_lds((const void*)kern, W_LDS, configured, name)) return rc;
+    dim3 grid((unsigned)((p.N / 2) / 128), (unsigned)grouped_row_tiles(p.M, p.E, W_BM));
+    if (grid.x == 0 || grid.y == 0) return LLMK_OK;
+    kern<<<grid, W_THREADS, W_LDS, stream>>>(p);
+    LLMK_CHECK_LAUNCH(name);
     return LLMK_OK;
 }
 

@@ -152,43 +152,9 @@ __global__ void pre_reorder_kernel(const void* __restrict__ x, void* __restrict_
     }
 }
 
-// round-trip through the storage type: the reference multiplies in the tensor dtype
-template <int DT> __device__ __forceinline__ float rnd(float v) {
-    if constexpr (DT == LLMK_F16) return f16_to_f32(f32_to_f16(v));
-    else if constexpr (DT == LLMK_BF16) return bf16_to_f32(f32_to_bf16(v));
-    else return v;
-}
-
 // groups per thread of the fused activation + quantisation kernel (8192 x 28672 bf16 -> e4m3: 121 us with 1,
 // 117 us with 2, 131 us with 4, 146 us with 8)
 constexpr int AMQ_UNROLL = 2;
-
-// 1 / (1 + e^-x).  For 16-bit tensors the result is rounded to 8 or 11 significant bits right after, so the
-// hardware exp2 and reciprocal (1 ulp each in fp32) are used: large |x| gives exp2 -> inf or 0 and the
-// quotient 0 or 1, as the exact expression does.  fp32 tensors keep the library routines.
-template <int IDT>
-__device__ __forceinline__ float sigmoid_f(float x) {
-    if constexpr (IDT == LLMK_F32) return 1.0f / (1.0f + expf(-x));
-    else return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
-}
-
-// gated activation of one element with the reference's rounding points (activation in fp32, rounded to the
-// tensor dtype, product in the tensor dtype, optional per-expert scale in the tensor dtype)
-template <int IDT>
-__device__ __forceinline__ float gated_act(float gv, float up, int act, bool has_scale, float scale) {
-    if (act == 0) {
-        gv = gv * sigmoid_f<IDT>(gv);
-    } else {
-        const float kAlpha = 0.7978845608028654f;
-        const float u = kAlpha * (gv + 0.044715f * gv * gv * gv);
-        const float th = 2.0f * sigmoid_f<IDT>(2.0f * u) - 1.0f;
-        gv = 0.5f * gv * (1.0f + th);
-    }
-    gv = rnd<IDT>(gv);
-    float r = rnd<IDT>(gv * up);
-    if (has_scale) r = rnd<IDT>(r * scale);
-    return r;
-}
 
 template <int IDT, int ODT>
 __global__ void act_and_mul_kernel(const void* __restrict__ gateup, void* __restrict__ out,
@@ -538,4 +504,61 @@ extern "C" int llmk_grouped_gemm(const void* a, const void* b, void* c, int kind
         case LLMK_KIND_BF16: return launch_direct<K_BF16, true>(p, (int)M, st, "grouped_gemm(bf16)");
         default: LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm: kind %d", kind);
     }
+}
+
+// which tile kernel the gated-activation form would run on for this shape: 8 / 4 = tile rows per wave of the 256-column
+// kernel, 0 = none (the caller runs the grouped GEMM and the activation kernel instead)
+static int swiglu_tile_rows(int kind, const DirectArgs& p) {
+    if (p.N % 256 || p.K % 128 || !dma_eligible(p)) return 0;
+    const bool big = p.M > 64 * (int64_t)p.E || (p.M > 2 * (int64_t)p.E && (int64_t)p.N * p.K >= ((int64_t)20 << 20)) ||
+                     grouped_row_tiles(p.M, p.E, 16) >= 6;
+    if (!big) return 0;
+    const int choice = kind == LLMK_KIND_FP8 ? dma_tile_choice<K_FP8_BLOCK, true>(p) : dma_tile_choice<K_I8_BLOCK, true>(p);
+    return choice == 8 ? 8 : (choice == 9 ? 4 : 0);
+}
+
+extern "C" int llmk_grouped_gemm_swiglu_quant_fused(int kind, int E, int64_t M, int64_t two_i, int64_t K) {
+    if ((kind != LLMK_KIND_I8 && kind != LLMK_KIND_FP8) || E <= 0 || M <= 0 || two_i <= 0 || K <= 0) return 0;
+    if (M > 0x7fffffff || two_i > 0x7fffffff || K > 0x7fffffff) return 0;
+    DirectArgs p{};
+    p.M = (int)M; p.N = (int)two_i; p.K = (int)K; p.E = E;
+    return swiglu_tile_rows(kind, p) ? 1 : 0;
+}
+
+extern "C" int llmk_grouped_gemm_swiglu_quant(const void* a, const void* b, void* q_out, void* s_out, int kind, int mid_dtype,
+                                              int round_mode, int E, int64_t M, int64_t two_i, int64_t K,
+                                              const int64_t* seg_indptr, const int64_t* weight_indices, const void* scale_a,
+                                              const void* scale_b, int s_dtype, int act, void* workspace,
+                                              int64_t workspace_bytes, void* stream) {
+    if (M < 0 || two_i < 0 || K < 0 || E < 0) LLMK_FAIL(LLMK_ERR_SHAPE, "grouped_gemm_swiglu_quant: negative dimension");
+    if (kind != LLMK_KIND_I8 && kind != LLMK_KIND_FP8) LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm_swiglu_quant: kind %d", kind);
+    if (mid_dtype != LLMK_F16 && mid_dtype != LLMK_BF16) LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm_swiglu_quant: mid_dtype %d (the dtype the gate / up sums are rounded to: fp16 or bf16)", mid_dtype);
+    if (act != 0 && act != 1) LLMK_FAIL(LLMK_ERR_ARG, "grouped_gemm_swiglu_quant: act %d", act);
+    if (round_mode != LLMK_ROUND_HALF_AWAY && round_mode != LLMK_ROUND_HALF_UP) LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm_swiglu_quant: round_mode %d", round_mode);
+    if (M > 0x7fffffff || two_i > 0x7fffffff || K > 0x7fffffff) LLMK_FAIL(LLMK_ERR_SHAPE, "grouped_gemm_swiglu_quant: dimension exceeds int32");
+    if (M == 0 || two_i == 0 || E == 0) return LLMK_OK;
+    if (!a || !b || !q_out || !s_out || !seg_indptr || !scale_a || !scale_b) LLMK_FAIL(LLMK_ERR_ARG, "grouped_gemm_swiglu_quant: null pointer");
+    if ((((uintptr_t)a) | ((uintptr_t)b)) & 15 || ((uintptr_t)q_out & 7)) LLMK_FAIL(LLMK_ERR_ARG, "grouped_gemm_swiglu_quant: operands must be 16-byte aligned, q_out 8-byte aligned");
+    DirectArgs p{};
+    p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.c = q_out; p.q_scale = s_out; p.a_s = scale_a; p.b_s = scale_b;
+    p.seg_indptr = seg_indptr; p.weight_indices = weight_indices;
+    p.c_dtype = mid_dtype; p.s_dtype = s_dtype; p.M = (int)M; p.N = (int)two_i; p.K = (int)K; p.E = E;
+    p.act = act; p.round_mode = round_mode;
+    const int rows = swiglu_tile_rows(kind, p);
+    if (!rows) LLMK_FAIL(LLMK_ERR_SHAPE, "grouped_gemm_swiglu_quant: shape E=%d M=%lld 2I=%lld K=%lld is not one the fused kernel takes (ask llmk_grouped_gemm_swiglu_quant_fused first)", E, (long long)M, (long long)two_i, (long long)K);
+    hipStream_t st = (hipStream_t)stream;
+    if (s_dtype != LLMK_F32) {
+        // 16-bit activation scales are widened first, as in front of the plain kernel
+        const int64_t n = M * (K >> 7);
+        if (!workspace || workspace_bytes < n * 4 || ((uintptr_t)workspace & 15)) LLMK_FAIL(LLMK_ERR_ARG, "grouped_gemm_swiglu_quant: 16-bit activation scales need %lld bytes of workspace", (long long)(n * 4));
+        const unsigned blocks = (unsigned)cdiv64(n, 256);
+        if (s_dtype == LLMK_F16) scales_to_f32_kernel<LLMK_F16><<<blocks, 256, 0, st>>>(scale_a, (float*)workspace, n);
+        else if (s_dtype == LLMK_BF16) scales_to_f32_kernel<LLMK_BF16><<<blocks, 256, 0, st>>>(scale_a, (float*)workspace, n);
+        else LLMK_FAIL(LLMK_ERR_DTYPE, "grouped_gemm_swiglu_quant: s_dtype %d", s_dtype);
+        LLMK_CHECK_LAUNCH("grouped_gemm_swiglu_quant(scales)");
+        p.a_s = workspace;
+    }
+    if (kind == LLMK_KIND_FP8)
+        return rows == 8 ? launch_wide_swiglu<K_FP8_BLOCK, 8>(p, st, "grouped_gemm_swiglu_quant(fp8)") : launch_wide_swiglu<K_FP8_BLOCK, 4>(p, st, "grouped_gemm_swiglu_quant(fp8)");
+    return rows == 8 ? launch_wide_swiglu<K_I8_BLOCK, 8>(p, st, "grouped_gemm_swiglu_quant(i8)") : launch_wide_swiglu<K_I8_BLOCK, 4>(p, st, "grouped_gemm_swiglu_quant(i8)");
 }

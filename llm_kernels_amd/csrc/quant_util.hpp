@@ -107,4 +107,38 @@ __device__ __forceinline__ void quant_store8(const float (&v)[EPL], float m, voi
     }
 }
 
+// round-trip through the storage type: the reference multiplies in the tensor dtype
+template <int DT> __device__ __forceinline__ float rnd(float v) {
+    if constexpr (DT == LLMK_F16) return f16_to_f32(f32_to_f16(v));
+    else if constexpr (DT == LLMK_BF16) return bf16_to_f32(f32_to_bf16(v));
+    else return v;
+}
+
+// 1 / (1 + e^-x).  For 16-bit tensors the result is rounded to 8 or 11 significant bits right after, so the
+// hardware exp2 and reciprocal (1 ulp each in fp32) are used: large |x| gives exp2 -> inf or 0 and the
+// quotient 0 or 1, as the exact expression does.  fp32 tensors keep the library routines.
+template <int IDT>
+__device__ __forceinline__ float sigmoid_f(float x) {
+    if constexpr (IDT == LLMK_F32) return 1.0f / (1.0f + expf(-x));
+    else return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+
+// gated activation of one element with the reference's rounding points (activation in fp32, rounded to the
+// tensor dtype, product in the tensor dtype, optional per-expert scale in the tensor dtype)
+template <int IDT>
+__device__ __forceinline__ float gated_act(float gv, float up, int act, bool has_scale, float scale) {
+    if (act == 0) {
+        gv = gv * sigmoid_f<IDT>(gv);
+    } else {
+        const float kAlpha = 0.7978845608028654f;
+        const float u = kAlpha * (gv + 0.044715f * gv * gv * gv);
+        const float th = 2.0f * sigmoid_f<IDT>(2.0f * u) - 1.0f;
+        gv = 0.5f * gv * (1.0f + th);
+    }
+    gv = rnd<IDT>(gv);
+    float r = rnd<IDT>(gv * up);
+    if (has_scale) r = rnd<IDT>(r * scale);
+    return r;
+}
+
 }  // namespace

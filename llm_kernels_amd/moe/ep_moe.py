@@ -13,7 +13,8 @@ import torch
 from torch import nn
 
 from .group_gemm_kernel import (grouped_gemm_triton, post_reorder, pre_reorder, run_moe_ep_preproess,
-                                silu_and_mul, gelu_and_mul, pre_reorder_quant, act_and_mul_quant)
+                                silu_and_mul, gelu_and_mul, pre_reorder_quant, act_and_mul_quant,
+                                grouped_gemm_swiglu_quant, grouped_gemm_swiglu_quant_fused)
 
 
 def softmax_topk_router(router_logits: torch.Tensor, top_k: int = 2, renormalize: bool = True):
@@ -70,12 +71,21 @@ def ep_moe_forward(hidden_states: torch.Tensor, topk_ids: torch.Tensor, topk_wei
     else:
         gateup_input, a1_s = torch.empty((T * top_k, H), device=dev, dtype=dt), None
         pre_reorder(hidden_states, gateup_input, src2dst, topk_ids, None, start_expert_id, end_expert_id, top_k, H)
-    gateup_output = torch.empty(gateup_input.shape[0], w13_weight.shape[1], device=dev, dtype=dt)
-    grouped_gemm_triton(a=gateup_input, b=w13_weight, c=gateup_output, batch_size=E, weight_column_major=True,
-                        seg_indptr=seg_cur, weight_indices=widx, use_fp8_w8a8=False, scale_a=a1_s,
-                        scale_b=w13_weight_scale, block_shape=block_shape)
+    # large launches: the gated activation and the quantiser of the down projection run in the epilogue of the gate / up
+    # GEMM (same bits, the [rows, 2I] tensor is never written)
+    one_kernel = fused and w2_weight.dtype == w13_weight.dtype and grouped_gemm_swiglu_quant_fused(gateup_input, w13_weight, E)
+    if one_kernel:
+        down_input, a2_s = grouped_gemm_swiglu_quant(gateup_input, a1_s, w13_weight, w13_weight_scale, E, seg_cur, widx, dt,
+                                                     activation)
+    else:
+        gateup_output = torch.empty(gateup_input.shape[0], w13_weight.shape[1], device=dev, dtype=dt)
+        grouped_gemm_triton(a=gateup_input, b=w13_weight, c=gateup_output, batch_size=E, weight_column_major=True,
+                            seg_indptr=seg_cur, weight_indices=widx, use_fp8_w8a8=False, scale_a=a1_s,
+                            scale_b=w13_weight_scale, block_shape=block_shape)
 
-    if fused:
+    if one_kernel:
+        pass
+    elif fused:
         down_input, a2_s = act_and_mul_quant(gateup_output, gateup_output.shape[1], reorder_topk_ids, None,
                                              start_expert_id, end_expert_id, w2_weight.dtype, activation)
     else:

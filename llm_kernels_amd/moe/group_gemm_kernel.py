@@ -158,6 +158,44 @@ def act_and_mul_quant(gateup_output, hidden_size, reorder_topk_ids, scales, star
     return q, s
 
 
+def grouped_gemm_swiglu_quant_fused(a, b, batch_size):
+    """True when `grouped_gemm_swiglu_quant` runs this gate / up projection in one kernel (shapes that the 256-column
+    tile kernel takes); otherwise run grouped_gemm_triton and act_and_mul_quant."""
+    kind = {torch.int8: _lib.KIND_I8, torch.float8_e4m3fn: _lib.KIND_FP8}.get(b.dtype)
+    if kind is None or a.dtype != b.dtype or b.dim() != 3:
+        return False
+    return bool(_lib.load().llmk_grouped_gemm_swiglu_quant_fused(kind, int(batch_size), a.shape[0], b.shape[1], b.shape[2]))
+
+
+def grouped_gemm_swiglu_quant(a, scale_a, b, scale_b, batch_size, seg_indptr, weight_indices, mid_dtype, activation="silu"):
+    """Gate / up projection of a gated MLP over expert segments with the gated activation and the 1 x 128 quantiser of
+    the down projection in the GEMM's epilogue: equal bit for bit to
+    act_and_mul_quant(grouped_gemm_triton(a, b, c of `mid_dtype`, ...)), without the [M, 2I] tensor (the reference runs
+    the three kernels one after the other, sglang_moe_all_gather_all_reduce.py:330-408).  a [M, K] and b [E, 2I, K]
+    int8 or float8_e4m3fn with 1 x 128 / 128 x 128 block scales.  Returns (q [M, I], s [M, I/128]); rows outside every
+    segment are left unwritten.  Only for shapes for which grouped_gemm_swiglu_quant_fused() is true."""
+    _lib.require_gpu(a, b, scale_a, scale_b, seg_indptr)
+    assert a.is_contiguous() and b.is_contiguous() and a.dtype == b.dtype and b.dim() == 3 and a.shape[-1] == b.shape[-1]
+    assert mid_dtype in (torch.float16, torch.bfloat16)
+    M, two_i, K = a.shape[0], b.shape[1], b.shape[2]
+    q, s, kind, mode = _quant_buffers(M, two_i // 2, b.dtype, a.device)
+    scale_a, scale_b = scale_a.contiguous(), scale_b.contiguous()
+    if scale_b.dtype != scale_a.dtype:
+        scale_b = scale_b.to(scale_a.dtype)
+    seg = (seg_indptr if seg_indptr.dtype == torch.int64 else seg_indptr.to(torch.int64)).contiguous()
+    wi = None
+    if weight_indices is not None:
+        wi = (weight_indices if weight_indices.dtype == torch.int64 else weight_indices.to(torch.int64)).contiguous()
+    ws, ws_bytes = None, 0
+    if scale_a.dtype != torch.float32:
+        ws_bytes = M * (K // 128) * 4
+        ws = _lib.ptr(_lib.workspace(a.device, ws_bytes))
+    _lib.call("llmk_grouped_gemm_swiglu_quant", _lib.ptr(a), _lib.ptr(b), _lib.ptr(q), _lib.ptr(s), kind, _lib.dt(mid_dtype),
+              mode, int(batch_size), M, two_i, K, _lib.ptr(seg), _lib.ptr(wi), _lib.ptr(scale_a), _lib.ptr(scale_b),
+              _lib.dt(scale_a.dtype), {"silu": 0, "gelu": 1}[activation], ws, ws_bytes, _lib.stream(a), exc=AssertionError)
+    return q, s
+
+
 class _GridCall:
     """Accepts `obj[grid](*args, BLOCK_SIZE=...)`; the grid and the tile size are chosen by the HIP launcher."""
 

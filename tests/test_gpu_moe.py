@@ -508,6 +508,52 @@ def test_ep_moe_forward_fused_equals_unfused(dev, kind):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("qdt", [torch.float8_e4m3fn, torch.int8])
+@pytest.mark.parametrize("dtype,act", [(torch.bfloat16, "silu"), (torch.float16, "gelu")])
+@pytest.mark.parametrize("rows,two_i,K", [(8000, 4096, 256), (4800, 4096, 256), (8000, 3840, 384)])
+def test_gate_up_gemm_with_activation_epilogue_equals_three_kernels(dev, qdt, dtype, act, rows, two_i, K):
+    """grouped_gemm_swiglu_quant == act_and_mul_quant(grouped_gemm_triton(...)) bit for bit, values and scales, on shapes
+    that the dispatch gives to the 256-row (8000 rows) and 128-row (4800 rows) tiles of the large grouped kernel: a
+    number of column tiles that is and is not a multiple of the XCD count, one empty segment, one shorter than a tile,
+    ragged ends, permuted weight indices, rows behind the last segment untouched."""
+    announce("gate/up + activation epilogue", qdt, dtype, act, rows, two_i, K)
+    E = 8
+    torch.manual_seed(rows + two_i)
+    used = rows - 5
+    cuts = sorted(torch.randint(0, used, (E - 3,)).tolist())
+    seg = torch.tensor([0, 37, 37] + cuts + [used], dtype=torch.int64, device=dev)     # segment 0: 37 rows, segment 1: empty
+    widx = torch.randperm(E).to(dev)
+    act_quant = fp8_kernel.act_quant if qdt == torch.float8_e4m3fn else int8_kernel.act_quant
+    wq = fp8_kernel.weight_quant if qdt == torch.float8_e4m3fn else int8_kernel.weight_quant
+    a, a_s = act_quant((torch.randn(rows, K) * 2).to(dtype).to(dev))
+    ws = [wq((torch.randn(two_i, K) * 0.3).to(dev)) for _ in range(E)]
+    b = torch.stack([t[0].view(torch.uint8) for t in ws]).view(qdt)
+    b_s = torch.stack([t[1] for t in ws])
+    assert gk.grouped_gemm_swiglu_quant_fused(a, b, E)
+    q1, s1 = gk.grouped_gemm_swiglu_quant(a, a_s, b, b_s, E, seg, widx, dtype, act)
+
+    c = torch.zeros(rows, two_i, dtype=dtype, device=dev)
+    gk.grouped_gemm_triton(a=a, b=b, c=c, batch_size=E, weight_column_major=True, seg_indptr=seg, weight_indices=widx,
+                           scale_a=a_s, scale_b=b_s, block_shape=[128, 128])
+    ids = torch.zeros(rows, dtype=torch.int64, device=dev)
+    q0, s0 = gk.act_and_mul_quant(c, two_i, ids, None, 0, E - 1, qdt, act)
+    assert q1.shape == q0.shape and s1.shape == s0.shape and s1.dtype == s0.dtype
+    assert torch.equal(s1[:used].cpu(), s0[:used].cpu())
+    assert torch.equal(q1[:used].view(torch.uint8).cpu(), q0[:used].view(torch.uint8).cpu())
+    assert float(s0[:used].float().abs().max()) > 0
+
+
+def test_gate_up_activation_epilogue_refuses_small_shapes(dev):
+    """Shapes that run on the smaller tile kernels are not taken: the query says so and the entry point fails."""
+    a = torch.zeros(64, 256, dtype=torch.int8, device=dev)
+    b = torch.zeros(4, 512, 256, dtype=torch.int8, device=dev)
+    assert not gk.grouped_gemm_swiglu_quant_fused(a, b, 4)
+    seg = torch.tensor([0, 16, 32, 48, 64], dtype=torch.int64, device=dev)
+    with pytest.raises(AssertionError, match="not one the fused kernel takes"):
+        gk.grouped_gemm_swiglu_quant(a, torch.ones(64, 2, dtype=torch.float16, device=dev), b,
+                                     torch.ones(4, 4, 2, dtype=torch.float16, device=dev), 4, seg, None, torch.bfloat16)
+
+
 def test_grouped_gemm_per_expert_scalar_scales(dev):
     """use_fp8_w8a8 without block_shape: c = (a . b^T) * scale_a[e] * scale_b[e] (reference :417-420, commented out there)."""
     announce("grouped gemm per-expert scales")
