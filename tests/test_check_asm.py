@@ -58,6 +58,15 @@ def test_rejects_spills_in_kernels_with_such_loads(tmp_path):
     assert n == 1 and len(bad) == 1 and "spilled" in bad[0]
 
 
+def test_rejects_spills_in_any_kernel(tmp_path):
+    p = os.path.join(tmp_path, "k.s")
+    with open(p, "w") as f:
+        f.write(HEAD + "\tv_mov_b32_e32 v4, v10\n\ts_endpgm\n"
+                "amdhsa.kernels:\n  - .name:           kern\n    .private_segment_fixed_size: 472\n    .vgpr_spill_count: 0\n")
+    n, bad = check_asm.check_file(p)
+    assert n == 0 and len(bad) == 1 and "scratch" in bad[0]
+
+
 WAIT = "\ts_waitcnt vmcnt(0)\n"
 
 
