@@ -70,15 +70,28 @@ __device__ __forceinline__ WideTile wide_tile_of(const DirectArgs& p, int lin, i
         int64_t s0 = p.seg_indptr[0];
         if (gx % 8 == 0) {
             // XCD x (workgroup id mod 8) owns the column tiles x, x + 8, ...; it walks them segment by
-            // segment, and for every column tile all row tiles of the segment back to back, so the workgroups
-            // that share a weight tile run at the same time on the L2 that holds it.
+            // segment, and for every column tile the row tiles of the segment back to back, so the workgroups
+            // that share a weight tile run at the same time on the L2 that holds it.  Long segments go in strips of
+            // four row tiles (the last strip takes what is left, one to five), each strip across all column tiles
+            // of the XCD: its 32 concurrent workgroups then share 8 weight tiles and 4 activation tiles, where one
+            // column tile x 32 row tiles would pull 33 operand tiles per K step through the L2 instead of 12.
             const int x = lin & 7, cx = gx >> 3;
             int s = lin >> 3;
             for (; e < p.E; ++e) {
                 const int64_t s1 = p.seg_indptr[e + 1];
                 const int tl = (int)((s1 - s0 + W_BM - 1) / W_BM);
                 if (s < tl * cx) {
-                    const int bl = s / tl, rt = s - bl * tl;
+                    const int full = max(1, (tl + 2) >> 2) - 1;          // strips of four in front of the last one
+                    int bl, rt;
+                    if (s < 4 * cx * full) {
+                        const int st = s / (4 * cx), r4 = s - st * 4 * cx;
+                        bl = r4 >> 2;
+                        rt = 4 * st + (r4 & 3);
+                    } else {
+                        const int r4 = s - 4 * cx * full, h = tl - 4 * full;
+                        bl = r4 / h;
+                        rt = 4 * full + (r4 - bl * h);
+                    }
                     t.found = true;
                     t.bx = bl * 8 + x;
                     t.m_start = (int)s0 + rt * W_BM;
