@@ -905,7 +905,15 @@ template <int KIND, bool GROUPED>
 int launch_big_half(DirectArgs p, hipStream_t stream, const char* name, void* workspace = nullptr, int64_t workspace_bytes = 0) {
     if (!dma_eligible(p, 2)) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: shape not supported by the tiled half-precision kernel", name);
     if constexpr (!GROUPED) {
-        const int z = splitk_factor_half(p.M, p.N, p.K);
+        int z = splitk_factor_half(p.M, p.N, p.K);
+        if constexpr (KIND == K_W4MARLIN) {
+            // a round of 64-row tiles costs this kind 44 us at K = 4096 whatever its width (the scatter of the Marlin
+            // layout), so the slices must not open a second round: at most 256 / tiles of them (128 x 14336 x 4096:
+            // 51.9 us in two slices, 44.0 unsplit; 256 x 6144 x 4096 51.1 -> 43.9; 128 x 8192 x 4096 keeps two: 30.2 vs 43.5)
+            const int64_t tiles = (((int64_t)p.M + 63) / 64) * (((int64_t)p.N + 127) / 128);
+            const int zmax = (int)(LLMK_CUS / tiles > 1 ? LLMK_CUS / tiles : 1);
+            if (z > zmax) z = zmax;
+        }
         if (z > 1 && workspace && workspace_bytes >= (int64_t)z * p.M * p.N * 4 && !(((uintptr_t)workspace) & 15)) {
             p.partial = (float*)workspace;
             p.ksplit = z;
