@@ -89,11 +89,11 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
     const int n0 = blockIdx.x * MD_BN, m_start = blockIdx.y * BM, m_end = min(p.M, m_start + BM);
 
     // LDS map
-    uint8_t* const a_st = lds;                              // [3][MD_A]
-    uint8_t* const b_st = lds + MD_NA * MD_A;               // [MD_B]
-    uint8_t* const s_st = lds + MD_NA * MD_A + MD_NBS * MD_B;        // [3][MD_S]
+    uint8_t* const a_st = lds;                              // [MD_NA][MD_A]
+    uint8_t* const b_st = lds + MD_NA * MD_A;               // [MD_NBS][MD_B]
+    uint8_t* const s_st = lds + MD_NA * MD_A + MD_NBS * MD_B;        // [MD_NA][MD_S]
     float* const bsl = (float*)(lds + md_stages(MT));       // weight scale of the tile's column block per sub-block
-    uint8_t* const w4tab = lds + md_stages(MT) + D_MAX_KT * 4;   // K_W4A8: [s4 | z4][sub-block][64 rows] bytes
+    uint8_t* const w4tab = lds + md_stages(MT) + D_MAX_KT * 4;   // [s4 | z4][sub-block][64 rows] bytes
 
     // ---- per-thread source offsets.  A piece = 8 rows x 128 bytes = what one load instruction of a wave covers
     // (lane: row lane >> 3, 16-byte chunk lane & 7, XOR-swizzled with (row >> 1) & 7 on the global side so that
