@@ -59,7 +59,7 @@ static int64_t workspace_core_bytes(int64_t M, int64_t N, int64_t K) {
     }
     const int64_t scales = (M * (K / 128) * 4 + 255) & ~(int64_t)255;
     int z = splitk_factor(M, N, K);
-    if (M <= 512) z = std::max(z, mid_plan(M, N, K).z);      // the mid-size kernel's K slices
+    if (M <= 512) z = std::max({z, mid_plan(M, N, K).z, midw_plan(M, N, K).z});      // the mid-size kernels' K slices
     return scales + (z > 1 ? (int64_t)z * M * N * 4 : 0);
 }
 

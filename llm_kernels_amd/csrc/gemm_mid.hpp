@@ -313,13 +313,24 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_kernel(DirectArgs p) {
 //       (4 MT matrix instructions for MT + 4 fragment reads) and never touches global memory inside the loop.
 // Two stages (activations | weights | activation-scale column); one barrier per step, after which the stage just filled
 // is complete and the one just multiplied is free.  The four sub-block sums meet in LDS at the end as before.
+// WIDE: the same roles on a 16 MT x 128 tile with K steps of 256 bytes = two sub-blocks (MT = 4 or 8), for weights with
+// more 64-column tiles than CUs: producer 4 + q moves sub-block q & 1 of the step for the row half and the column half
+// q >> 1, consumer q multiplies sub-block q & 1 for the column half q >> 1; two partial sums per output meet at the end.
 constexpr int MDP_RB = 3;
-constexpr int mdp_stage(int mt) { return md_a(mt) + MD_B + MD_S; }
-constexpr int mdp_lds(int mt) { return (2 * mdp_stage(mt) > md_red(mt) ? 2 * mdp_stage(mt) : md_red(mt)) + D_MAX_KT * 4; }
+constexpr int mdp_bn(bool wide) { return wide ? 128 : 64; }
+constexpr int mdp_nsub(bool wide) { return wide ? 2 : 4; }                       // 128-byte sub-blocks per K step
+constexpr int mdp_a(int mt, bool wide) { return mdp_nsub(wide) * 16 * mt * 128; }
+constexpr int mdp_stage(int mt, bool wide = false) { return mdp_a(mt, wide) + MD_B + MD_S; }
+constexpr int mdp_red(int mt, bool wide) { return mdp_nsub(wide) * 16 * mt * (mdp_bn(wide) + 4) * 4; }
+constexpr int mdp_lds(int mt, bool wide = false) {
+    return (2 * mdp_stage(mt, wide) > mdp_red(mt, wide) ? 2 * mdp_stage(mt, wide) : mdp_red(mt, wide)) + D_MAX_KT * 4;
+}
 
-template <int KIND, int MT, bool AS16 = false>
+template <int KIND, int MT, bool AS16 = false, bool WIDE = false>
 __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
-    static_assert(MT == 4 || MT == 2, "tile rows");
+    static_assert(WIDE ? (MT == 8 || MT == 4) : (MT == 4 || MT == 2), "tile rows");
+    constexpr int BN = mdp_bn(WIDE), NSUB = mdp_nsub(WIDE), RED_ROW = BN + 4;
+    static_assert(BN * NSUB * 128 == MD_B && RED_ROW == (WIDE ? 132 : MD_RED_ROW), "weight stage of 32 KB");
     static_assert(KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK || KIND == K_I8_ROWCOL || KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK,
                   "8- and 16-bit operands, or fp16 activations with row-packed 4-bit weights");
     constexpr int BM = 16 * MT;
@@ -329,9 +340,10 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
     constexpr bool SCALED = (KIND == K_FP8_BLOCK || KIND == K_I8_BLOCK);
     constexpr bool ROWCOL = (KIND == K_I8_ROWCOL);
     constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || W4NK) ? 2 : 1;
-    constexpr int MD_A = md_a(MT), STAGE = mdp_stage(MT);
+    constexpr int MD_A = mdp_a(MT, WIDE), STAGE = mdp_stage(MT, WIDE);
     constexpr int RB = MDP_RB;
-    constexpr int NAP = 2 * MT + (SCALED ? 1 : 0);          // direct-to-LDS loads per producer wave and step
+    constexpr int NPA = 2 * MT * NSUB / 4;                  // activation pieces per producer wave and step
+    constexpr int NAP = NPA + (SCALED ? 1 : 0);             // direct-to-LDS loads per producer wave and step
     constexpr int NBR = W4NK ? 2 : 8;                       // 16-byte weight registers per producer lane and step
     constexpr int NBP = W4NK ? 4 : 8;                       // register loads per producer wave and step (K_W4NK: + two scales)
     constexpr int LP = NAP + NBP;
@@ -341,6 +353,7 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4, q = wave & 3;
     const bool producer = wave >= 4;
+    const int ksub = WIDE ? (q & 1) : q, half = WIDE ? (q >> 1) : 0;     // sub-block of the step, row / column half
     const int N = p.N;
     const int K = p.K * ESZ;                                // row length in bytes
     const int KT_all = K >> 7;                              // 128-byte sub-blocks per row
@@ -350,11 +363,11 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
         kt0 = (int)blockIdx.z * per;
         KT = max(0, min(per, KT_all - kt0));
     }
-    const int nsteps = (KT + 3) >> 2;
-    const int n0 = blockIdx.x * MD_BN, m_start = blockIdx.y * BM, m_end = min(p.M, m_start + BM);
-    float* const bsl = (float*)(lds + (mdp_lds(MT) - D_MAX_KT * 4));
+    const int nsteps = (KT + NSUB - 1) / NSUB;
+    const int n0 = blockIdx.x * BN, m_start = blockIdx.y * BM, m_end = min(p.M, m_start + BM);
+    float* const bsl = (float*)(lds + (mdp_lds(MT, WIDE) - D_MAX_KT * 4));
 
-    // acc[i][j][e] = C[row 16 i + r][column 16 j + 4 g + e] summed over sub-blocks q of all steps (consumers)
+    // acc[i][j][e] = C[row 16 i + r][column 64 half + 16 j + 4 g + e] summed over sub-block ksub of all steps (consumers)
     v4f acc[MT][4];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
@@ -366,12 +379,14 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
         // 16-byte chunk lane & 7); the chunk index is XOR-swizzled with (row >> 1) & 7, on the global side for the
         // direct-to-LDS loads and on the LDS side for the weight rows, so that the fragment reads are conflict-free.
         const int row8 = lane >> 3;
-        uint32_t aoff[2 * MT], boff[NBR], blds[NBR], w4_soff[2] = {0, 0}, w4_chunk[2] = {0, 0};
+        uint32_t aoff[NPA], boff[NBR], blds[NBR], w4_soff[2] = {0, 0}, w4_chunk[2] = {0, 0};
         int w4_shift = 0;
-        const int w4_sub = (tid >> 1) & 3;                  // K_W4NK: sub-block of this lane's 32 weights
+        constexpr int SEGS = 4 * NSUB / 2;                  // K_W4NK: 32-weight segments of a row per step (8 or 4)
+        const int w4_sub = (tid & (SEGS - 1)) >> 1;         // K_W4NK: sub-block of this lane's 32 weights
+        const int arow0 = half * (8 * NPA);                 // WIDE: the two producers of a sub-block halve the rows
 #pragma unroll
-        for (int i = 0; i < 2 * MT; ++i) {
-            const int row = 8 * i + row8;
+        for (int i = 0; i < NPA; ++i) {
+            const int row = arow0 + 8 * i + row8;
             aoff[i] = (uint32_t)min(m_start + row, m_end - 1) * (uint32_t)K + (uint32_t)((lane & 7) ^ ((row >> 1) & 7)) * 16u;
         }
 #pragma unroll
@@ -380,31 +395,33 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
                 // producer thread t = 0 .. 255: the 32 weights k = 32 seg .. + 31 (seg = t & 7) of the step's 256 of rows
                 // t >> 3 and 32 + (t >> 3): 16 bytes of packed words each, four 16-byte chunks of the fp16 row of
                 // sub-block seg >> 1, and the group scale of those weights
-                const int row = ((tid - 256) >> 3) + 32 * i, seg = tid & 7;
+                // (WIDE: 128 weights per row and step, four segments; rows t >> 2 and 64 + (t >> 2))
+                const int row = ((tid - 256) / SEGS) + (256 / SEGS) * i, seg = tid & (SEGS - 1);
                 const uint32_t n = (uint32_t)min(n0 + row, N - 1);
                 boff[i] = n * (uint32_t)(p.K >> 1) + (uint32_t)(seg & 1) * 16u;       // + 32 bytes per sub-block
                 w4_soff[i] = n * (uint32_t)(p.K / p.group) * 2u;
-                blds[i] = (uint32_t)(MD_A + (seg >> 1) * (MD_BN * 128) + row * 128);
+                blds[i] = (uint32_t)(MD_A + (seg >> 1) * (BN * 128) + row * 128);
                 w4_chunk[i] = (uint32_t)(((4 * (seg & 1)) ^ ((row >> 1) & 7)) * 16);  // first chunk; chunk c is at ^ (c * 16)
             } else {
-                const int row = 8 * i + row8;
+                const int row = 64 * half + 8 * i + row8;
                 boff[i] = (uint32_t)min(n0 + row, N - 1) * (uint32_t)K + (uint32_t)(lane & 7) * 16u;
-                blds[i] = (uint32_t)(MD_A + q * (MD_BN * 128) + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16));
+                blds[i] = (uint32_t)(MD_A + ksub * (BN * 128) + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16));
             }
         }
         if constexpr (W4NK) w4_shift = __builtin_ctz((unsigned)(p.group >> 6));
-        auto kblock_sub = [&](int s, int sub) { return kt0 + min(4 * min(max(s, 0), nsteps - 1) + sub, KT - 1); };
+        auto kblock_sub = [&](int s, int sub) { return kt0 + min(NSUB * min(max(s, 0), nsteps - 1) + sub, KT - 1); };
         constexpr uint32_t SSZ = AS16 ? 2u : 4u;
-        const uint32_t soff = (uint32_t)min(m_start + min(lane, BM - 1), m_end - 1) * (uint32_t)KT_all * SSZ;
-        // sub-block q of step s, clamped to the last one of the range (requests past the end repeat it)
-        auto kblock = [&](int s) { return kt0 + min(4 * min(max(s, 0), nsteps - 1) + q, KT - 1); };
+        // scale column of a sub-block: 64 rows per producer (WIDE: the two producers of the sub-block take 64 rows each)
+        const uint32_t soff = (uint32_t)min(m_start + min(lane + 64 * half, BM - 1), m_end - 1) * (uint32_t)KT_all * SSZ;
+        // sub-block ksub of step s, clamped to the last one of the range (requests past the end repeat it)
+        auto kblock = [&](int s) { return kt0 + min(NSUB * min(max(s, 0), nsteps - 1) + ksub, KT - 1); };
         auto issue_a = [&](int s) {
             const uint32_t st = lds_base + (uint32_t)(s & 1) * STAGE;
             const int kb = kblock(s);
 #pragma unroll
-            for (int i = 0; i < 2 * MT; ++i) dma16(st + (uint32_t)(q * (BM * 128) + 8 * i * 128), aoff[i], p.a + (int64_t)kb * 128);
+            for (int i = 0; i < NPA; ++i) dma16(st + (uint32_t)(ksub * (BM * 128) + (arow0 + 8 * i) * 128), aoff[i], p.a + (int64_t)kb * 128);
             if constexpr (SCALED) {
-                const uint32_t ss = st + MD_A + MD_B + (uint32_t)q * 256u;
+                const uint32_t ss = st + MD_A + MD_B + (uint32_t)(WIDE ? 2 * ksub + half : q) * 256u;
                 if constexpr (AS16) dma2(ss, soff, (const uint8_t*)p.a_s + (int64_t)kb * 2);
                 else dma4(ss, soff, (const uint8_t*)p.a_s + (int64_t)kb * 4);
             }
@@ -509,16 +526,16 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
         __syncthreads();                                    // barrier 0
         for (int s = 0; s < nsteps; ++s) {
             const uint8_t* st = lds + (s & 1) * STAGE;
-            const uint8_t* As = st + q * (BM * 128);
-            const uint8_t* Bs = st + MD_A + q * (MD_BN * 128);
-            const int kb = 4 * s + q;
+            const uint8_t* As = st + ksub * (BM * 128);
+            const uint8_t* Bs = st + MD_A + ksub * (BN * 128) + half * (64 * 128);
+            const int kb = NSUB * s + ksub;
             const bool live = kb < KT;                     // wave-uniform: sub-blocks past the range add nothing
             v8i bf[4], af[2];
 #pragma unroll
             for (int j = 0; j < 4; ++j) bf[j] = ldfrag(Bs + j * 2048);
             af[0] = ldfrag(As);
             if constexpr (SCALED) {
-                const float* Ss = (const float*)(st + MD_A + MD_B) + q * 64 + r;
+                const float* Ss = (const float*)(st + MD_A + MD_B) + ksub * (WIDE ? 128 : 64) + r;
                 const float bs = live ? bsl[min(kb, KT - 1)] : 0.f;
                 float sa[MT];
 #pragma unroll
@@ -558,58 +575,62 @@ __global__ __launch_bounds__(MD_THREADS) void gemm_mid_pc_kernel(DirectArgs p) {
     }
     __syncthreads();
 
-    // ---- the four sub-block sums of every output meet in LDS: red[q][row][column], rows of 68 floats
+    // ---- the NSUB sub-block sums of every output meet in LDS: red[sub-block][row][column], rows of BN + 4 floats
     float* red = (float*)lds;
     if (!producer) {
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                *(v4f*)(red + (q * BM + 16 * i + r) * MD_RED_ROW + 16 * j + 4 * g) = acc[i][j];
+                *(v4f*)(red + (ksub * BM + 16 * i + r) * RED_ROW + 64 * half + 16 * j + 4 * g) = acc[i][j];
     }
     __syncthreads();
-    // thread: row tid >> 3, columns 8 (tid & 7) .. + 7
-    const int orow = tid >> 3, ocol = 8 * (tid & 7);
-    if (orow >= BM) return;
-    const int m = m_start + orow, n = n0 + ocol;
-    if (m >= m_end || n >= N) return;
-    v4f sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (ROWCOL) {
-        v4i ia = {0, 0, 0, 0}, ib = {0, 0, 0, 0};
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float* src = red + (k * BM + orow) * MD_RED_ROW + ocol;
-            ia += *(const v4i*)src;
-            ib += *(const v4i*)(src + 4);
-        }
-        __builtin_memcpy(&sa, &ia, 16);
-        __builtin_memcpy(&sb, &ib, 16);
-    } else {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float* src = red + (k * BM + orow) * MD_RED_ROW + ocol;
-            sa += *(const v4f*)src;
-            sb += *(const v4f*)(src + 4);
-        }
-    }
+    // thread: columns 8 (tid % (BN / 8)) .. + 7 of row tid / (BN / 8), then the rows 4096 / BN further on
+    constexpr int RUNS = BN / 8, ROWS_PASS = MD_THREADS / RUNS;
     const bool split = p.ksplit > 1;
     void* cout = split ? (void*)(p.partial + (int64_t)blockIdx.z * p.M * N) : p.c;
     const int cdt = split ? LLMK_F32 : p.c_dtype;
     const int esz = cdt == LLMK_F32 ? 4 : 2;
     const bool vec_ok = ((((uintptr_t)cout) & 15) == 0) && (((int64_t)N * esz) % 16 == 0);
-    const int nv = N - n;
-    const int64_t off = (int64_t)m * N + n;
-    if constexpr (ROWCOL) {
-        // (a K slice leaves its int32 sums, bit for bit, in the fp32 partial buffer: the summing pass adds them as
-        // integers and scales once, so the result does not depend on the split)
-        if (!split) {
-            rowcol_epilogue8(p, sa, sb, m, off, n, nv);
-            if (!p.c) return;
+    const int ocol = 8 * (tid % RUNS), n = n0 + ocol, nv = N - n;
+    if (n >= N) return;
+#pragma unroll
+    for (int pass = 0; pass < (BM + ROWS_PASS - 1) / ROWS_PASS; ++pass) {
+        const int orow = pass * ROWS_PASS + tid / RUNS;
+        const int m = m_start + orow;
+        if (orow >= BM || m >= m_end) continue;
+        v4f sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (ROWCOL) {
+            v4i ia = {0, 0, 0, 0}, ib = {0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < NSUB; ++k) {
+                const float* src = red + (k * BM + orow) * RED_ROW + ocol;
+                ia += *(const v4i*)src;
+                ib += *(const v4i*)(src + 4);
+            }
+            __builtin_memcpy(&sa, &ia, 16);
+            __builtin_memcpy(&sb, &ib, 16);
+        } else {
+#pragma unroll
+            for (int k = 0; k < NSUB; ++k) {
+                const float* src = red + (k * BM + orow) * RED_ROW + ocol;
+                sa += *(const v4f*)src;
+                sb += *(const v4f*)(src + 4);
+            }
         }
+        const int64_t off = (int64_t)m * N + n;
+        if constexpr (ROWCOL) {
+            // (a K slice leaves its int32 sums, bit for bit, in the fp32 partial buffer: the summing pass adds them as
+            // integers and scales once, so the result does not depend on the split)
+            if (!split) {
+                rowcol_epilogue8(p, sa, sb, m, off, n, nv);
+                if (!p.c) continue;
+            }
+        }
+        if (cdt == LLMK_BF16) store_run8<LLMK_BF16>(cout, off, sa, sb, nv, vec_ok);
+        else if (cdt == LLMK_F16) store_run8<LLMK_F16>(cout, off, sa, sb, nv, vec_ok);
+        else store_run8<LLMK_F32>(cout, off, sa, sb, nv, vec_ok);
     }
-    if (cdt == LLMK_BF16) store_run8<LLMK_BF16>(cout, off, sa, sb, nv, vec_ok);
-    else if (cdt == LLMK_F16) store_run8<LLMK_F16>(cout, off, sa, sb, nv, vec_ok);
-    else store_run8<LLMK_F32>(cout, off, sa, sb, nv, vec_ok);
 }
 
 // K slices of the mid-size kernel: as many as bring the grid to about one workgroup per CU, in whole steps of 512
@@ -638,6 +659,17 @@ inline MidPlan mid_plan(int64_t M, int64_t N, int64_t kbytes) {
     return pl;
 }
 
+// The 128-column form: 64-row tiles while they fit one round of workgroups, else 128-row tiles; K slices as above.
+inline MidPlan midw_plan(int64_t M, int64_t N, int64_t kbytes) {
+    MidPlan pl;
+    const int64_t gx = (N + 127) / 128;
+    const int64_t t4 = ((M + 63) / 64) * gx, t8 = ((M + 127) / 128) * gx;
+    pl.mt = t4 <= LLMK_CUS ? 4 : 8;
+    pl.tiles = pl.mt == 4 ? t4 : t8;
+    pl.z = mid_splitk(pl.tiles, kbytes);
+    return pl;
+}
+
 // Eligibility: 32-bit source offsets, whole 128-byte sub-blocks, scale table size (as dma_eligible), and for the
 // K_W4A8 kind room for its table behind the stages.
 template <int KIND>
@@ -652,27 +684,29 @@ inline bool mid_eligible(const DirectArgs& p, int mt, int ksplit) {
 
 // p.a_s: fp32, or with AS16 the 16-bit scales of dtype p.s_dtype as the caller passed them; p.s_dtype describes b_s
 // (and those).  p.ksplit / p.partial select the K split.
-template <int KIND, int MT, bool AS16 = false>
+template <int KIND, int MT, bool AS16 = false, bool WIDE = false>
 int launch_mid(const DirectArgs& p, hipStream_t stream, const char* name) {
     static std::atomic<uint64_t> configured{0};
     constexpr bool W4 = (KIND == K_W4A8);
+    static_assert(!(W4 && WIDE), "the 128-column form exists for the producer / consumer kernel only");
     // the producer / consumer form, except for w4a8 (whose expansion is vector-ALU work that wants all eight waves)
     auto kern = [] {
         if constexpr (W4) return gemm_mid_kernel<KIND, MT, AS16>;
-        else return gemm_mid_pc_kernel<KIND, MT, AS16>;
+        else return gemm_mid_pc_kernel<KIND, MT, AS16, WIDE>;
     }();
     constexpr int ESZ = (KIND == K_F16 || KIND == K_BF16 || KIND == K_W4NK) ? 2 : 1;
     const int KT_all = (p.K * ESZ) >> 7;
     const bool split = p.ksplit > 1 && p.partial;
     const int per = split ? ((((KT_all + p.ksplit - 1) / p.ksplit) + 3) & ~3) : KT_all;
-    const int lds_bytes = W4 ? md_lds(MT, per) : mdp_lds(MT);
+    const int lds_bytes = W4 ? md_lds(MT, per) : mdp_lds(MT, WIDE);
     if (lds_bytes > D_LDS_MAX) LLMK_FAIL(LLMK_ERR_SHAPE, "%s: %d bytes of LDS needed", name, lds_bytes);
     if (int rc = llmk_reserve_lds((const void*)kern, D_LDS_MAX, configured, name)) return rc;
     // slices that would start past the end of K are not launched
     const int z = split ? (KT_all + per - 1) / per : 1;
     DirectArgs q = p;
     q.ksplit = split ? p.ksplit : 1;
-    dim3 grid((unsigned)((p.N + MD_BN - 1) / MD_BN), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)), (unsigned)z);
+    constexpr int BN = mdp_bn(WIDE);
+    dim3 grid((unsigned)((p.N + BN - 1) / BN), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)), (unsigned)z);
     if (grid.x == 0 || grid.y == 0) return LLMK_OK;
     kern<<<grid, MD_THREADS, lds_bytes, stream>>>(q);
     LLMK_CHECK_LAUNCH(name);

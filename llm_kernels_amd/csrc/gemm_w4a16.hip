@@ -1015,6 +1015,14 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
                                   : llmk::launch_mid<llmk::K_W4NK, 2>(p, st, "gemm_w4a16_nk(mid)");
             }
         }
+        // wider weights on one round of 128-column tiles: the 128-column form of that kernel
+        if (llmk::midw_wanted(M, N, 2 * K) && llmk::dma_eligible(p, 2) && (groupsize & (groupsize - 1)) == 0) {
+            llmk::MidPlan pl = llmk::midw_plan(M, N, 2 * K);
+            if (pl.z > 1 && !(workspace && workspace_bytes >= (int64_t)pl.z * M * N * 4 && !((uintptr_t)workspace & 15))) pl.z = 1;
+            if (pl.z > 1) { p.partial = (float*)workspace; p.ksplit = pl.z; }
+            return pl.mt == 4 ? llmk::launch_mid<llmk::K_W4NK, 4, false, true>(p, st, "gemm_w4a16_nk(mid, 128 columns)")
+                              : llmk::launch_mid<llmk::K_W4NK, 8, false, true>(p, st, "gemm_w4a16_nk(mid, 128 columns)");
+        }
         if (llmk::dma_eligible(p, 2))
             return llmk::launch_big_half<llmk::K_W4NK, false>(p, st, "gemm_w4a16_nk(fused tiles)", workspace, workspace_bytes);
     }

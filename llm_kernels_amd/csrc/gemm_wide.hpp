@@ -768,6 +768,18 @@ inline bool mid_wanted(int64_t M, int64_t N, int64_t kbytes) {
     return pl.tiles <= LLMK_CUS && kbytes <= (pl.mt == 4 ? 16384 : 8192);
 }
 
+// Shapes for the 128-column form of that kernel: weights too wide for the 64-column form, one round of 64- or 128-row
+// tiles, rows of at most 8 KB.  Taken for fp8 and for fp16 activations with row-packed 4-bit weights, where it beats
+// the 128-column tile kernels (fp8, us per launch, cold weights: 128 x 14336 x 4096 26.3 -> 23.2, 256 x 14336 x 4096
+// 37.6 -> 29.6, 256 x 6144 x 4096 23.6 -> 20.2, 128 x 28672 x 4096 44.3 -> 38.6, 384 x 8192 x 4096 35.1 -> 27.7,
+// 128 x 14336 x 8192 53.5 -> 38.9; 4-bit 128 x 14336 x 4096 37.1 -> 33.2, same elsewhere); the int8 kinds lose on it
+// (per-token 128 x 14336 x 4096 23.9 -> 25.9, 256 x 14336 x 4096 28.9 -> 34.7; block-scaled 34.8 -> 37.4) and stay where
+// they were, and two rounds of its workgroups lose everywhere (fp8 256 x 28672 x 4096 48.6 -> 62.6).
+inline bool midw_wanted(int64_t M, int64_t N, int64_t kbytes) {
+    if (M <= 64 || M > 512 || kbytes > 8192) return false;
+    return midw_plan(M, N, kbytes).tiles <= LLMK_CUS;
+}
+
 // 16 < M <= 64: the weight-streaming kernel re-reads the activations for every 16 columns, which costs more
 // than the 64-row tile kernel (with split-K when its tiles are few) once the weight matrix is large (measured
 // crossover between 17 M and 25 M elements).
@@ -850,6 +862,19 @@ int launch_big(DirectArgs p, void* workspace, int64_t workspace_bytes, hipStream
                         return pl.mt == 4 ? launch_mid<KIND, 4, true>(p, stream, name) : launch_mid<KIND, 2, true>(p, stream, name);
                 }
                 return pl.mt == 4 ? launch_mid<KIND, 4>(p, stream, name) : launch_mid<KIND, 2>(p, stream, name);
+            }
+        }
+    }
+    if constexpr (!GROUPED) {
+        // wider weights: the 128-column form of the same kernel (fp8; see midw_wanted)
+        if (KIND == K_FP8_BLOCK && p.s_dtype == LLMK_F32 && midw_wanted(p.M, p.N, p.K)) {
+            MidPlan pl = midw_plan(p.M, p.N, p.K);
+            const int64_t need = (int64_t)pl.z * p.M * p.N * 4;
+            if (pl.z > 1 && !(workspace && workspace_bytes >= need && !(((uintptr_t)workspace) & 15))) pl.z = 1;
+            if (dma_eligible(p)) {
+                if (pl.z > 1) { p.partial = (float*)workspace; p.ksplit = pl.z; }
+                if constexpr (KIND == K_FP8_BLOCK)
+                    return pl.mt == 4 ? launch_mid<KIND, 4, false, true>(p, stream, name) : launch_mid<KIND, 8, false, true>(p, stream, name);
             }
         }
     }

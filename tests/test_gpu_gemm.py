@@ -296,6 +296,30 @@ def test_mid_and_small_tile_kernels_exact_integers(dev, M, N, K):
         assert torch.equal(acc.cpu().long(), ref), "int8 per token"
 
 
+@pytest.mark.parametrize("M,N,K", [(130, 9000, 640), (300, 5000, 1152), (500, 3208, 384), (100, 16000, 256), (128, 20000, 640),
+                                   (256, 14336, 4096), (512, 6144, 8192)])
+def test_fp8_one_round_of_128_column_tiles(dev, M, N, K):
+    """fp8 block GEMM on weights too wide for the 64-column mid-size kernel that fit one round of 64- or 128-row by
+    128-column tiles (the 128-column form of the producer / consumer kernel): ragged rows and columns, odd numbers of
+    K blocks.  Small integers with unit scales must come out exactly; quantised random operands within 1e-2 of the
+    oracle."""
+    announce("fp8 128-column mid-size", M, N, K)
+    torch.manual_seed(M + N + K)
+    a = torch.randint(-7, 8, (M, K), dtype=torch.int8)
+    b = torch.randint(-7, 8, (N, K), dtype=torch.int8)
+    with default_dtype(torch.float32):
+        c = fp8_kernel.fp8_gemm(a.float().to(torch.float8_e4m3fn).to(dev), torch.ones(M, K // 128).to(dev),
+                                b.float().to(torch.float8_e4m3fn).to(dev), torch.ones((N + 127) // 128, K // 128).to(dev))
+    assert torch.equal(c.cpu().long(), (a.double() @ b.double().T).long())
+    x = torch.randn(M, K).bfloat16()
+    w = torch.randn(N, K) * 0.02
+    aq, a_s = q.act_quant_fp8(x)
+    bq, b_s = q.weight_quant_fp8(w)
+    with default_dtype(torch.bfloat16):
+        c = fp8_kernel.fp8_gemm(aq.to(dev), a_s.to(dev), bq.to(dev), b_s.to(dev))
+    assert_close_scaled(c, g.gemm_blockwise(aq, a_s, bq, b_s), what="fp8 128-column mid-size")
+
+
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("M,N,K,out", [(128, 1024, 4096, torch.bfloat16), (200, 520, 3200, torch.float32),
                                        (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16),

@@ -179,7 +179,11 @@ def test_mul_mid_m_fused_tiles(dev, M, N, K, gs):
 
 @pytest.mark.parametrize("M,N,K,gs", [(65, 136, 128, 64), (128, 4096, 4096, 128), (200, 1000, 1152, 128), (256, 520, 8192, 256),
                                       (512, 264, 2048, 64), (100, 129, 14336, -1), (130, 4100, 4224, 128), (96, 28672, 1024, 128),
-                                      (48, 4096, 14336, 128), (64, 28672, 4096, 128), (33, 2400, 14336, 256)])
+                                      (48, 4096, 14336, 128), (64, 28672, 4096, 128), (33, 2400, 14336, 256),
+                                      # one round of 128-column tiles of the producer / consumer kernel: 64- and 128-row tiles,
+                                      # ragged rows and columns, groups of 64 and of the whole row
+                                      (130, 9000, 640, 64), (300, 5000, 1152, 128), (100, 16000, 256, -1), (128, 20000, 384, 64),
+                                      (128, 14336, 4096, 128)])
 def test_w4a16_nk_mid_m_fused_tiles(dev, M, N, K, gs):
     """64 < M <= 512, and 32 < M <= 64 with large weights: the tile kernels expand the packed words themselves
     (one or several K slices, ragged rows and columns, group sizes from 64 to the whole row)."""
