@@ -1016,7 +1016,7 @@ extern "C" int llmk_gemm_w4a16_nk(const void* a, const int32_t* b_packed, void* 
             }
         }
         // wider weights on one round of 128-column tiles: the 128-column form of that kernel
-        if (llmk::midw_wanted(M, N, 2 * K) && llmk::dma_eligible(p, 2) && (groupsize & (groupsize - 1)) == 0) {
+        if (2 * K <= 8192 && llmk::midw_wanted(M, N, 2 * K) && llmk::dma_eligible(p, 2) && (groupsize & (groupsize - 1)) == 0) {       // (longer rows: measured for fp8 only)
             llmk::MidPlan pl = llmk::midw_plan(M, N, 2 * K);
             if (pl.z > 1 && !(workspace && workspace_bytes >= (int64_t)pl.z * M * N * 4 && !((uintptr_t)workspace & 15))) pl.z = 1;
             if (pl.z > 1) { p.partial = (float*)workspace; p.ksplit = pl.z; }

@@ -768,15 +768,16 @@ inline bool mid_wanted(int64_t M, int64_t N, int64_t kbytes) {
     return pl.tiles <= LLMK_CUS && kbytes <= (pl.mt == 4 ? 16384 : 8192);
 }
 
-// Shapes for the 128-column form of that kernel: weights too wide for the 64-column form, one round of 64- or 128-row
-// tiles, rows of at most 8 KB.  Taken for fp8 and for fp16 activations with row-packed 4-bit weights, where it beats
+// Shapes for the 128-column form of that kernel: shapes the 64-column form does not take, one round of 64- or 128-row
+// tiles, rows of at most 16 KB (256 x 14336 x 14336 118.4 -> 86.3 us, 128 x 14336 x 14336 85.4 -> 65.7, 128 x 4096 x 14336
+// in four K slices 28.4 -> 27.0).  Taken for fp8 and for fp16 activations with row-packed 4-bit weights, where it beats
 // the 128-column tile kernels (fp8, us per launch, cold weights: 128 x 14336 x 4096 26.3 -> 23.2, 256 x 14336 x 4096
 // 37.6 -> 29.6, 256 x 6144 x 4096 23.6 -> 20.2, 128 x 28672 x 4096 44.3 -> 38.6, 384 x 8192 x 4096 35.1 -> 27.7,
 // 128 x 14336 x 8192 53.5 -> 38.9; 4-bit 128 x 14336 x 4096 37.1 -> 33.2, same elsewhere); the int8 kinds lose on it
 // (per-token 128 x 14336 x 4096 23.9 -> 25.9, 256 x 14336 x 4096 28.9 -> 34.7; block-scaled 34.8 -> 37.4) and stay where
 // they were, and two rounds of its workgroups lose everywhere (fp8 256 x 28672 x 4096 48.6 -> 62.6).
 inline bool midw_wanted(int64_t M, int64_t N, int64_t kbytes) {
-    if (M <= 64 || M > 512 || kbytes > 8192) return false;
+    if (M <= 64 || M > 512 || kbytes > 16384) return false;
     return midw_plan(M, N, kbytes).tiles <= LLMK_CUS;
 }
 

@@ -324,7 +324,10 @@ def test_fp8_one_round_of_128_column_tiles(dev, M, N, K):
 @pytest.mark.parametrize("M,N,K,out", [(128, 1024, 4096, torch.bfloat16), (200, 520, 3200, torch.float32),
                                        (70, 136, 1152, torch.float16), (300, 2048, 8192, torch.bfloat16),
                                        (48, 2560, 16384, torch.bfloat16), (64, 14336, 4096, torch.float16),
-                                       (256, 4096, 14336, torch.bfloat16)])
+                                       (256, 4096, 14336, torch.bfloat16),
+                                       # fp8: K slices of the 128-column form of the mid-size kernel (rows beyond 8 KB on few tiles)
+                                       (128, 4096, 14336, torch.bfloat16), (100, 3000, 10240, torch.float32),
+                                       (256, 14336, 14336, torch.float16)])
 def test_mid_m_split_k_shapes(dev, kind, M, N, K, out):
     """Mid-size M with few column tiles: the K range is split over workgroups (uneven slices included)."""
     announce("split-K", kind, M, N, K, out)
