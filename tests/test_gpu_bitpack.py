@@ -41,6 +41,27 @@ def test_pack_unpack_all_widths(dev, nbits, width):
         assert torch.equal(bitpack.unpack_over_cols_torch(pc, nbits, w.shape[1]), uc)
 
 
+@pytest.mark.parametrize("nbits,width", list(itertools.product([1, 2, 4, 8], [8, 16, 32, 64])))
+def test_pack_unpack_all_widths_16_byte_kernels(dev, nbits, width):
+    """The same for shapes that the 16-bytes-per-thread kernels take (uint8 elements, 192 columns: a multiple of 16 and
+    of every e), plus a partial unpack (fewer rows than the words hold) on those kernels."""
+    announce("bitpack 16-byte kernels", nbits, width)
+    rng = np.random.default_rng(nbits * 1000 + width)
+    e = width // nbits
+    w = rng.integers(0, 2 ** nbits, size=(3 * e, 192), dtype=np.uint8)
+    wt = torch.from_numpy(w).to(dev)
+    pr, _ = bitpack.pack_weights_over_rows(wt, nbits, width, transpose=False)
+    pc, _ = bitpack.pack_weights_over_cols(wt, nbits, width, transpose=False)
+    assert torch.equal(pr.cpu(), torch.from_numpy(bp.pack_rows(w, nbits, width)[0]))
+    assert torch.equal(pc.cpu(), torch.from_numpy(bp.pack_cols(w, nbits, width)[0]))
+    assert torch.equal(bitpack.unpack_over_rows(pr, nbits, w.shape[0]).cpu(), torch.from_numpy(w))
+    assert torch.equal(bitpack.unpack_over_cols(pc, nbits, w.shape[1]).cpu(), torch.from_numpy(w))
+    if e > 1:
+        part = bitpack.unpack_over_rows(pr, nbits, 3 * (e // 2))      # e / 2 elements of every word
+        ref = w.reshape(3, e, 192)[:, :e // 2, :].reshape(3 * (e // 2), 192)
+        assert torch.equal(part.cpu(), torch.from_numpy(np.ascontiguousarray(ref)))
+
+
 def test_reference_recipe_and_transpose(dev):
     announce("bitpack recipe 8x16")
     torch.manual_seed(0)
