@@ -121,44 +121,76 @@ __global__ void weight_quant_block_kernel(const void* __restrict__ x, void* __re
     const int64_t r0 = (int64_t)blockIdx.y * block, c0 = (int64_t)blockIdx.x * block;
     const int t = threadIdx.x;
     const int cc = (t & 15) * EPL;
+    // whole tiles of rows that are whole 16-byte chunks: 8 elements per load and per store
+    const bool vec = r0 + block <= M && c0 + block <= N && N % EPL == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
     float v[8][EPL];
     float m = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int rr = (t >> 4) + 16 * j;
         const int64_t r = r0 + rr;
+        if (vec) {
+            if (rr < block && cc < block) {
+                load8<DT>(x, r * N + c0 + cc, v[j]);
+            } else {
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            const int64_t c = c0 + cc + e;
-            float val = 0.f;
-            if (rr < block && cc + e < block && r < M && c < N) {
-                val = FloatIO<DT>::ld(x, r * N + c);
+                for (int e = 0; e < EPL; ++e) v[j][e] = 0.f;
             }
-            v[j][e] = val;
-            m = fmaxf(m, fabsf(val));
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const int64_t c = c0 + cc + e;
+                float val = 0.f;
+                if (rr < block && cc + e < block && r < M && c < N) val = FloatIO<DT>::ld(x, r * N + c);
+                v[j][e] = val;
+            }
         }
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) m = fmaxf(m, fabsf(v[j][e]));
     }
     m = wave_max(m);
     if ((t & 63) == 0) red[t >> 6] = m;
     __syncthreads();
     m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     const float sc = m / qmax;
+    // v / sc by the shared reciprocal and one residual correction where the operands allow it (see div_by)
+    const bool fast = div_by_ok(sc);
+    const float rcp = fast ? 1.0f / sc : 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int rr = (t >> 4) + 16 * j;
         const int64_t r = r0 + rr;
+        float q[EPL];
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
-            const int64_t c = c0 + cc + e;
-            if (rr < block && cc + e < block && r < M && c < N) {
-                float q = v[j][e] / sc;
+            q[e] = fast ? div_by(v[j][e], sc, rcp) : v[j][e] / sc;
+            if constexpr (!FP8) {
+                q[e] = round_mode(q[e], mode);
+                if (clamp) q[e] = fminf(fmaxf(q[e], -qmax), qmax);
+            }
+        }
+        if (vec) {
+            if (rr < block && cc < block) {
+                uint2 o;
                 if constexpr (FP8) {
-                    unsigned w = pack_fp8x4(q, 0.f, 0.f, 0.f);
-                    ((uint8_t*)y)[r * N + c] = (uint8_t)(w & 0xff);
+                    o.x = pack_fp8x4(q[0], q[1], q[2], q[3]);
+                    o.y = pack_fp8x4(q[4], q[5], q[6], q[7]);
                 } else {
-                    q = round_mode(q, mode);
-                    if (clamp) q = fminf(fmaxf(q, -qmax), qmax);
-                    ((int8_t*)y)[r * N + c] = (int8_t)(int)q;
+                    unsigned w[2] = {0, 0};
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) w[e >> 2] |= ((unsigned)((int)q[e] & 0xff)) << (8 * (e & 3));
+                    o.x = w[0];
+                    o.y = w[1];
+                }
+                *(uint2*)((uint8_t*)y + r * N + c0 + cc) = o;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const int64_t c = c0 + cc + e;
+                if (rr < block && cc + e < block && r < M && c < N) {
+                    if constexpr (FP8) ((uint8_t*)y)[r * N + c] = (uint8_t)(pack_fp8x4(q[e], 0.f, 0.f, 0.f) & 0xff);
+                    else ((int8_t*)y)[r * N + c] = (int8_t)(int)q[e];
                 }
             }
         }
@@ -217,6 +249,47 @@ __global__ void weight_dequant_block_kernel(const uint8_t* __restrict__ x, const
         xv = (float)(int8_t)x[idx];
     }
     FloatIO<ODT>::st(y, idx, xv * sc);
+}
+
+// the same with 16 elements of a row per thread (N and the block size multiples of 16: one scale per thread)
+template <int ODT, int SDT, bool FP8>
+__global__ void weight_dequant_block_vec_kernel(const uint8_t* __restrict__ x, const void* __restrict__ s,
+                                                void* __restrict__ y, int64_t M, int64_t N, int block) {
+    const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 16;
+    if (idx >= M * N) return;
+    const int64_t r = idx / N, c = idx - r * N;
+    const int64_t nb = (N + block - 1) / block;
+    const float sc = FloatIO<SDT>::ld(s, (r / block) * nb + c / block);
+    const uint4 w = *(const uint4*)(x + idx);
+    const unsigned ws[4] = {w.x, w.y, w.z, w.w};
+    float v[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        if constexpr (FP8) {
+            v[4 * q + 0] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 0) * sc;
+            v[4 * q + 1] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 1) * sc;
+            v[4 * q + 2] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 2) * sc;
+            v[4 * q + 3] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 3) * sc;
+        } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) v[4 * q + b] = (float)(int8_t)(ws[q] >> (8 * b)) * sc;
+        }
+    }
+    if constexpr (ODT == LLMK_F32) {
+        float4* dst = (float4*)((float*)y + idx);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dst[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+    } else {
+        uint4 o[2];
+        unsigned* op = (unsigned*)o;
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            op[q] = ODT == LLMK_F16 ? ((unsigned)f32_to_f16(v[2 * q]) | ((unsigned)f32_to_f16(v[2 * q + 1]) << 16))
+                                    : ((unsigned)f32_to_bf16(v[2 * q]) | ((unsigned)f32_to_bf16(v[2 * q + 1]) << 16));
+        uint4* dst = (uint4*)((unsigned short*)y + idx);
+        dst[0] = o[0];
+        dst[1] = o[1];
+    }
 }
 
 __global__ void w4a8_dequant_kernel(const int32_t* __restrict__ packed, const unsigned short* __restrict__ s,
@@ -372,6 +445,12 @@ extern "C" int llmk_weight_dequant_fp8_block(const void* x, const float* s, void
     if (M == 0 || N == 0) return LLMK_OK;
     if (!x || !s || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_fp8_block: null pointer");
     dim3 grid((unsigned)cdiv64(M * N, 256)), blk(256);
+    if (N % 16 == 0 && block % 16 == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0) {
+        dim3 vgrid((unsigned)cdiv64(M * N / 16, 256));
+        LLMK_DISPATCH_FLOAT(y_dtype, ODT, (weight_dequant_block_vec_kernel<ODT, LLMK_F32, true><<<vgrid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block)));
+        LLMK_CHECK_LAUNCH("weight_dequant_fp8_block");
+        return LLMK_OK;
+    }
     LLMK_DISPATCH_FLOAT(y_dtype, ODT, (weight_dequant_block_kernel<ODT, LLMK_F32, true><<<grid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block)));
     LLMK_CHECK_LAUNCH("weight_dequant_fp8_block");
     return LLMK_OK;
@@ -383,6 +462,12 @@ extern "C" int llmk_weight_dequant_i8_block(const int8_t* x, const void* s, int 
     if (M == 0 || N == 0) return LLMK_OK;
     if (!x || !s || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_i8_block: null pointer");
     dim3 grid((unsigned)cdiv64(M * N, 256)), blk(256);
+    if (N % 16 == 0 && block % 16 == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0) {
+        dim3 vgrid((unsigned)cdiv64(M * N / 16, 256));
+        LLMK_DISPATCH_FLOAT(y_dtype, ODT, LLMK_DISPATCH_FLOAT(s_dtype, SDT, (weight_dequant_block_vec_kernel<ODT, SDT, false><<<vgrid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block))));
+        LLMK_CHECK_LAUNCH("weight_dequant_i8_block");
+        return LLMK_OK;
+    }
     LLMK_DISPATCH_FLOAT(y_dtype, ODT, LLMK_DISPATCH_FLOAT(s_dtype, SDT, (weight_dequant_block_kernel<ODT, SDT, false><<<grid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block))));
     LLMK_CHECK_LAUNCH("weight_dequant_i8_block");
     return LLMK_OK;
