@@ -167,6 +167,13 @@ int64_t llmk_gemm_w4a16_marlin_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int llmk_gemm_w4a16_marlin(const void* a_f16, const int32_t* b, void* c_f16, const void* s_f16,
                            int64_t M, int64_t N, int64_t K, int groupsize,
                            void* workspace, int64_t workspace_bytes, void* stream);
+/* Quantiser of the [N, K] bit-packed W4A16 layout (the reference states this rule only in its benchmark
+ * configuration: groups along K, s = absmax / 7 as fp16, q = clamp(rne(w / s), -8, 7) + 8, 8 K-consecutive nibbles
+ * per int32 as quantization/bitpack.py:38-145 packs columns).  w fp32 / fp16 / bf16 [N, K], 16-byte aligned;
+ * packed int32 [N, K/8]; scales fp16 [N, K/group]; q (optional, 8-byte aligned) uint8 [N, K]; group a power
+ * of two in 8..512 dividing K. */
+int llmk_quant_w4_nk(const void* w, int w_dtype, int32_t* packed, void* scales_f16, uint8_t* q, int64_t N,
+                     int64_t K, int group, void* stream);
 /* Same product for W stored [N, K/8] int32 by pack_weights_over_cols (nibble i of a word = k*8+i)
  * with s fp16 [N, K/g]; a/c fp16 or bf16 (ac_dtype; bf16: M <= 64 with 128-wide groups streams the weights,
  * every other bf16 call multiplies a bf16 copy of W and needs the N*K*2-byte workspace).  workspace is optional for fp16:

@@ -34,6 +34,7 @@ SIGNATURES = {
     "llmk_quant_i8_rowwise": [_p, _i, _p, _p, _l, _l, _p],
     "llmk_weight_quant_i8_block": [_p, _i, _p, _p, _l, _l, _i, _f, _i, _i, _p],
     "llmk_weight_quant_fp8_block": [_p, _i, _p, _p, _l, _l, _i, _p],
+    "llmk_quant_w4_nk": [_p, _i, _p, _p, _p, _l, _l, _i, _p],
     "llmk_weight_quant_w4a8_level2": [_p, _p, _p, _l, _l, _i, _p],
     "llmk_weight_dequant_fp8_block": [_p, _p, _p, _i, _l, _l, _i, _p],
     "llmk_weight_dequant_i8_block": [_p, _p, _i, _p, _i, _l, _l, _i, _p],

@@ -312,6 +312,43 @@ __global__ void w4a8_dequant_kernel(const int32_t* __restrict__ packed, const un
     }
 }
 
+// ---------------------------------------------------------------- symmetric int4 along K for W [N, K] (W4A16)
+// s = absmax / 7 rounded to fp16; q = clamp(rne(w / s), -8, 7) + 8 with the division by the rounded scale in
+// fp32.  A lane owns 8 consecutive k: its 8 nibbles are exactly one int32 of the [N, K/8] bit-packed layout
+// (nibble i of a word is k = 8 word + i), so the packed word, the 8 bytes of q and the group's scale leave in
+// one pass over W.  A group of zeros has scale 0 and stores q = 8 (the value 0).
+template <int DT, int LPG>
+__global__ void w4_quant_nk_kernel(const void* __restrict__ w, int32_t* __restrict__ packed,
+                                   unsigned short* __restrict__ s, uint8_t* __restrict__ q, int64_t n_groups) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t grp = tid / LPG;
+    const bool live = grp < n_groups;
+    const int64_t off = live ? tid * EPL : 0;
+    float v[EPL];
+    load8<DT>(w, off, v);
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) m = fmaxf(m, fabsf(v[j]));
+    m = group_max<LPG>(m);
+    if (!live) return;
+    const unsigned short sh = f32_to_f16(m / 7.0f);
+    const float sc = f16_to_f32(sh);
+    const bool fast = div_by_ok(sc);
+    const float r = fast ? 1.0f / sc : 0.f;
+    unsigned word = 0, b[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+        const float t = fast ? div_by(v[j], sc, r) : v[j] / sc;
+        const float c = fminf(fmaxf(rintf(t), -8.f), 7.f);        // fmin / fmax drop a NaN (0 / 0): the value 0
+        const unsigned n = (unsigned)((int)(t != t ? 0.f : c) + 8);
+        word |= n << (4 * j);
+        b[j >> 2] |= n << (8 * (j & 3));
+    }
+    packed[tid] = (int32_t)word;
+    if (q) *(uint2*)(q + off) = make_uint2(b[0], b[1]);
+    if (tid % LPG == 0) s[grp] = sh;
+}
+
 bool lpg_ok(int block) {
     return block == 8 || block == 16 || block == 32 || block == 64 || block == 128 || block == 256 || block == 512;
 }
@@ -336,6 +373,24 @@ extern "C" int llmk_act_quant_fp8(const void* x, int x_dtype, void* y, float* s,
     LPG_SWITCH(block, CALL)
 #undef CALL
     LLMK_CHECK_LAUNCH("act_quant_fp8");
+    return LLMK_OK;
+}
+
+/* W [N, K] float -> int32 [N, K/8] nibbles along K, fp16 scales [N, K/group], optionally q uint8 [N, K] */
+extern "C" int llmk_quant_w4_nk(const void* w, int w_dtype, int32_t* packed, void* scales, uint8_t* q, int64_t N,
+                                int64_t K, int group, void* stream) {
+    if (!lpg_ok(group)) LLMK_FAIL(LLMK_ERR_SHAPE, "quant_w4_nk: group %d unsupported (power of two in 8..512)", group);
+    if (N < 0 || K < 0 || K % group) LLMK_FAIL(LLMK_ERR_SHAPE, "quant_w4_nk: K %lld is not a multiple of the group %d", (long long)K, group);
+    if (N == 0 || K == 0) return LLMK_OK;
+    if (!w || !packed || !scales) LLMK_FAIL(LLMK_ERR_ARG, "quant_w4_nk: bad argument");
+    if (((uintptr_t)w & 15) || ((uintptr_t)q & 7)) LLMK_FAIL(LLMK_ERR_ARG, "quant_w4_nk: W needs 16-byte and q 8-byte alignment");
+    const int64_t n_groups = N * (K / group);
+    const int64_t threads = n_groups * (group / EPL);
+    dim3 grid((unsigned)cdiv64(threads, 256)), blk(256);
+#define CALL(L) LLMK_DISPATCH_FLOAT(w_dtype, DT, (w4_quant_nk_kernel<DT, L><<<grid, blk, 0, (hipStream_t)stream>>>(w, packed, (unsigned short*)scales, q, n_groups)))
+    LPG_SWITCH(group, CALL)
+#undef CALL
+    LLMK_CHECK_LAUNCH("quant_w4_nk");
     return LLMK_OK;
 }
 

@@ -8,21 +8,26 @@ import torch
 
 try:
     from .. import _lib
-    from ..quantization.bitpack import pack_weights_over_cols
 except ImportError:  # this directory itself is on sys.path (the reference's top-level module layout)
     import _lib
-    from quantization.bitpack import pack_weights_over_cols
 
 
 def quantize_nk(w: torch.Tensor, group_size: int = 128):
-    """W [N, K] float -> (packed int32 [N, K/8], scales fp16 [N, K/group_size], q uint8 [N, K])."""
+    """W [N, K] float -> (packed int32 [N, K/8], scales fp16 [N, K/group_size], q uint8 [N, K]).
+
+    One pass over W on the GPU: s = absmax / 7 rounded to fp16, q = clamp(rne(w / s), -8, 7) + 8 with the
+    quotient by the rounded scale in fp32, nibble i of a packed word is k = 8 * word + i (the layout of
+    quantization.bitpack.pack_weights_over_cols(q, 4, 32, transpose=False))."""
     assert w.dim() == 2 and w.shape[1] % group_size == 0
+    assert w.dtype in (torch.float32, torch.float16, torch.bfloat16), 'weights must be fp32, fp16 or bf16'
+    _lib.require_gpu(w)
+    w = w.contiguous()
     N, K = w.shape
-    g = w.float().reshape(N, K // group_size, group_size)
-    amax = g.abs().amax(dim=2)
-    s = (amax / torch.full_like(amax, 7.0)).to(torch.float16)     # tensor divisor: a true IEEE division on every device
-    q = (torch.clamp(torch.round(g / s.float().unsqueeze(-1)), -8, 7) + 8).reshape(N, K).to(torch.uint8)
-    packed, _ = pack_weights_over_cols(q, 4, 32, transpose=False)
+    packed = torch.empty(N, K // 8, dtype=torch.int32, device=w.device)
+    s = torch.empty(N, K // group_size, dtype=torch.float16, device=w.device)
+    q = torch.empty(N, K, dtype=torch.uint8, device=w.device)
+    _lib.call("llmk_quant_w4_nk", _lib.ptr(w), _lib.dt(w.dtype), _lib.ptr(packed), _lib.ptr(s), _lib.ptr(q),
+              N, K, group_size, _lib.stream(w), exc=AssertionError)
     return packed, s, q
 
 

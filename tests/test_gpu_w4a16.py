@@ -108,19 +108,35 @@ def test_w4a16_nk(dev, M, N, K, gs):
     assert_close_scaled(y, ref, what="w4a16 nk")
 
 
-def test_w4a16_nk_device_quantize_round_trip(dev):
-    announce("w4a16 nk quantize on device")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,K,gs", [(4096, 4096, 128), (257, 1024, 64), (96, 512, 32), (33, 1024, 512), (5, 64, 8)])
+def test_w4a16_nk_device_quantize_round_trip(dev, dtype, N, K, gs):
+    """One-pass quantiser of the [N, K/8] layout: codes, scales and packed words bit-exact against the oracle's
+    absmax/7 rule and the bit-packing oracle (every division is an IEEE fp32 division on both sides)."""
+    announce("w4a16 nk quantize on device", dtype, N, K, gs)
     torch.manual_seed(3)
     from llm_kernels_amd.quantization.bitpack import unpack_over_cols
-    w = torch.randn(4096, 4096, device=dev) * 0.02
-    packed, s, qd = w4a16.quantize_nk(w, 128)
-    oq, os_ = q.w4a16_quant_nk(w.cpu(), 128)
-    assert packed.shape == (4096, 512)
+    w = (torch.randn(N, K) * 0.02).to(dtype)
+    w[N // 2, :gs] = 0                                              # a group of zeros: scale 0, codes 8
+    packed, s, qd = w4a16.quantize_nk(w.to(dev), gs)
+    oq, os_ = q.w4a16_quant_nk(w, gs)
+    oq[N // 2, :gs] = 8
+    assert packed.shape == (N, K // 8) and packed.dtype == torch.int32
     assert torch.equal(s.cpu(), os_)
-    # torch's device-side division may differ from the host's in the last place: allow isolated off-by-one codes
-    diff = (qd.cpu().int() - oq.int()).abs()
-    assert diff.max() <= 1 and (diff != 0).sum() <= 64
-    assert torch.equal(unpack_over_cols(packed, 4, 4096), qd)       # pack/unpack round trip, bit exact
+    assert torch.equal(qd.cpu(), oq)
+    opacked, _ = bp.pack_cols(oq.numpy(), 4, 32)
+    assert torch.equal(packed.cpu(), torch.from_numpy(opacked))
+    assert torch.equal(unpack_over_cols(packed, 4, K), qd)          # pack/unpack round trip, bit exact
+
+
+def test_w4a16_nk_device_quantize_refuses_bad_shapes(dev):
+    w = torch.randn(16, 256, device=dev)
+    with pytest.raises(AssertionError):
+        w4a16.quantize_nk(w, 96)                                    # not a divisor of K
+    with pytest.raises(AssertionError):
+        w4a16.quantize_nk(w[:, :48].contiguous(), 48)               # not a power of two
+    with pytest.raises(AssertionError):
+        w4a16.quantize_nk(w.double(), 128)
 
 
 @pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 1024, 4096), (64, 512, 8192), (16, 256, 14336)])
