@@ -174,6 +174,40 @@ __global__ void act_and_mul_kernel(const void* __restrict__ gateup, void* __rest
     }
 }
 
+// the same with 8 outputs per thread and pass (I a multiple of 8, 16-byte aligned tensors); a thread requests
+// the operands of two passes before it converts the first
+template <int IDT, int ODT>
+__global__ void act_and_mul_vec_kernel(const void* __restrict__ gateup, void* __restrict__ out,
+                                       const void* __restrict__ reorder_topk_ids, int ids_bytes,
+                                       const float* __restrict__ scales, int start_e, int end_e, int64_t two_i, int act) {
+    const int64_t row = blockIdx.x;
+    const int64_t e = ld_id(reorder_topk_ids, row, ids_bytes);
+    if (e < start_e || e > end_e) return;
+    const int64_t I = two_i / 2;
+    const bool has_scale = scales != nullptr;
+    const float scale = has_scale ? rnd<IDT>(1.0f / scales[e - start_e]) : 1.0f;
+    const int64_t step = (int64_t)blockDim.x * EPL;
+    for (int64_t c0 = (int64_t)threadIdx.x * EPL; c0 < I; c0 += 2 * step) {
+        const int64_t c1 = c0 + step;
+        const bool two = c1 < I;
+        float gv[2][EPL], up[2][EPL], r[EPL];
+        load8<IDT>(gateup, row * two_i + c0, gv[0]);
+        load8<IDT>(gateup, row * two_i + I + c0, up[0]);
+        if (two) {
+            load8<IDT>(gateup, row * two_i + c1, gv[1]);
+            load8<IDT>(gateup, row * two_i + I + c1, up[1]);
+        }
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) r[j] = gated_act<IDT>(gv[0][j], up[0][j], act, has_scale, scale);
+        store8<ODT>(out, row * I + c0, r);
+        if (two) {
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) r[j] = gated_act<IDT>(gv[1][j], up[1][j], act, has_scale, scale);
+            store8<ODT>(out, row * I + c1, r);
+        }
+    }
+}
+
 // Gated activation and 1 x 128 activation quantisation in one pass: 16 lanes own one group of 128 outputs,
 // 8 each.  The values quantised are exactly those the separate activation kernel would have stored in the
 // tensor dtype, so q and s equal those of the two-kernel sequence bit for bit.
@@ -402,6 +436,13 @@ extern "C" int llmk_moe_act_and_mul(const void* gateup, int in_dtype, void* out,
     if (act != 0 && act != 1) LLMK_FAIL(LLMK_ERR_DTYPE, "moe_act_and_mul: act %d", act);
     if (M == 0 || two_i == 0) return LLMK_OK;
     if (!gateup || !out || !reorder_topk_ids) LLMK_FAIL(LLMK_ERR_ARG, "moe_act_and_mul: null pointer");
+    const int in_al = in_dtype == LLMK_F32 ? 31 : 15, out_al = out_dtype == LLMK_F32 ? 31 : 15;
+    if ((two_i / 2) % 8 == 0 && ((uintptr_t)gateup & in_al) == 0 && ((uintptr_t)out & out_al) == 0) {
+        LLMK_DISPATCH_FLOAT(in_dtype, IDT, LLMK_DISPATCH_FLOAT(out_dtype, ODT,
+            (act_and_mul_vec_kernel<IDT, ODT><<<(unsigned)M, 256, 0, (hipStream_t)stream>>>(gateup, out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, two_i, act))));
+        LLMK_CHECK_LAUNCH("moe_act_and_mul");
+        return LLMK_OK;
+    }
     LLMK_DISPATCH_FLOAT(in_dtype, IDT, LLMK_DISPATCH_FLOAT(out_dtype, ODT,
         (act_and_mul_kernel<IDT, ODT><<<(unsigned)M, 256, 0, (hipStream_t)stream>>>(gateup, out, reorder_topk_ids, ids_bytes, scales, start_expert, end_expert, two_i, act))));
     LLMK_CHECK_LAUNCH("moe_act_and_mul");

@@ -312,6 +312,35 @@ __global__ void w4a8_dequant_kernel(const int32_t* __restrict__ packed, const un
     }
 }
 
+// the same with 8 consecutive k per thread: 8 packed words in, one 16-byte store per row out (K, the group
+// and 16-byte alignment of the words and of y are the caller's to check)
+__global__ void w4a8_dequant_vec_kernel(const int32_t* __restrict__ packed, const unsigned short* __restrict__ s,
+                                        const int8_t* __restrict__ s4, const int8_t* __restrict__ z4,
+                                        unsigned short* __restrict__ y, int64_t N, int64_t K, int block, int group) {
+    const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    const int64_t np = N / 8;
+    if (idx >= np * K) return;
+    const int64_t pr = idx / K, k = idx - pr * K;
+    const uint4 a = *(const uint4*)(packed + idx), b = *(const uint4*)(packed + idx + 4);
+    const unsigned w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const int64_t kg = (K + group - 1) / group, kb = (K + block - 1) / block;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int64_t n = pr * 8 + i;
+        const int8_t z = z4[n * kg + k / group], m = s4[n * kg + k / group];
+        const float sc = f16_to_f32(s[(n / block) * kb + k / block]);
+        unsigned o[4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int8_t q = (int8_t)((w[j] >> (4 * i)) & 0xf);
+            const int8_t d8 = (int8_t)((int8_t)(q - z) * m);          // int8 wrap-around, as the reference evaluates it
+            const unsigned h = f32_to_f16((float)d8 * sc);
+            o[j >> 1] = (j & 1) ? (o[j >> 1] | (h << 16)) : h;
+        }
+        *(uint4*)(y + n * K + k) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
 // ---------------------------------------------------------------- symmetric int4 along K for W [N, K] (W4A16)
 // s = absmax / 7 rounded to fp16; q = clamp(rne(w / s), -8, 7) + 8 with the division by the rounded scale in
 // fp32.  A lane owns 8 consecutive k: its 8 nibbles are exactly one int32 of the [N, K/8] bit-packed layout
@@ -534,6 +563,13 @@ extern "C" int llmk_weight_dequant_w4a8(const int32_t* packed, const void* s, co
     if (N == 0 || K == 0) return LLMK_OK;
     if (!packed || !s || !s4 || !z4 || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_w4a8: null pointer");
     dim3 grid((unsigned)cdiv64((N / 8) * K, 256)), blk(256);
+    if (K % 8 == 0 && group % 8 == 0 && block % 8 == 0 && ((((uintptr_t)packed) | ((uintptr_t)y)) & 15) == 0) {
+        dim3 vgrid((unsigned)cdiv64((N / 8) * K / 8, 256));
+        w4a8_dequant_vec_kernel<<<vgrid, blk, 0, (hipStream_t)stream>>>(packed, (const unsigned short*)s, s4, z4,
+                                                                       (unsigned short*)y, N, K, block, group);
+        LLMK_CHECK_LAUNCH("weight_dequant_w4a8");
+        return LLMK_OK;
+    }
     w4a8_dequant_kernel<<<grid, blk, 0, (hipStream_t)stream>>>(packed, (const unsigned short*)s, s4, z4,
                                                                (unsigned short*)y, N, K, block, group);
     LLMK_CHECK_LAUNCH("weight_dequant_w4a8");

@@ -25,6 +25,23 @@ __device__ __forceinline__ void load8(const void* p, int64_t i, float (&v)[EPL])
     }
 }
 
+// 8 consecutive elements in the storage type DT (16-byte aligned for the 16-bit types, 32-byte for fp32)
+template <int DT>
+__device__ __forceinline__ void store8(void* p, int64_t i, const float (&v)[EPL]) {
+    if constexpr (DT == LLMK_F32) {
+        float4* q = (float4*)((float*)p + i);
+        q[0] = make_float4(v[0], v[1], v[2], v[3]);
+        q[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        unsigned w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            w[j] = DT == LLMK_F16 ? ((unsigned)f32_to_f16(v[2 * j]) | ((unsigned)f32_to_f16(v[2 * j + 1]) << 16))
+                                  : ((unsigned)f32_to_bf16(v[2 * j]) | ((unsigned)f32_to_bf16(v[2 * j + 1]) << 16));
+        *(uint4*)((unsigned short*)p + i) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
 __device__ __forceinline__ float round_mode(float v, int mode) {
     // half-away: roundf is exact; half-up: floor(v + 0.5f) with the fp32 add as the reference states it
     return mode == LLMK_ROUND_HALF_AWAY ? roundf(v) : floorf(v + 0.5f);

@@ -151,6 +151,27 @@ def _segments(T, E, topk, seed, empty_last=True):
     return ids, w, m.run_moe_ep_preprocess(ids, E)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("I", [100, 2056, 4096 + 8])
+def test_activation_kernel_row_lengths(dev, dtype, I):
+    """Row lengths on both forms of the activation kernel (8 outputs per thread when I % 8 == 0, single elements
+    otherwise; 2056 = 257 passes of 8 ends on an odd pass), per-expert scales, a local expert range."""
+    announce("moe activation rows", dtype, I)
+    torch.manual_seed(5)
+    E, rows = 6, 37
+    rids = torch.sort(torch.randint(0, E, (rows,), dtype=torch.int64))[0]
+    gu = torch.randn(rows, 2 * I).to(dtype)
+    sc = torch.rand(4) + 0.5
+    for act, fn in (("silu", gk.silu_and_mul), ("gelu", gk.gelu_and_mul)):
+        di = torch.full((rows, I), -3.0, dtype=dtype, device=dev)
+        fn(gu.to(dev), di, 2 * I, rids.to(dev), sc.to(dev), 1, 4)
+        odi, mask = m.silu_and_mul(gu, rids, sc, 1, 4, act=act)
+        assert 0 < mask.sum() < rows
+        assert_close_scaled(di.cpu()[mask], odi[mask], rtol=2 ** -6 if dtype == torch.bfloat16 else 4e-3, atol=1e-5,
+                            what=act)
+        assert torch.all(di.cpu()[~mask] == -3.0)                 # rows of other ranks' experts stay untouched
+
+
 @pytest.mark.parametrize("kind", ["int8", "fp8", "fp16", "bf16"])
 @pytest.mark.parametrize("T,E,N,K", [(40, 4, 256, 256), (300, 8, 200, 512), (9, 8, 128, 128)])
 def test_grouped_gemm(dev, kind, T, E, N, K):

@@ -1,9 +1,12 @@
 """HIP quantizers / dequantizers vs the torch-CPU oracle: bit-exact integers and scales."""
+import ctypes
+
 import pytest
 import torch
 
 from oracle import quant_ref as q, bitpack_ref as bp
 from llm_kernels_amd.quantization import fp8_kernel, int8_kernel, w4a8_kernel
+from llm_kernels_amd import _lib
 from helpers import announce, default_dtype
 
 pytestmark = pytest.mark.gpu
@@ -95,6 +98,12 @@ def test_w4a8_weight_quant_dequant(dev, shape):
     assert d.dtype == torch.float16 and torch.equal(d.cpu(), q.w4a8_weight_dequant(oq, os_, os4, oz4))
     cos = torch.nn.functional.cosine_similarity(d.float().flatten().cpu(), w.float().flatten(), dim=0)
     assert cos > 0.98
+    # an output that is not 16-byte aligned takes the one-word-per-thread form of the kernel: same bits
+    buf = torch.empty(shape[0] * shape[1] + 1, dtype=torch.float16, device=dev)
+    _lib.call("llmk_weight_dequant_w4a8", _lib.ptr(yp), _lib.ptr(s), _lib.ptr(s4), _lib.ptr(z4),
+              ctypes.c_void_p(buf.data_ptr() + 2), shape[0], shape[1], 128, 128, None)
+    torch.cuda.synchronize()
+    assert torch.equal(buf[1:].view(shape), d)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
