@@ -73,6 +73,115 @@ class CopyCase:
         return time.perf_counter() - t0, 0
 
 
+def _stream_ops():
+    """name -> (inputs(dev), device launch(*inputs), oracle pass(*host inputs)) of the streaming operators beside
+    the GEMMs: quantisers, dequantisers, the bit packers and the gated activation, at the sizes of the benchmark
+    configurations (14336 x 4096 weights, 8192 tokens).  The oracle pass takes the first rows of the host copies."""
+    import numpy as np
+    from llm_kernels_amd.quantization import fp8_kernel, int8_kernel, w4a8_kernel, bitpack
+    from llm_kernels_amd.fast_dequant import w4a16
+    from llm_kernels_amd.moe import group_gemm_kernel as gk
+    from oracle import quant_ref as q, bitpack_ref as bp, moe_ref
+    N, K, T, I = 14336, 4096, 8192, 14336
+    act = lambda dev: (torch.randn(T, K, device=dev).bfloat16(),)
+    wgt = lambda dev: (torch.randn(N, K, device=dev) * 0.02,)
+    nib = lambda dev: (torch.randint(0, 16, (N, K), dtype=torch.uint8, device=dev),)
+
+    def quantised(kernel):
+        def make(dev):
+            y, s = kernel.weight_quant(torch.randn(N, K, device=dev) * 0.02)
+            return y, s
+        return make
+
+    def w4a8_packed(dev):
+        return w4a8_kernel.weight_quant((torch.randn(N, K, device=dev) * 0.02).half())
+
+    def gate_up(dev):
+        ids = torch.sort(torch.randint(0, 8, (T,), dtype=torch.int64, device=dev))[0]
+        return torch.randn(T, 2 * I, device=dev).bfloat16(), ids
+
+    def silu(gu, ids):
+        out = torch.empty(gu.size(0), gu.size(1) // 2, dtype=gu.dtype, device=gu.device)
+        return gk.silu_and_mul(gu, out, gu.size(1), ids, None, 0, 7)
+
+    R = 1024                                           # oracle sample: the first R rows
+    return {
+        "stream_act_quant_fp8": (act, fp8_kernel.act_quant, lambda x: q.act_quant_fp8(x[:R])),
+        "stream_act_quant_int8": (act, int8_kernel.act_quant, lambda x: q.act_quant_int8(x[:R])),
+        "stream_act_quant_int8_per_token": (act, int8_kernel.act_quant_per_token, lambda x: q.int8_quant_rowwise(x[:R])),
+        "stream_weight_quant_fp8": (wgt, fp8_kernel.weight_quant, lambda w: q.weight_quant_fp8(w[:R])),
+        "stream_weight_quant_int8": (wgt, int8_kernel.weight_quant, lambda w: q.weight_quant_int8(w[:R])),
+        "stream_weight_dequant_fp8": (quantised(fp8_kernel), fp8_kernel.weight_dequant,
+                                      lambda y, s: q.weight_dequant_block(y[:R], s[:R // 128])),
+        "stream_weight_dequant_int8": (quantised(int8_kernel), int8_kernel.weight_dequant,
+                                       lambda y, s: q.weight_dequant_block(y[:R], s[:R // 128])),
+        "stream_weight_dequant_w4a8": (w4a8_packed, w4a8_kernel.weight_dequant,
+                                       lambda y, s, s4, z4: q.w4a8_weight_dequant(
+                                           torch.from_numpy(bp.unpack_rows(y[:R // 8].numpy(), 4, R)), s[:R // 128], s4[:R], z4[:R])),
+        "stream_quantize_w4a16_nk": (lambda dev: (wgt(dev)[0].half(),), lambda w: w4a16.quantize_nk(w, 128),
+                                     lambda w: (q.w4a16_quant_nk(w[:R], 128), bp.pack_cols(q.w4a16_quant_nk(w[:R], 128)[0].numpy(), 4, 32))),
+        "stream_pack_rows_4in32": (nib, lambda w: bitpack.pack_weights_over_rows(w, 4, 32, False)[0],
+                                   lambda w: bp.pack_rows(w[:R].numpy(), 4, 32)),
+        "stream_pack_cols_4in32": (nib, lambda w: bitpack.pack_weights_over_cols(w, 4, 32, False)[0],
+                                   lambda w: bp.pack_cols(w[:R].numpy(), 4, 32)),
+        "stream_unpack_rows_4in32": (lambda dev: (bitpack.pack_weights_over_rows(nib(dev)[0], 4, 32, False)[0],),
+                                     lambda p: bitpack.unpack_over_rows(p, 4, N), lambda p: bp.unpack_rows(p[:R // 8].numpy(), 4, R)),
+        "stream_unpack_cols_4in32": (lambda dev: (bitpack.pack_weights_over_cols(nib(dev)[0], 4, 32, False)[0],),
+                                     lambda p: bitpack.unpack_over_cols(p, 4, K), lambda p: bp.unpack_cols(p[:R].numpy(), 4, K)),
+        "stream_silu_and_mul": (gate_up, silu, lambda gu, ids: moe_ref.silu_and_mul(gu[:R], ids[:R], None, 0, 7)),
+    }
+
+
+STREAM_WORKLOADS = ("stream_act_quant_fp8", "stream_act_quant_int8", "stream_act_quant_int8_per_token",
+                    "stream_weight_quant_fp8", "stream_weight_quant_int8", "stream_weight_dequant_fp8",
+                    "stream_weight_dequant_int8", "stream_weight_dequant_w4a8", "stream_quantize_w4a16_nk",
+                    "stream_pack_rows_4in32", "stream_pack_cols_4in32", "stream_unpack_rows_4in32",
+                    "stream_unpack_cols_4in32", "stream_silu_and_mul")
+
+
+def _tensors(v):
+    if isinstance(v, torch.Tensor):
+        return [v]
+    return [t for x in v for t in _tensors(x)] if isinstance(v, (tuple, list)) else []
+
+
+class StreamCase:
+    """One streaming operator (a quantiser, dequantiser, bit packer or the gated activation): every byte is read
+    or written once, so the algorithmic bytes are the sizes of the operator's inputs and outputs."""
+
+    def __init__(self, name):
+        self.name, self.op, self.M, self.N, self.K, self.flops = name, "stream", 0, 0, 0, 0.0
+        self.bound, self.mfma_dtype, self.dtype, self.nbuf, self.bytes = "hbm", "fp8", "u8", 1, 0
+
+    def setup(self, dev):
+        make, self.fn, self.oracle = _stream_ops()[self.name]
+        torch.manual_seed(0)
+        prev = torch.get_default_dtype()
+        torch.set_default_dtype(torch.float32)        # the dequantisers return the default dtype: fp32, as the reference's tests run them
+        self.inputs = make(dev)
+        outs = self.fn(*self.inputs)
+        torch.set_default_dtype(prev)
+        self.bytes = sum(t.numel() * t.element_size() for t in _tensors(self.inputs) + _tensors(outs))
+        del outs
+
+        def launch(i):
+            torch.set_default_dtype(torch.float32)
+            self.fn(*self.inputs)
+            torch.set_default_dtype(prev)
+        self.launch = launch
+
+    def cpu_seconds(self, max_rows):
+        host = [t.cpu() for t in self.inputs]
+        torch.set_default_dtype(torch.float32)
+        dt, self.cpu_passes = _timed_passes(lambda: self.oracle(*host), min(CPU_BUDGET_S, 3.0))
+        torch.set_default_dtype(torch.bfloat16)
+        # the sample is the first 1024 of the operator's rows: scale its bytes by the rows' share
+        rows = {"stream_silu_and_mul": 8192, "stream_act_quant_fp8": 8192, "stream_act_quant_int8": 8192,
+                "stream_act_quant_int8_per_token": 8192}.get(self.name, 14336)
+        self.cpu_bytes = self.bytes * 1024.0 / rows
+        return dt, 1024
+
+
 class MoECase:
     """Mixtral-8x7B shaped expert set on one GPU: permute -> grouped GEMM -> SwiGLU -> grouped GEMM -> un-permute.
 
@@ -450,6 +559,11 @@ def cpu_baseline(case, budget):
     if case.op == "copy":
         return {"value": round(case.bytes / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": "host memcpy of the same size"}
+    if case.op == "stream":
+        return {"value": round(case.cpu_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                "cpu_model": _cpu_model(),
+                "sample": "the oracle's restatement of the operator on the first %d rows of the same inputs, 1 warm-up + "
+                          "%d timed passes of %.4f s each" % (rows, case.cpu_passes, dt)}
     cpu_flops = case.flops * rows / case.T if case.op == "moe" else 2.0 * rows * case.N * case.K
     out = {"value": round(cpu_flops / dt / 1e12, 4), "unit": "TFLOP/s",
            "cores": torch.get_num_threads(), "kind": "port", "cpu_model": _cpu_model(),
@@ -566,6 +680,9 @@ def main():
     if args.workload == "copy_256m":
         op, M, N, K = "copy", 0, 0, 0
         case = CopyCase(args.workload, 256 << 20)
+    elif args.workload in STREAM_WORKLOADS:
+        op, M, N, K = "stream", 0, 0, 0
+        case = StreamCase(args.workload)
     elif args.workload in MOE_WORKLOADS or re.fullmatch(r"moe_mixtral_(fp8|int8)_t(\d+)", args.workload):
         if args.workload not in MOE_WORKLOADS:          # any other token count of the registered expert layer
             mm = re.fullmatch(r"moe_mixtral_(fp8|int8)_t(\d+)", args.workload)
@@ -590,6 +707,18 @@ def main():
             if name == args.workload:
                 continue
             c = MoECase(name, *MOE_WORKLOADS[name]) if name in MOE_WORKLOADS else Case(name, *WORKLOADS[name])
+            r2 = record(c, run_case(c, dev, args.steps, args.warmup, args.eager), args.steps)
+            if not args.no_cpu:
+                r2["cpu_baseline"] = cpu_baseline(c, CPU_BUDGET_OTHER_S)
+            cases.append(r2)
+            del c
+            torch.cuda.empty_cache()
+
+    if not args.headline_only and args.workload in STREAM_WORKLOADS:      # the other streaming operators, same method
+        for name in STREAM_WORKLOADS:
+            if name == args.workload:
+                continue
+            c = StreamCase(name)
             r2 = record(c, run_case(c, dev, args.steps, args.warmup, args.eager), args.steps)
             if not args.no_cpu:
                 r2["cpu_baseline"] = cpu_baseline(c, CPU_BUDGET_OTHER_S)

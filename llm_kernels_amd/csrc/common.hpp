@@ -72,6 +72,14 @@ __device__ __forceinline__ float f16_to_f32(unsigned short h) {
     __builtin_memcpy(&v, &h, 2);
     return (float)v;
 }
+// Keeps an fp32 value as computed.  Without it the compiler folds an fp32 multiply and the conversion of its
+// result to fp16 into one v_fma_mixlo_f16, which rounds the exact product once; an operator defined as
+// "multiply in fp32, then cast" rounds twice, and the two differ by an fp16 ulp where the fp32 product lands
+// on a tie.  Needed only where the product is not exact in fp32 (fp32 scales).
+__device__ __forceinline__ float keep_f32(float v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
 __device__ __forceinline__ unsigned short f32_to_f16(float f) {
     _Float16 v = (_Float16)f;   // v_cvt_f16_f32, RNE
     unsigned short h;

@@ -248,47 +248,68 @@ __global__ void weight_dequant_block_kernel(const uint8_t* __restrict__ x, const
     } else {
         xv = (float)(int8_t)x[idx];
     }
-    FloatIO<ODT>::st(y, idx, xv * sc);
+    FloatIO<ODT>::st(y, idx, ODT == LLMK_F16 ? keep_f32(xv * sc) : xv * sc);
 }
 
-// the same with 16 elements of a row per thread (N and the block size multiples of 16: one scale per thread)
+// One workgroup per 4096 columns of a row, every store instruction of a wave one contiguous KB: a lane takes
+// the 4 (fp32 output) or 8 (16-bit output) elements at 256 E q + E tid of the span, q = 0 .. 16 / E - 1.  With
+// 16 consecutive elements per lane the four 16-byte stores of a lane leave partly written lines between the
+// instructions (fp32 output: 77 us for 14336 x 4096 against 49.5 us; 6.6 TB/s is what the byte -> fp16
+// converter reaches with contiguous 16-byte stores).  N and the block size multiples of 16.
 template <int ODT, int SDT, bool FP8>
-__global__ void weight_dequant_block_vec_kernel(const uint8_t* __restrict__ x, const void* __restrict__ s,
-                                                void* __restrict__ y, int64_t M, int64_t N, int block) {
-    const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 16;
-    if (idx >= M * N) return;
-    const int64_t r = idx / N, c = idx - r * N;
-    const int64_t nb = (N + block - 1) / block;
-    const float sc = FloatIO<SDT>::ld(s, (r / block) * nb + c / block);
-    const uint4 w = *(const uint4*)(x + idx);
-    const unsigned ws[4] = {w.x, w.y, w.z, w.w};
-    float v[16];
+__global__ void weight_dequant_block_row_kernel(const uint8_t* __restrict__ x, const void* __restrict__ s,
+                                                void* __restrict__ y, int64_t N, int block) {
+    constexpr int E = ODT == LLMK_F32 ? 4 : 8, CH = 16 / E;
+    const int64_t r = blockIdx.x;
+    const int nb = (int)((N + block - 1) / block);
+    const int64_t srow = (r / block) * nb;
+    const int c0 = blockIdx.y * 4096 + threadIdx.x * E;
+    unsigned w[CH][E / 4];
+    float sc[CH];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        if constexpr (FP8) {
-            v[4 * q + 0] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 0) * sc;
-            v[4 * q + 1] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 1) * sc;
-            v[4 * q + 2] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 2) * sc;
-            v[4 * q + 3] = __builtin_amdgcn_cvt_f32_fp8((int)ws[q], 3) * sc;
+    for (int q = 0; q < CH; ++q) {
+        const int c = c0 + q * 256 * E;
+        const bool live = c < N;
+        const int cs = live ? c : 0;
+        if constexpr (E == 4) {
+            w[q][0] = *(const unsigned*)(x + r * N + cs);
         } else {
-#pragma unroll
-            for (int b = 0; b < 4; ++b) v[4 * q + b] = (float)(int8_t)(ws[q] >> (8 * b)) * sc;
+            const uint2 t = *(const uint2*)(x + r * N + cs);
+            w[q][0] = t.x; w[q][1] = t.y;
         }
+        sc[q] = FloatIO<SDT>::ld(s, srow + cs / block);
     }
-    if constexpr (ODT == LLMK_F32) {
-        float4* dst = (float4*)((float*)y + idx);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) dst[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
-    } else {
-        uint4 o[2];
-        unsigned* op = (unsigned*)o;
+    for (int q = 0; q < CH; ++q) {
+        const int c = c0 + q * 256 * E;
+        if (c >= N) continue;
+        float v[E];
 #pragma unroll
-        for (int q = 0; q < 8; ++q)
-            op[q] = ODT == LLMK_F16 ? ((unsigned)f32_to_f16(v[2 * q]) | ((unsigned)f32_to_f16(v[2 * q + 1]) << 16))
-                                    : ((unsigned)f32_to_bf16(v[2 * q]) | ((unsigned)f32_to_bf16(v[2 * q + 1]) << 16));
-        uint4* dst = (uint4*)((unsigned short*)y + idx);
-        dst[0] = o[0];
-        dst[1] = o[1];
+        for (int h = 0; h < E / 4; ++h) {
+            if constexpr (FP8) {
+                v[4 * h + 0] = __builtin_amdgcn_cvt_f32_fp8((int)w[q][h], 0) * sc[q];
+                v[4 * h + 1] = __builtin_amdgcn_cvt_f32_fp8((int)w[q][h], 1) * sc[q];
+                v[4 * h + 2] = __builtin_amdgcn_cvt_f32_fp8((int)w[q][h], 2) * sc[q];
+                v[4 * h + 3] = __builtin_amdgcn_cvt_f32_fp8((int)w[q][h], 3) * sc[q];
+            } else {
+#pragma unroll
+                for (int b = 0; b < 4; ++b) v[4 * h + b] = (float)(int8_t)(w[q][h] >> (8 * b)) * sc[q];
+            }
+        }
+        if constexpr (ODT == LLMK_F16) {            // the products are fp32 values of their own: round twice, as the reference does
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[e] = keep_f32(v[e]);
+        }
+        if constexpr (ODT == LLMK_F32) {
+            *(float4*)((float*)y + r * N + c) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+            unsigned o[4];
+#pragma unroll
+            for (int h = 0; h < 4; ++h)
+                o[h] = ODT == LLMK_F16 ? ((unsigned)f32_to_f16(v[2 * h]) | ((unsigned)f32_to_f16(v[2 * h + 1]) << 16))
+                                       : ((unsigned)f32_to_bf16(v[2 * h]) | ((unsigned)f32_to_bf16(v[2 * h + 1]) << 16));
+            *(uint4*)((unsigned short*)y + r * N + c) = make_uint4(o[0], o[1], o[2], o[3]);
+        }
     }
 }
 
@@ -529,9 +550,9 @@ extern "C" int llmk_weight_dequant_fp8_block(const void* x, const float* s, void
     if (M == 0 || N == 0) return LLMK_OK;
     if (!x || !s || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_fp8_block: null pointer");
     dim3 grid((unsigned)cdiv64(M * N, 256)), blk(256);
-    if (N % 16 == 0 && block % 16 == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0) {
-        dim3 vgrid((unsigned)cdiv64(M * N / 16, 256));
-        LLMK_DISPATCH_FLOAT(y_dtype, ODT, (weight_dequant_block_vec_kernel<ODT, LLMK_F32, true><<<vgrid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block)));
+    if (N % 16 == 0 && block % 16 == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0 && M < (1ll << 31) && N <= 4096ll * 65535) {
+        dim3 rgrid((unsigned)M, (unsigned)cdiv64(N, 4096));
+        LLMK_DISPATCH_FLOAT(y_dtype, ODT, (weight_dequant_block_row_kernel<ODT, LLMK_F32, true><<<rgrid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, N, block)));
         LLMK_CHECK_LAUNCH("weight_dequant_fp8_block");
         return LLMK_OK;
     }
@@ -546,9 +567,9 @@ extern "C" int llmk_weight_dequant_i8_block(const int8_t* x, const void* s, int 
     if (M == 0 || N == 0) return LLMK_OK;
     if (!x || !s || !y) LLMK_FAIL(LLMK_ERR_ARG, "weight_dequant_i8_block: null pointer");
     dim3 grid((unsigned)cdiv64(M * N, 256)), blk(256);
-    if (N % 16 == 0 && block % 16 == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0) {
-        dim3 vgrid((unsigned)cdiv64(M * N / 16, 256));
-        LLMK_DISPATCH_FLOAT(y_dtype, ODT, LLMK_DISPATCH_FLOAT(s_dtype, SDT, (weight_dequant_block_vec_kernel<ODT, SDT, false><<<vgrid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, M, N, block))));
+    if (N % 16 == 0 && block % 16 == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0 && M < (1ll << 31) && N <= 4096ll * 65535) {
+        dim3 rgrid((unsigned)M, (unsigned)cdiv64(N, 4096));
+        LLMK_DISPATCH_FLOAT(y_dtype, ODT, LLMK_DISPATCH_FLOAT(s_dtype, SDT, (weight_dequant_block_row_kernel<ODT, SDT, false><<<rgrid, blk, 0, (hipStream_t)stream>>>((const uint8_t*)x, s, y, N, block))));
         LLMK_CHECK_LAUNCH("weight_dequant_i8_block");
         return LLMK_OK;
     }

@@ -53,7 +53,7 @@ def test_act_quant_fp8_zero_group_nan_and_asserts(dev):
         int8_kernel.act_quant(torch.randn(4, 256, device=dev).t())
 
 
-@pytest.mark.parametrize("shape", [(128, 128), (512, 1024), (200, 300), (4096, 4096)])
+@pytest.mark.parametrize("shape", [(128, 128), (512, 1024), (200, 300), (4096, 4096), (136, 4144), (72, 14336)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_weight_quant_int8_and_dequant(dev, shape, dtype):
     announce("weight_quant_i8", shape, dtype)
@@ -69,7 +69,7 @@ def test_weight_quant_int8_and_dequant(dev, shape, dtype):
         assert torch.equal(d.cpu(), q.weight_dequant_block(oy, os_, 128, dd))
 
 
-@pytest.mark.parametrize("shape", [(128, 256), (300, 200), (4096, 4096)])
+@pytest.mark.parametrize("shape", [(128, 256), (300, 200), (4096, 4096), (130, 7168), (40, 4144)])
 def test_weight_quant_fp8_and_dequant(dev, shape):
     announce("weight_quant_fp8", shape)
     torch.manual_seed(3)
@@ -78,9 +78,10 @@ def test_weight_quant_fp8_and_dequant(dev, shape):
     oy, os_ = q.weight_quant_fp8(w)
     assert torch.equal(s.cpu(), os_)
     assert torch.equal(y.cpu().view(torch.uint8), oy.view(torch.uint8))
-    with default_dtype(torch.bfloat16):
-        d = fp8_kernel.weight_dequant(y, s)
-    assert torch.equal(d.cpu(), q.weight_dequant_block(oy, os_, 128, torch.bfloat16))
+    for dd in (torch.bfloat16, torch.float16, torch.float32):
+        with default_dtype(dd):
+            d = fp8_kernel.weight_dequant(y, s)
+        assert d.dtype == dd and torch.equal(d.cpu(), q.weight_dequant_block(oy, os_, 128, dd))
 
 
 @pytest.mark.parametrize("shape", [(128, 128), (1024, 7168), (4096, 4096)])
