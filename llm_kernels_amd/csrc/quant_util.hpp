@@ -70,16 +70,19 @@ __device__ __forceinline__ float group_min(float v) {
 }
 
 
-// a / b from r = RN(1 / b): one product and the residual correction q + (a - q b) r, both in fma.  The
+// a / b from r = RN(1 / b): one product and the residual correction q - (q b - a) r, both in fma.  The
 // residual is exact whenever q is within an ulp of the quotient, and the corrected value is then the rounded
 // quotient (the final step of the usual fma division); in 80 M random trials over the quantisers' operand
 // ranges it equalled the IEEE division every time.  Nothing may leave the normal range: callers check b
 // and take the division otherwise.  A quantiser divides the 8 values of a lane by one scale, so the
 // reciprocal is shared and a quotient costs three instructions instead of about ten.
+// The residual is formed as its negative, q b - a, and subtracted: with a = -0 the sum q b - a is +0 and
+// q - (+0) r keeps the -0 of the quotient, where q + (a - q b) r would return +0 (an e4m3 result keeps the sign
+// of a zero: 0x80).
 __device__ __forceinline__ float div_by(float a, float b, float r) {
     const float q = a * r;
-    const float rem = fmaf(-q, b, a);
-    return fmaf(rem, r, q);
+    const float nrem = fmaf(q, b, -a);
+    return fmaf(-nrem, r, q);
 }
 // scales whose reciprocal, products and residuals stay normal for every |a| <= 448 b that does not round to
 // zero in the 8-bit result anyway
@@ -125,8 +128,11 @@ __device__ __forceinline__ void quant_store8(const float (&v)[EPL], float m, voi
 }
 
 // round-trip through the storage type: the reference multiplies in the tensor dtype
+// (fp16: the value is pinned first.  A product that is only converted to fp16 otherwise becomes
+// v_fma_mixlo_f16(a, b, +0), and (-0) + (+0) = +0 loses the sign of a zero product, which the e4m3 quantiser
+// behind the activation would store as 0x00 instead of 0x80.)
 template <int DT> __device__ __forceinline__ float rnd(float v) {
-    if constexpr (DT == LLMK_F16) return f16_to_f32(f32_to_f16(v));
+    if constexpr (DT == LLMK_F16) return f16_to_f32(f32_to_f16(keep_f32(v)));
     else if constexpr (DT == LLMK_BF16) return bf16_to_f32(f32_to_bf16(v));
     else return v;
 }

@@ -136,3 +136,21 @@ def test_rowwise_int8_quantizer_zero_row_is_nan_free_of_crash(dev):
     oy, os_ = q.int8_quant_rowwise(x)
     assert s.cpu()[0].item() == 0.0 and torch.equal(s.cpu(), os_)
     assert torch.equal(y.cpu()[1], oy[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_fp8_quantisers_keep_the_sign_of_zero(dev, dtype):
+    """-0.0 / s is -0.0, which e4m3 stores as 0x80: the quotient by the shared reciprocal must not turn it into
+    +0 (fp16 weights of small magnitude underflow to -0.0 often enough to meet this in 4096 x 4096 elements)."""
+    announce("fp8 quantisers, signed zeros", dtype)
+    torch.manual_seed(11)
+    x = (torch.randn(256, 512) * 0.02).to(dtype)
+    x[::3, ::5] = -0.0
+    x[1::3, 1::5] = 0.0
+    y, s = fp8_kernel.act_quant(x.to(dev))
+    oy, os_ = q.act_quant_fp8(x)
+    assert torch.equal(s.cpu(), os_) and torch.equal(y.cpu().view(torch.uint8), oy.view(torch.uint8))
+    assert (oy.view(torch.uint8)[::3, ::5] == 0x80).all()
+    y, s = fp8_kernel.weight_quant(x.to(dev))
+    oy, os_ = q.weight_quant_fp8(x)
+    assert torch.equal(s.cpu(), os_) and torch.equal(y.cpu().view(torch.uint8), oy.view(torch.uint8))
