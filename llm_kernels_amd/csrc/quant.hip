@@ -53,13 +53,14 @@ __global__ void block_dequant_kernel(const uint8_t* __restrict__ y, const void* 
         } else {
             q = (float)(int)(int8_t)b;
         }
-        float pr = q * sc;
-        if constexpr (SDT == LLMK_F16) pr = f16_to_f32(f32_to_f16(pr));
-        else if constexpr (SDT == LLMK_BF16) pr = bf16_to_f32(f32_to_bf16(pr));
-        v[j] = pr;
+        v[j] = rnd<SDT>(q * sc);
     }
+    if ((((uintptr_t)x) & (ODT == LLMK_F32 ? 31 : 15)) == 0) {
+        store8<ODT>(x, off, v);
+    } else {
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) FloatIO<ODT>::st(x, off + j, v[j]);
+        for (int j = 0; j < EPL; ++j) FloatIO<ODT>::st(x, off + j, v[j]);
+    }
 }
 
 // ---------------------------------------------------------------- one group per row (per-token / per-channel int8)

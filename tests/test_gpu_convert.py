@@ -82,3 +82,21 @@ def test_fp8_payload_round_trip_bit_exact(dev, dtype):
     # reference recipe (quant_utils.py:228-251): cosine similarity of the round trip
     back = qc.fp8_dequant(y, s, dtype).float().cpu().flatten()
     assert torch.nn.functional.cosine_similarity(back, x.float().flatten(), dim=0) > 0.999
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_payload_dequantisers_keep_the_sign_of_zero(dev, dtype):
+    """-0.0 survives quantisation as the e4m3 code 0x80 and comes back as -0.0 in every output dtype (compared as
+    bit patterns: the float comparison calls the two zeros equal)."""
+    announce("comm signed zeros", dtype)
+    torch.manual_seed(4)
+    x = (torch.randn(9, 384) * 2).to(dtype)
+    x[::2, ::7] = -0.0
+    y, s = qc.fp8_quant(x.to(dev), 128)
+    oy, os_ = c.fp8_quant(x, 128)
+    assert torch.equal(y.view(torch.uint8).cpu(), oy.view(torch.uint8)) and torch.equal(s.cpu(), os_)
+    assert (oy.view(torch.uint8)[::2, ::7] == 0x80).all()
+    for odt in (torch.float16, torch.bfloat16):
+        d, ref = qc.fp8_dequant(y, s, odt).cpu(), c.dequant(oy, os_, odt)
+        assert torch.equal(d.view(torch.int16), ref.view(torch.int16))
+        assert (d.view(torch.int16)[::2, ::7] == -32768).all()
