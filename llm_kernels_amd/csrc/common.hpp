@@ -75,7 +75,7 @@ __device__ __forceinline__ float f16_to_f32(unsigned short h) {
 // Keeps an fp32 value as computed.  Without it the compiler folds an fp32 multiply and the conversion of its
 // result to fp16 into one v_fma_mixlo_f16, which rounds the exact product once; an operator defined as
 // "multiply in fp32, then cast" rounds twice, and the two differ by an fp16 ulp where the fp32 product lands
-// on a tie.  Needed only where the product is not exact in fp32 (fp32 scales).
+// on a tie.  The fused form also adds +0, so a product of -0 comes out as +0.
 __device__ __forceinline__ float keep_f32(float v) {
     asm volatile("" : "+v"(v));
     return v;
@@ -97,7 +97,8 @@ template <> struct FloatIO<LLMK_F32> {
 template <> struct FloatIO<LLMK_F16> {
     typedef unsigned short T;
     static __device__ __forceinline__ float ld(const void* p, int64_t i) { return f16_to_f32(((const unsigned short*)p)[i]); }
-    static __device__ __forceinline__ void st(void* p, int64_t i, float v) { ((unsigned short*)p)[i] = f32_to_f16(v); }
+    // the value as the caller computed it in fp32, then one conversion (see keep_f32)
+    static __device__ __forceinline__ void st(void* p, int64_t i, float v) { ((unsigned short*)p)[i] = f32_to_f16(keep_f32(v)); }
 };
 template <> struct FloatIO<LLMK_BF16> {
     typedef unsigned short T;

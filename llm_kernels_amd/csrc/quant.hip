@@ -249,7 +249,7 @@ __global__ void weight_dequant_block_kernel(const uint8_t* __restrict__ x, const
     } else {
         xv = (float)(int8_t)x[idx];
     }
-    FloatIO<ODT>::st(y, idx, ODT == LLMK_F16 ? keep_f32(xv * sc) : xv * sc);
+    FloatIO<ODT>::st(y, idx, xv * sc);
 }
 
 // One workgroup per 4096 columns of a row, every store instruction of a wave one contiguous KB: a lane takes

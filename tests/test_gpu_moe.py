@@ -112,6 +112,14 @@ def test_reorder_and_activation_kernels(dev, dtype):
     gk.pre_reorder_triton_kernel[(T,)](x.to(dev), gin, s2d.to(dev), ids.to(dev), None, 2, 5, topk, H, BLOCK_SIZE=512)
     ogin = m.pre_reorder(x, s2d, ids, None, 2, 5, topk, out=torch.full((T * topk, H), -3.0, dtype=dtype))
     assert torch.equal(gin.cpu(), ogin)
+    # the copy keeps the sign of a zero (compared as bit patterns)
+    xz = x.clone()
+    xz[:, ::3] = -0.0
+    ginz = torch.zeros((T * topk, H), dtype=dtype, device=dev)
+    gk.pre_reorder(xz.to(dev), ginz, s2d.to(dev), ids.to(dev), None, 0, E - 1, topk, H)
+    oginz = m.pre_reorder(xz, s2d, ids, None, 0, E - 1, topk)
+    as_bits = lambda t: t.contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32)
+    assert torch.equal(as_bits(ginz.cpu()), as_bits(oginz))
     a1 = torch.rand(4) + 0.5
     gin2 = torch.zeros((T * topk, H), dtype=dtype, device=dev)
     gk.pre_reorder(x.to(dev), gin2, s2d.to(dev), ids.to(dev), a1.to(dev), 2, 5, topk, H)
