@@ -28,6 +28,9 @@ the reference CUDA kernel are used; see ``tests/test_oracle_*.py``):
 Parity unpinned (bit level only; irrelevant at the stated tolerances): the
 fp32->e4m3 rounding and the fp32 summation order inside Triton's ``tl.dot``
 (the reference has no test for ``fp8_gemm`` and only prints cosine similarity
-for ``int8_gemm`` / ``w4a8_gemm``).  The oracle assumes IEEE round-to-nearest-
-even casts and exact fp32 division, which is what torch-CPU does.
+for ``int8_gemm`` / ``w4a8_gemm``), and whether the reference's compiler
+rounds an fp32 product once or twice on its way into an fp16 tensor and which
+sign a zero product keeps.  The oracle assumes IEEE round-to-nearest-even
+casts, exact fp32 division, every product rounded to fp32 before a cast and
+signed zeros kept, which is what torch-CPU does.
 """
